@@ -1,0 +1,87 @@
+// Shared by every kernel file of the library: element types, conversions, wave reductions and
+// the error convention of the C entry points (0 = launched, anything else = refused; the text is
+// read with mllm_last_error()).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define MLLM_API extern "C" __attribute__((visibility("default")))
+
+// Element types as the Python side names them.
+enum MllmDtype : int { MLLM_F32 = 0, MLLM_BF16 = 1 };
+
+// What a matrix product does to its sums before it stores them.
+enum MllmEpilogue : int {
+    MLLM_EPI_NONE = 0,       // (+ bias)
+    MLLM_EPI_GELU_TANH = 1,  // gelu_new(+ bias)
+    MLLM_EPI_GELU_ERF = 2,   // gelu(+ bias)
+};
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int WAVE = 64;
+
+void mllm_set_error(const char* format, ...);
+int mllm_check_launch(const char* what);
+
+#define MLLM_REQUIRE(condition, ...)      \
+    do {                                  \
+        if (!(condition)) {               \
+            mllm_set_error(__VA_ARGS__);  \
+            return 1;                     \
+        }                                 \
+    } while (0)
+
+__device__ __forceinline__ float to_float(float x) { return x; }
+__device__ __forceinline__ float to_float(bf16_t x) { return static_cast<float>(x); }
+
+template <typename T>
+__device__ __forceinline__ T from_float(float x);
+template <>
+__device__ __forceinline__ float from_float<float>(float x) {
+    return x;
+}
+template <>
+__device__ __forceinline__ bf16_t from_float<bf16_t>(float x) {
+    return static_cast<bf16_t>(x);  // round to nearest even
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
+    return v;
+}
+
+// tanh form of GELU, in the reference's order of operations (engine/include/gelu_math.h:6-11).
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float coefficient = 0.7978845608f;
+    const float cubic = 0.044715f;
+    float argument = coefficient * (x + cubic * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(argument));
+}
+
+// exact GELU (engine/src/gelu.c:5-9).
+__device__ __forceinline__ float gelu_erf(float x) {
+    return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+template <int EPI>
+__device__ __forceinline__ float apply_activation(float x) {
+    if constexpr (EPI == MLLM_EPI_GELU_TANH) return gelu_tanh(x);
+    if constexpr (EPI == MLLM_EPI_GELU_ERF) return gelu_erf(x);
+    return x;
+}
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -1,0 +1,149 @@
+// Embedding gather with the learned position rows added, row LayerNorm, and the plain residual
+// add for parts that do not fuse it into a matrix product.
+#include "common.h"
+
+// out[t, :] = wte[token[t], :] + wpe[position[t], :]   (reference: engine/src/embedding.cu:7-27,
+// per-row positions as in embed_batch_kernel :89-104). One block per row; a negative token marks
+// a padding row, which is filled with zeros.
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                             const T* __restrict__ wte, const T* __restrict__ wpe,
+                             float* __restrict__ out, int width) {
+    int row = blockIdx.x;
+    int token = tokens[row];
+    float* out_row = out + (size_t)row * width;
+    if (token < 0) {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) out_row[i] = 0.0f;
+        return;
+    }
+    const T* token_row = wte + (size_t)token * width;
+    const T* position_row = wpe + (size_t)positions[row] * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+        out_row[i] = to_float(token_row[i]) + to_float(position_row[i]);
+}
+
+MLLM_API int mllm_embed(const int* tokens, const int* positions, const void* wte, const void* wpe,
+                        float* out, int n_rows, int width, int table_dtype, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && width > 0, "embed: bad sizes rows=%d width=%d", n_rows, width);
+    if (n_rows == 0) return 0;
+    int threads = width >= 256 ? 256 : 64;
+    if (table_dtype == MLLM_F32)
+        embed_kernel<float><<<n_rows, threads, 0, stream>>>(tokens, positions, (const float*)wte,
+                                                            (const float*)wpe, out, width);
+    else if (table_dtype == MLLM_BF16)
+        embed_kernel<bf16_t><<<n_rows, threads, 0, stream>>>(tokens, positions, (const bf16_t*)wte,
+                                                             (const bf16_t*)wpe, out, width);
+    else
+        MLLM_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
+    return mllm_check_launch("embed");
+}
+
+// Row LayerNorm in 32-bit with a centred second pass (reference: engine/src/layernorm.cu:44-72):
+// mean = sum/n, var = sum((x-mean)^2)/n, y = (x-mean) * 1/sqrt(var+eps) * gamma + beta.
+// One wave per row, the row kept in registers when it fits (ROW_REGS*64 >= width), re-read
+// otherwise. row_index, if given, names the input row of each output row.
+template <typename OutT, int ROW_REGS>
+__global__ void layernorm_kernel(const float* __restrict__ x, const int* __restrict__ row_index,
+                                 const float* __restrict__ gamma, const float* __restrict__ beta,
+                                 OutT* __restrict__ out, int n_rows, int width, float eps) {
+    int lane = threadIdx.x % WAVE;
+    int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (row >= n_rows) return;
+    int source = row_index ? row_index[row] : row;
+    const float* in_row = x + (size_t)source * width;
+    OutT* out_row = out + (size_t)row * width;
+    float inverse_width = 1.0f / (float)width;
+
+    if constexpr (ROW_REGS > 0) {
+        float values[ROW_REGS];
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < ROW_REGS; r++) {
+            int i = lane + r * WAVE;
+            values[r] = i < width ? in_row[i] : 0.0f;
+            sum += values[r];
+        }
+        float mean = wave_sum(sum) * inverse_width;
+        float squares = 0.0f;
+#pragma unroll
+        for (int r = 0; r < ROW_REGS; r++) {
+            int i = lane + r * WAVE;
+            float diff = i < width ? values[r] - mean : 0.0f;
+            squares += diff * diff;
+        }
+        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) * inverse_width + eps);
+#pragma unroll
+        for (int r = 0; r < ROW_REGS; r++) {
+            int i = lane + r * WAVE;
+            if (i < width)
+                out_row[i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gamma[i] + beta[i]);
+        }
+    } else {
+        float sum = 0.0f;
+        for (int i = lane; i < width; i += WAVE) sum += in_row[i];
+        float mean = wave_sum(sum) * inverse_width;
+        float squares = 0.0f;
+        for (int i = lane; i < width; i += WAVE) {
+            float diff = in_row[i] - mean;
+            squares += diff * diff;
+        }
+        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) * inverse_width + eps);
+        for (int i = lane; i < width; i += WAVE)
+            out_row[i] = from_float<OutT>((in_row[i] - mean) * inverse_stddev * gamma[i] + beta[i]);
+    }
+}
+
+template <typename OutT>
+static void launch_layernorm(const float* x, const int* row_index, const float* gamma,
+                             const float* beta, void* out, int n_rows, int width, float eps,
+                             hipStream_t stream) {
+    const int waves = 4;
+    dim3 grid(ceil_div(n_rows, waves)), block(waves * WAVE);
+    OutT* o = (OutT*)out;
+    if (width <= 4 * WAVE)
+        layernorm_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+    else if (width <= 16 * WAVE)
+        layernorm_kernel<OutT, 16><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+    else if (width <= 32 * WAVE)
+        layernorm_kernel<OutT, 32><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+    else
+        layernorm_kernel<OutT, 0><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+}
+
+MLLM_API int mllm_layernorm(const float* x, const int* row_index, const float* gamma,
+                            const float* beta, void* out, int n_rows, int width, float eps,
+                            int out_dtype, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && width > 0, "layernorm: bad sizes rows=%d width=%d", n_rows, width);
+    MLLM_REQUIRE(eps > 0.0f, "layernorm: eps must be positive");
+    if (n_rows == 0) return 0;
+    if (out_dtype == MLLM_F32)
+        launch_layernorm<float>(x, row_index, gamma, beta, out, n_rows, width, eps, stream);
+    else if (out_dtype == MLLM_BF16)
+        launch_layernorm<bf16_t>(x, row_index, gamma, beta, out, n_rows, width, eps, stream);
+    else
+        MLLM_REQUIRE(false, "layernorm: unknown output dtype %d", out_dtype);
+    return mllm_check_launch("layernorm");
+}
+
+// out = a + b in 32-bit, b of either element type (the residual sum of a part that does not
+// fuse it; reference: engine/src/vector_addition.cu:5-11).
+template <typename T>
+__global__ void add_kernel(const float* __restrict__ a, const T* __restrict__ b,
+                           float* __restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + to_float(b[i]);
+}
+
+MLLM_API int mllm_add(const float* a, const void* b, float* out, long long n, int b_dtype,
+                      hipStream_t stream) {
+    MLLM_REQUIRE(n >= 0, "add: negative size");
+    if (n == 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (b_dtype == MLLM_F32)
+        add_kernel<float><<<blocks, 256, 0, stream>>>(a, (const float*)b, out, (size_t)n);
+    else if (b_dtype == MLLM_BF16)
+        add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(a, (const bf16_t*)b, out, (size_t)n);
+    else
+        MLLM_REQUIRE(false, "add: unknown dtype %d", b_dtype);
+    return mllm_check_launch("add");
+}

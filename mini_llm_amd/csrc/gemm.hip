@@ -1,0 +1,218 @@
+// Matrix products on the matrix cores: out[M,N] = act(A[M,K] . W[N,K]^T + bias[N]) (+ residual).
+//
+// W is kept [out, in] (rows contiguous in K), which is what an MFMA operand wants and what the
+// tied head's token table already is. 32-bit inputs use the 32-bit MFMA (no reduced-precision
+// matrix mode); bfloat16 inputs use the bf16 MFMA; sums are 32-bit in both. Replaces the
+// reference's mult_kernel + add_bias + gelu + vector_addition (engine/src/matrixmult.cu:7-34,
+// linear.cu:9-18) and its epilogue order sum -> +bias -> activation -> residual + that
+// (engine/include/matvec_common.h:40-54).
+#include "common.h"
+
+namespace {
+
+template <typename T>
+struct Tile;
+template <>
+struct Tile<float> {
+    static constexpr int BK = 16;   // k elements per LDS tile
+    static constexpr int VEC = 4;   // elements per 16-byte vector
+    static constexpr int PAD = 4;
+};
+template <>
+struct Tile<bf16_t> {
+    static constexpr int BK = 32;
+    static constexpr int VEC = 8;
+    static constexpr int PAD = 8;
+};
+
+struct alignas(16) Vec16 {
+    uint32_t w[4];
+};
+
+// One 16-byte piece of a row, zero where the matrix ends. `aligned` says that every row starts
+// on a 16-byte boundary (K a multiple of VEC), else the piece is gathered element by element.
+template <typename T>
+__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k,
+                                            int K, bool aligned) {
+    constexpr int VEC = Tile<T>::VEC;
+    Vec16 v = {{0u, 0u, 0u, 0u}};
+    if (row >= n_rows || k >= K) return v;
+    const T* p = base + (size_t)row * K + k;
+    if (aligned && k + VEC <= K) {
+        v = *reinterpret_cast<const Vec16*>(p);
+    } else {
+        T* e = reinterpret_cast<T*>(&v);
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            if (k + i < K) e[i] = p[i];
+    }
+    return v;
+}
+
+// Block tile BM x BN, 4 waves laid out WAVES_M x WAVES_N, each wave TM x TN tiles of 32x32.
+template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, const T* __restrict__ W,
+                                                   const float* __restrict__ bias,
+                                                   const float* __restrict__ residual,
+                                                   OutT* __restrict__ out, int M, int N, int K,
+                                                   int epilogue) {
+    constexpr int BK = Tile<T>::BK, VEC = Tile<T>::VEC, PAD = Tile<T>::PAD;
+    constexpr int LDK = BK + PAD;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    constexpr int VPR = BK / VEC;  // 16-byte pieces per tile row
+    constexpr int A_PIECES = (BM * VPR + 255) / 256, W_PIECES = (BN * VPR + 255) / 256;
+    static_assert(WAVES_M * WAVES_N == 4 && TM >= 1 && TN >= 1, "tile layout");
+
+    __shared__ __attribute__((aligned(16))) T a_tile[BM * LDK];
+    __shared__ __attribute__((aligned(16))) T w_tile[BN * LDK];
+
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const bool aligned = (K % VEC) == 0;
+    const int half = lane / 32, lane32 = lane % 32;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    Vec16 a_next[A_PIECES], w_next[W_PIECES];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < A_PIECES; i++) {
+            int piece = tid + i * 256;
+            if (piece < BM * VPR) a_next[i] = load_piece<T>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K, aligned);
+        }
+#pragma unroll
+        for (int i = 0; i < W_PIECES; i++) {
+            int piece = tid + i * 256;
+            if (piece < BN * VPR) w_next[i] = load_piece<T>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, aligned);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_PIECES; i++) {
+            int piece = tid + i * 256;
+            if (piece < BM * VPR) *reinterpret_cast<Vec16*>(&a_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = a_next[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_PIECES; i++) {
+            int piece = tid + i * 256;
+            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = w_next[i];
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        __syncthreads();  // the previous tile has been consumed
+        stage();
+        __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);
+
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int kk = 0; kk < BK / 16; kk++) {
+                bf16x8 a[TM], b[TN];
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+                    a[i] = *reinterpret_cast<const bf16x8*>(
+                        &a_tile[(wave_m * TM * 32 + i * 32 + lane32) * LDK + kk * 16 + half * 8]);
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    b[j] = *reinterpret_cast<const bf16x8*>(
+                        &w_tile[(wave_n * TN * 32 + j * 32 + lane32) * LDK + kk * 16 + half * 8]);
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        } else {
+            // A lane takes four consecutive k of its row; component c of every lane forms the
+            // k pair of one 32x32x2 product, the same pairing on both operands.
+#pragma unroll
+            for (int kk = 0; kk < BK / 8; kk++) {
+                f32x4 a[TM], b[TN];
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+                    a[i] = *reinterpret_cast<const f32x4*>(
+                        &a_tile[(wave_m * TM * 32 + i * 32 + lane32) * LDK + kk * 8 + half * 4]);
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    b[j] = *reinterpret_cast<const f32x4*>(
+                        &w_tile[(wave_n * TN * 32 + j * 32 + lane32) * LDK + kk * 8 + half * 4]);
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][c], b[j][c], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+
+    // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
+            if (col >= N) continue;
+            float b = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                int row = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                if (row >= M) continue;
+                float value = acc[i][j][v] + b;
+                if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
+                else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+                size_t at = (size_t)row * N + col;
+                if (residual) value = residual[at] + value;
+                out[at] = from_float<OutT>(value);
+            }
+        }
+    }
+}
+
+template <typename T, typename OutT>
+void launch_gemm(const void* A, const void* W, const float* bias, const float* residual, void* out,
+                 int M, int N, int K, int epilogue, hipStream_t stream) {
+    const T* a = (const T*)A;
+    const T* w = (const T*)W;
+    OutT* o = (OutT*)out;
+    if (M <= 32) {
+        dim3 grid(ceil_div(N, 128), ceil_div(M, 32));
+        gemm_kernel<T, OutT, 32, 128, 1, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    } else if (M <= 64 || (long long)ceil_div(M, 128) * ceil_div(N, 128) < 128) {
+        dim3 grid(ceil_div(N, 64), ceil_div(M, 64));
+        gemm_kernel<T, OutT, 64, 64, 2, 2><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    } else {
+        dim3 grid(ceil_div(N, 128), ceil_div(M, 128));
+        gemm_kernel<T, OutT, 128, 128, 2, 2><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    }
+}
+
+}  // namespace
+
+MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const float* residual,
+                       void* out, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,
+                       hipStream_t stream) {
+    MLLM_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    MLLM_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
+    MLLM_REQUIRE(ceil_div(M, 32) <= 65535, "gemm: M=%d has too many row tiles", M);
+    if (M == 0) return 0;
+    if (in_dtype == MLLM_F32 && out_dtype == MLLM_F32)
+        launch_gemm<float, float>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+    else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_BF16)
+        launch_gemm<bf16_t, bf16_t>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+    else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_F32)
+        launch_gemm<bf16_t, float>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+    else
+        MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
+    return mllm_check_launch("gemm");
+}

@@ -1,0 +1,146 @@
+// Token choice on the device: argmax with numpy's rules, and temperature / top-p sampling.
+#include "common.h"
+
+namespace {
+
+constexpr int SAMPLE_THREADS = 1024;
+
+// (value, index) a comes before b: a NaN beats every number, a larger number a smaller one, and
+// among equals (-0 equals +0) the smaller index wins. These are numpy.argmax's rules, which the
+// reference keeps (engine/include/argmax.h:10-16, engine/src/argmax.cu:8-18).
+__device__ __forceinline__ bool beats(float value, int index, float best, int best_index) {
+    bool value_nan = value != value, best_nan = best != best;
+    if (value_nan != best_nan) return value_nan;
+    if (value_nan || value == best) return index < best_index;
+    return value > best;
+}
+
+__device__ __forceinline__ void block_best(float& value, int& index, float* shared_values,
+                                           int* shared_indices) {
+#pragma unroll
+    for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+        float other = __shfl_xor(value, offset, WAVE);
+        int other_index = __shfl_xor(index, offset, WAVE);
+        if (beats(other, other_index, value, index)) {
+            value = other;
+            index = other_index;
+        }
+    }
+    int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
+    __syncthreads();
+    if (lane == 0) {
+        shared_values[wave] = value;
+        shared_indices[wave] = index;
+    }
+    __syncthreads();
+    value = shared_values[0];
+    index = shared_indices[0];
+    for (int w = 1; w < n_waves; w++)
+        if (beats(shared_values[w], shared_indices[w], value, index)) {
+            value = shared_values[w];
+            index = shared_indices[w];
+        }
+}
+
+__device__ __forceinline__ float block_sum(float value, float* shared_values) {
+    value = wave_sum(value);
+    int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, n_waves = blockDim.x / WAVE;
+    __syncthreads();
+    if (lane == 0) shared_values[wave] = value;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < n_waves; w++) total += shared_values[w];  // same order in every thread
+    return total;
+}
+
+// Counter-based generator: the uniform number of (seed, step, index) is a pure function of the
+// three, so a draw does not depend on the batch, the launch shape or the order of evaluation.
+__device__ __forceinline__ float uniform_open(uint64_t seed, uint32_t step, uint32_t index) {
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * ((uint64_t)step + 1) + 0xD1B54A32D192ED03ull * ((uint64_t)index + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    return ((float)(z >> 40) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+}
+
+// One block per row. temperature 0: argmax. Otherwise a draw from softmax(logits / temperature)
+// cut to the nucleus top_p (token i stays if the mass of all strictly more likely tokens is
+// below top_p), taken as argmax(logit/temperature + Gumbel noise): it reuses the argmax
+// reduction and does not depend on a summation order.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    const float* __restrict__ logits, int vocab, const float* __restrict__ temperatures,
+    const float* __restrict__ top_ps, const uint64_t* __restrict__ seeds,
+    const int* __restrict__ steps, int* __restrict__ out_tokens) {
+    __shared__ float shared_values[SAMPLE_THREADS / WAVE];
+    __shared__ int shared_indices[SAMPLE_THREADS / WAVE];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const float* x = logits + (size_t)row * vocab;
+    const float temperature = temperatures ? temperatures[row] : 0.0f;
+
+    float best = -INFINITY;
+    int best_index = 0x7fffffff;
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS)
+        if (beats(x[i], i, best, best_index)) {
+            best = x[i];
+            best_index = i;
+        }
+    block_best(best, best_index, shared_values, shared_indices);
+    if (!(temperature > 0.0f) || best != best) {  // greedy, or a NaN in the row
+        if (tid == 0) out_tokens[row] = best_index;
+        return;
+    }
+
+    const float inverse_t = 1.0f / temperature;
+    const float top_p = top_ps ? top_ps[row] : 1.0f;
+    float cut = 0.0f;  // keep tokens whose weight exp((x - max)/T) is >= cut
+    if (top_p < 1.0f) {
+        float local = 0.0f;
+        for (int i = tid; i < vocab; i += SAMPLE_THREADS) local += expf((x[i] - best) * inverse_t);
+        float mass = block_sum(local, shared_values) * top_p;
+        // Smallest weight w (as an ordered bit pattern) with sum(weights > w) < mass. The sum is
+        // monotone in w, the weights lie in [0, 1], and the largest one is exactly 1.
+        uint32_t low = 0u, high = 0x3f800000u;  // high always satisfies it: nothing is above 1
+        while (low < high) {
+            uint32_t middle = low + (high - low) / 2;
+            float w = __uint_as_float(middle);
+            float above = 0.0f;
+            for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+                float e = expf((x[i] - best) * inverse_t);
+                above += e > w ? e : 0.0f;
+            }
+            if (block_sum(above, shared_values) < mass) high = middle;
+            else low = middle + 1;
+        }
+        cut = __uint_as_float(low);
+    }
+
+    const uint64_t seed = seeds ? seeds[row] : 0ull;
+    const uint32_t step = steps ? (uint32_t)steps[row] : 0u;
+    float chosen = -INFINITY;
+    int chosen_index = 0x7fffffff;
+    for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
+        float scaled = (x[i] - best) * inverse_t;
+        if (expf(scaled) >= cut) {
+            float u = uniform_open(seed, step, (uint32_t)i);
+            float noisy = scaled - logf(-logf(u));
+            if (beats(noisy, i, chosen, chosen_index)) {
+                chosen = noisy;
+                chosen_index = i;
+            }
+        }
+    }
+    block_best(chosen, chosen_index, shared_values, shared_indices);
+    if (tid == 0) out_tokens[row] = chosen_index;
+}
+
+}  // namespace
+
+MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float* temperatures,
+                         const float* top_ps, const unsigned long long* seeds, const int* steps,
+                         int* out_tokens, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", n_rows, vocab);
+    if (n_rows == 0) return 0;
+    sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, vocab, temperatures, top_ps,
+                                                         (const uint64_t*)seeds, steps, out_tokens);
+    return mllm_check_launch("sample");
+}

@@ -1,0 +1,194 @@
+"""The HIP kernels as functions on torch tensors.
+
+Every function checks on the host that its operands have the element types, shapes and layout
+the kernel and its grid assume, and raises otherwise: a kernel is never launched on operands it
+would read or write out of bounds. Tensors only carry memory; no torch operator computes
+anything here. Kernels run on torch's current stream."""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .library import check, library
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+EPILOGUES = {None: 0, "none": 0, "gelu_new": 1, "gelu": 2}
+
+
+class OperandError(ValueError):
+    pass
+
+
+def _require(condition: bool, message: str) -> None:
+    if not condition:
+        raise OperandError(message)
+
+
+def _code(dtype: torch.dtype) -> int:
+    _require(dtype in _DTYPE_CODE, f"no kernel for element type {dtype}")
+    return _DTYPE_CODE[dtype]
+
+
+def _device_tensor(t: torch.Tensor, name: str, dtype=None, dim=None) -> None:
+    _require(isinstance(t, torch.Tensor), f"{name} is not a tensor")
+    _require(t.is_cuda, f"{name} is not on the GPU: there is no CPU path")
+    if dtype is not None:
+        _require(t.dtype == dtype, f"{name} must be {dtype}, not {t.dtype}")
+    if dim is not None:
+        _require(t.dim() == dim, f"{name} must have {dim} dimensions, not {t.dim()}")
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+
+
+def _ptr(t: torch.Tensor | None):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def embed(tokens, positions, wte, wpe, out=None):
+    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32. A negative token gives a zero row."""
+    _device_tensor(tokens, "tokens", torch.int32, 1)
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(wte, "wte", dim=2)
+    _device_tensor(wpe, "wpe", wte.dtype, 2)
+    n, width = tokens.shape[0], wte.shape[1]
+    _require(positions.shape[0] == n, "tokens and positions differ in length")
+    _require(wpe.shape[1] == width, "wte and wpe differ in width")
+    if out is None:
+        out = torch.empty((n, width), dtype=torch.float32, device=tokens.device)
+    _device_tensor(out, "out", torch.float32, 2)
+    _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+    check(library().mllm_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _ptr(wpe), _ptr(out), n, width, _code(wte.dtype), _stream()))
+    return out
+
+
+def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None):
+    """Row LayerNorm of float32 rows; ``row_index`` (int32) picks the input row of each output row."""
+    _device_tensor(x, "x", torch.float32, 2)
+    width = x.shape[1]
+    _device_tensor(gamma, "gamma", torch.float32, 1)
+    _device_tensor(beta, "beta", torch.float32, 1)
+    _require(gamma.shape[0] == width and beta.shape[0] == width, "gamma/beta do not match the row width")
+    n = x.shape[0]
+    if row_index is not None:
+        _device_tensor(row_index, "row_index", torch.int32, 1)
+        n = row_index.shape[0]
+    if out is None:
+        out = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    _device_tensor(out, "out", out_dtype, 2)
+    _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+    check(library().mllm_layernorm(_ptr(x), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
+    return out
+
+
+def add(a, b, out=None):
+    """a (float32) + b (float32 or bfloat16) in float32."""
+    _device_tensor(a, "a", torch.float32)
+    _device_tensor(b, "b")
+    _require(a.shape == b.shape, "a and b differ in shape")
+    if out is None:
+        out = torch.empty_like(a)
+    _device_tensor(out, "out", torch.float32)
+    _require(out.shape == a.shape, "out has the wrong shape")
+    check(library().mllm_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), _code(b.dtype), _stream()))
+    return out
+
+
+def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None, out=None):
+    """act(x @ weight.T + bias) (+ residual). ``weight`` is [out, in]; sums are float32.
+
+    x and weight share their element type (float32: true 32-bit MFMA; bfloat16: bf16 MFMA);
+    bias and residual are float32; a residual makes the output float32."""
+    _device_tensor(x, "x", dim=2)
+    _device_tensor(weight, "weight", x.dtype, 2)
+    m, k = x.shape
+    n = weight.shape[0]
+    _require(weight.shape[1] == k, f"x has {k} columns but weight has {weight.shape[1]}")
+    _require(activation in EPILOGUES, f"unknown activation {activation!r}")
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == n, "bias does not match weight")
+    if out_dtype is None:
+        out_dtype = torch.float32 if residual is not None else x.dtype
+    if residual is not None:
+        _device_tensor(residual, "residual", torch.float32, 2)
+        _require(tuple(residual.shape) == (m, n), "residual has the wrong shape")
+        _require(out_dtype == torch.float32, "a residual sum is float32")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _device_tensor(out, "out", out_dtype, 2)
+    _require(tuple(out.shape) == (m, n), "out has the wrong shape")
+    _require(x.dtype != torch.float32 or out_dtype == torch.float32, "float32 inputs give float32 outputs")
+    check(library().mllm_gemm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x.dtype), _code(out_dtype), EPILOGUES[activation], _stream()))
+    return out
+
+
+def _check_pages(k_pages, v_pages, n_kv_heads, head_size):
+    _device_tensor(k_pages, "k_pages", dim=4)
+    _device_tensor(v_pages, "v_pages", k_pages.dtype, 4)
+    _require(k_pages.shape == v_pages.shape, "key and value pages differ in shape")
+    _require(k_pages.shape[1] == n_kv_heads and k_pages.shape[3] == head_size, "pages do not match the heads")
+    return k_pages.shape[0], k_pages.shape[2]
+
+
+def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
+    """Copies the key and value columns of each row into cache slot slots[row] (negative: skip).
+
+    k_src / v_src are 2-D views [rows, n_kv_heads*head_size] whose rows may be strided (slices
+    of a fused projection); pages are [num_pages, n_kv_heads, page_size, head_size]."""
+    num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    width = n_kv_heads * head_size
+    for t, name in ((k_src, "k_src"), (v_src, "v_src")):
+        _require(t.is_cuda and t.dim() == 2 and t.dtype == k_pages.dtype, f"{name} must be a 2-D GPU tensor of the pages' type")
+        _require(t.shape[1] == width and t.stride(1) == 1, f"{name} must have {width} contiguous columns")
+    _require(k_src.shape[0] == v_src.shape[0] and k_src.stride(0) == v_src.stride(0), "k_src and v_src differ in rows or stride")
+    _device_tensor(slots, "slots", torch.int32, 1)
+    n = k_src.shape[0]
+    _require(slots.shape[0] >= n, "fewer slots than rows")
+    check(library().mllm_cache_write(_ptr(k_src), _ptr(v_src), k_src.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(slots), n, n_kv_heads, head_size, page_size, _code(k_pages.dtype), _stream()))
+
+
+def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, out=None):
+    """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
+
+    q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
+    row of block_tables that holds the request's pages (negative: padding row, output zero)."""
+    _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    page_size = k_pages.shape[2]
+    width = n_heads * head_size
+    _require(q.is_cuda and q.dim() == 2 and q.dtype == k_pages.dtype, "q must be a 2-D GPU tensor of the pages' type")
+    _require(q.shape[1] == width and q.stride(1) == 1, f"q must have {width} contiguous columns")
+    n = q.shape[0]
+    _device_tensor(token_request, "token_request", torch.int32, 1)
+    _device_tensor(positions, "positions", torch.int32, 1)
+    _device_tensor(block_tables, "block_tables", torch.int32, 2)
+    _require(token_request.shape[0] >= n and positions.shape[0] >= n, "fewer positions than rows")
+    if out is None:
+        out = torch.empty((n, width), dtype=q.dtype, device=q.device)
+    _device_tensor(out, "out", q.dtype, 2)
+    _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+    check(library().mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
+    return out
+
+
+def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=None):
+    """One token per row of float32 logits. Without temperatures (or where one is 0): argmax by
+    numpy's rules. Else a draw from softmax(logits/temperature) within the top_p nucleus; the
+    random numbers are a function of (seeds[row], steps[row], token index) alone."""
+    _device_tensor(logits, "logits", torch.float32, 2)
+    n, vocab = logits.shape
+    for t, name, dtype in ((temperatures, "temperatures", torch.float32), (top_ps, "top_ps", torch.float32), (seeds, "seeds", torch.int64), (steps, "steps", torch.int32)):
+        if t is not None:
+            _device_tensor(t, name, dtype, 1)
+            _require(t.shape[0] >= n, f"{name} has fewer entries than rows")
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _device_tensor(out, "out", torch.int32, 1)
+    _require(out.shape[0] >= n, "out is too short")
+    check(library().mllm_sample(_ptr(logits), n, vocab, _ptr(temperatures), _ptr(top_ps), _ptr(seeds), _ptr(steps), _ptr(out), _stream()))
+    return out

@@ -1,0 +1,60 @@
+"""Loads the HIP kernel library with ctypes and declares its entry points.
+
+There is no fallback: without the library (or without a GPU) every op raises. The reference
+loads its engine the same way (pytorch/src/mini_llm/native.py:203-214); the path may be given
+with MINI_LLM_LIBRARY, as there."""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_float, c_int, c_longlong, c_void_p
+from pathlib import Path
+
+_library: ctypes.CDLL | None = None
+
+P = c_void_p
+_SIGNATURES = {
+    "mllm_embed": [P, P, P, P, P, c_int, c_int, c_int, P],
+    "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
+    "mllm_add": [P, P, P, c_longlong, c_int, P],
+    "mllm_gemm": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P],
+}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def library() -> ctypes.CDLL:
+    global _library
+    if _library is None:
+        path = os.environ.get("MINI_LLM_LIBRARY")
+        if path:
+            if not Path(path).is_file():
+                raise KernelLibraryError(f"MINI_LLM_LIBRARY={path} does not exist")
+        else:
+            from ..csrc import build
+
+            try:
+                path = str(build.ensure_built())
+            except build.BuildError as error:
+                raise KernelLibraryError(f"the HIP kernel library is missing and cannot be built: {error}") from None
+        lib = ctypes.CDLL(path)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+        lib.mllm_last_error.restype = ctypes.c_char_p
+        lib.mllm_last_error.argtypes = []
+        lib.path = path
+        _library = lib
+    return _library
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise KernelLibraryError(library().mllm_last_error().decode())

@@ -1,0 +1,293 @@
+"""Each kernel alone against a plain float64 reference, at sizes other than the engine's: odd
+row counts, widths and vocabularies that are no power of two, head sizes in steps of 16."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2 as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def K():
+    from mini_llm_amd.ops import kernels
+
+    return kernels
+
+
+def dev(a, dtype=torch.float32):
+    return torch.as_tensor(np.asarray(a)).to(DEV).to(dtype).contiguous()
+
+
+def host(t):
+    return t.detach().float().cpu().double().numpy()
+
+
+def bf16_round(a):
+    return torch.as_tensor(np.asarray(a, dtype=np.float32)).bfloat16().float().double().numpy()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width,vocab,npos", [(1, 64, 50, 8), (7, 96, 1000, 64), (33, 777, 513, 40)])
+def test_embed(K, dtype, rows, width, vocab, npos):
+    rng = np.random.default_rng(0)
+    wte, wpe = rng.standard_normal((vocab, width)), rng.standard_normal((npos, width))
+    tok = rng.integers(0, vocab, rows)
+    pos = rng.integers(0, npos, rows)
+    if rows > 2:
+        tok[1] = -1  # a padding row
+    out = K.embed(dev(tok, torch.int32), dev(pos, torch.int32), dev(wte, dtype), dev(wpe, dtype))
+    a, b = (wte, wpe) if dtype == torch.float32 else (bf16_round(wte), bf16_round(wpe))
+    ref = a[np.maximum(tok, 0)].astype(np.float32) + b[pos].astype(np.float32)
+    ref[tok < 0] = 0
+    np.testing.assert_allclose(host(out), ref, rtol=0, atol=1e-6)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (9, 768, 1e-5), (3, 1030, 1e-3), (2, 2500, 1e-5)])
+def test_layernorm(K, out_dtype, rows, width, eps):
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((rows, width)) * 2 + 50).astype(np.float32)  # a large mean
+    g, b = rng.standard_normal(width).astype(np.float32), rng.standard_normal(width).astype(np.float32)
+    out = K.layernorm(dev(x), dev(g), dev(b), eps, out_dtype=out_dtype)
+    ref = P.layernorm(x.astype(np.float64), g, b, eps)
+    tol = 2e-5 if out_dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(out), ref, rtol=tol, atol=tol)
+    if rows > 2:  # rows chosen by index
+        idx = np.array([rows - 1, 0, rows - 1])
+        out = K.layernorm(dev(x), dev(g), dev(b), eps, out_dtype=out_dtype, row_index=dev(idx, torch.int32))
+        np.testing.assert_allclose(host(out), ref[idx], rtol=tol, atol=tol)
+
+
+def test_layernorm_constant_row_gives_beta(K):
+    b = np.linspace(-1, 1, 96).astype(np.float32)
+    out = K.layernorm(dev(np.full((2, 96), 7.0)), dev(np.ones(96)), dev(b), 1e-5)
+    np.testing.assert_allclose(host(out), np.stack([b, b]), atol=1e-6)
+
+
+GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
+               (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+@pytest.mark.parametrize("activation", [None, "gelu_new", "gelu"])
+def test_linear_f32(K, m, n, k, activation):
+    rng = np.random.default_rng(m * 1000 + n)
+    x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
+    res = rng.standard_normal((m, n))
+    y = x.astype(np.float32).astype(np.float64) @ w.astype(np.float32).astype(np.float64).T + b.astype(np.float32)
+    if activation:
+        y = P.ACTIVATIONS[activation](y)
+    out = K.linear(dev(x), dev(w), dev(b), activation=activation)
+    np.testing.assert_allclose(host(out), y, rtol=1e-5, atol=1e-5)
+    out = K.linear(dev(x), dev(w), dev(b), activation=activation, residual=dev(res))
+    np.testing.assert_allclose(host(out), y + res.astype(np.float32), rtol=1e-5, atol=1e-5)
+    out = K.linear(dev(x), dev(w))
+    np.testing.assert_allclose(host(out), x.astype(np.float32).astype(np.float64) @ w.astype(np.float32).astype(np.float64).T, rtol=1e-5, atol=1e-5)
+
+
+def test_linear_f32_is_true_32_bit(K):
+    # values that a reduced-precision matrix mode (tf32/bf16 inputs) would round away
+    m, n, k = 8, 64, 64
+    x = np.full((m, k), 1.0 + 2.0**-20, dtype=np.float32)
+    w = np.full((n, k), 1.0 + 2.0**-21, dtype=np.float32)
+    out = host(K.linear(dev(x), dev(w)))
+    exact = k * (1.0 + 2.0**-20) * (1.0 + 2.0**-21)
+    assert abs(out[0, 0] - exact) < 1e-5 and abs(out[0, 0] - k) > 5e-5
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_linear_bf16(K, m, n, k, out_dtype):
+    rng = np.random.default_rng(m * 1000 + n + 1)
+    x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
+    y = bf16_round(x) @ bf16_round(w).T + b.astype(np.float32)
+    out = K.linear(dev(x, torch.bfloat16), dev(w, torch.bfloat16), dev(b), activation="gelu_new", out_dtype=out_dtype)
+    tol = 1e-2 if out_dtype == torch.bfloat16 else 2e-5
+    np.testing.assert_allclose(host(out), P.gelu_new(y), rtol=tol, atol=tol)
+    if out_dtype == torch.float32:
+        res = rng.standard_normal((m, n)).astype(np.float32)
+        out = K.linear(dev(x, torch.bfloat16), dev(w, torch.bfloat16), dev(b), residual=dev(res))
+        np.testing.assert_allclose(host(out), y + res, rtol=2e-5, atol=2e-5)
+
+
+def test_linear_reads_nothing_past_its_operands(K):
+    # NaN guards right after every operand: an out-of-bounds read would poison the result
+    m, n, k = 5, 37, 20
+    rng = np.random.default_rng(3)
+    xg = torch.full((m * k + 64,), float("nan"), device=DEV)
+    wg = torch.full((n * k + 64,), float("nan"), device=DEV)
+    x, w = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((n, k)).astype(np.float32)
+    xg[: m * k] = dev(x).flatten()
+    wg[: n * k] = dev(w).flatten()
+    og = torch.full((m * n + 64,), 123.0, device=DEV)
+    K.linear(xg[: m * k].view(m, k), wg[: n * k].view(n, k), out=og[: m * n].view(m, n))
+    np.testing.assert_allclose(host(og[: m * n].view(m, n)), x.astype(np.float64) @ w.T, rtol=1e-5, atol=1e-5)
+    assert (og[m * n :] == 123.0).all()  # and nothing written past the output
+
+
+def plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window):
+    """Rows of q are the LAST len(q) positions of a sequence whose keys are k_all/v_all."""
+    total, nq = k_all.shape[0], q.shape[0]
+    qfull = np.zeros((total, q.shape[1]))
+    qfull[total - nq :] = q
+    out = P.multi_head_attention(qfull, k_all, v_all, n_heads, n_kv_heads, window)
+    return out[total - nq :]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "n_heads,n_kv_heads,head_size,page_size,window",
+    [(4, 4, 16, 16, 0), (3, 3, 32, 64, 0), (5, 5, 48, 32, 0), (6, 2, 64, 16, 0), (2, 1, 80, 64, 0),
+     (2, 2, 128, 64, 0), (4, 2, 32, 16, 37), (1, 1, 256, 16, 0)],
+)
+def test_paged_attention(K, dtype, n_heads, n_kv_heads, head_size, page_size, window):
+    rng = np.random.default_rng(n_heads * 100 + head_size)
+    # three requests: (cached context, new tokens); pages handed out in a scrambled order
+    shapes = [(0, 70), (150, 1), (61, 9)]
+    num_pages = 40
+    order = rng.permutation(num_pages).tolist()
+    kp = torch.full((num_pages, n_kv_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
+    vp = torch.full_like(kp, float("nan"))
+    max_blocks = max((c + n + page_size - 1) // page_size for c, n in shapes)
+    tables = np.zeros((len(shapes), max_blocks), dtype=np.int32)
+    q_rows, treq, tpos, refs = [], [], [], []
+    rnd = lambda *s: bf16_round(rng.standard_normal(s)) if dtype == torch.bfloat16 else rng.standard_normal(s).astype(np.float32).astype(np.float64)
+    for r, (ctx, new) in enumerate(shapes):
+        total = ctx + new
+        k_all, v_all = rnd(total, n_kv_heads * head_size), rnd(total, n_kv_heads * head_size)
+        q = rnd(new, n_heads * head_size)
+        if r == 0:  # one far key stands out for the last query: a missed tile would show
+            k_all[3] = q[-1].reshape(n_heads, head_size)[:: n_heads // n_kv_heads].reshape(-1) * 4
+            k_all[3], q[-1] = rnd(1)[0] * 0 + bf16_round(k_all[3]) if dtype == torch.bfloat16 else k_all[3], q[-1]
+        n_blocks = (total + page_size - 1) // page_size
+        pages = [order.pop() for _ in range(n_blocks)]
+        tables[r, :n_blocks] = pages
+        slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+        # context goes in with one call, the new tokens with another (as in a later step)
+        for lo, hi in ((0, ctx), (ctx, total)):
+            if hi > lo:
+                K.cache_write(dev(k_all[lo:hi], dtype), dev(v_all[lo:hi], dtype), kp, vp, dev(slots[lo:hi], torch.int32), n_kv_heads, head_size)
+        q_rows.append(q)
+        treq += [r] * new
+        tpos += list(range(ctx, total))
+        refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window or None))
+    # a padding row in the middle
+    q_rows.insert(1, np.zeros((1, n_heads * head_size)))
+    treq.insert(shapes[0][1], -1)
+    tpos.insert(shapes[0][1], 0)
+    refs.insert(1, np.zeros((1, n_heads * head_size)))
+    out = K.paged_attention(
+        dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+        n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window,
+    )
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
+
+
+def test_paged_attention_strided_q(K):
+    # q, k, v as column slices of one fused projection
+    rng = np.random.default_rng(5)
+    H, hs, ps, n = 3, 32, 16, 21
+    qkv = rng.standard_normal((n, 3 * H * hs)).astype(np.float32)
+    t = dev(qkv)
+    kp = torch.zeros((4, H, ps, hs), device=DEV)
+    vp = torch.zeros_like(kp)
+    table = np.array([[2, 0, 3]], dtype=np.int32)
+    slots = np.array([table[0, p // ps] * ps + p % ps for p in range(n)], dtype=np.int32)
+    d = H * hs
+    K.cache_write(t[:, d : 2 * d], t[:, 2 * d :], kp, vp, dev(slots, torch.int32), H, hs)
+    out = K.paged_attention(t[:, :d], kp, vp, dev(np.zeros(n), torch.int32), dev(np.arange(n), torch.int32), dev(table, torch.int32), H, H, hs, 1 / math.sqrt(hs))
+    ref = P.multi_head_attention(qkv[:, :d].astype(np.float64), qkv[:, d : 2 * d], qkv[:, 2 * d :], H)
+    np.testing.assert_allclose(host(out), ref, rtol=2e-5, atol=2e-5)
+
+
+def numpy_rule_argmax(row):
+    nan = np.isnan(row)
+    return int(np.argmax(nan)) if nan.any() else int(np.argmax(row))
+
+
+@pytest.mark.parametrize("vocab", [1, 2, 63, 64, 65, 1000, 1024, 1025, 2049, 50257])
+def test_argmax_rules(K, vocab):
+    # engine/tests/test_argmax.cu:50-173 : ties, signed zero, -inf, NaN, borders of waves and blocks
+    rng = np.random.default_rng(vocab)
+    rows = [rng.standard_normal(vocab) for _ in range(4)]
+    rows.append(np.zeros(vocab)); rows[-1][::2] = -0.0           # +-0 are equal: first index wins
+    rows.append(np.full(vocab, -np.inf))                          # all -inf: index 0
+    t = rng.standard_normal(vocab); t[vocab // 2] = np.nan; t[vocab - 1] = np.nan; rows.append(t)  # first NaN
+    t = np.full(vocab, 1.0); t[vocab - 1] = 2.0; rows.append(t)   # the maximum at the very end
+    t = rng.standard_normal(vocab); t[[0, vocab // 3, vocab - 1]] = 9.0; rows.append(t)  # a tie across threads
+    x = np.stack(rows).astype(np.float32)
+    out = K.sample(dev(x)).cpu().numpy()
+    assert out.tolist() == [numpy_rule_argmax(r) for r in x]
+
+
+def test_temperature_sampling_distribution(K):
+    vocab, draws = 37, 20000
+    rng = np.random.default_rng(0)
+    logits = (rng.standard_normal(vocab) * 2).astype(np.float32)
+    x = dev(np.tile(logits, (draws, 1)))
+    temps = dev(np.full(draws, 0.7))
+    seeds = dev(np.full(draws, 1234), torch.int64)
+    steps = dev(np.arange(draws), torch.int32)
+    out = K.sample(x, temps, None, seeds, steps).cpu().numpy()
+    freq = np.bincount(out, minlength=vocab) / draws
+    p = P.softmax(logits.astype(np.float64) / 0.7)
+    assert np.abs(freq - p).max() < 4 * np.sqrt(p.max() / draws) + 1e-3
+    # the draw is a function of (seed, step) alone: same again, and in another batch order
+    again = K.sample(x, temps, None, seeds, steps).cpu().numpy()
+    assert (again == out).all()
+    perm = rng.permutation(draws)
+    shuffled = K.sample(x, temps, None, seeds, dev(np.arange(draws)[perm], torch.int32)).cpu().numpy()
+    assert (shuffled == out[perm]).all()
+    other = K.sample(x, temps, None, dev(np.full(draws, 99), torch.int64), steps).cpu().numpy()
+    assert (other != out).mean() > 0.3
+    # temperature 0 rows in the same call are greedy
+    mixed = K.sample(x[:4], dev([0.0, 0.7, 0.0, 0.7]), None, seeds[:4], steps[:4]).cpu().numpy()
+    assert mixed[0] == mixed[2] == int(np.argmax(logits))
+
+
+def test_top_p_sampling(K):
+    vocab, draws = 50, 8000
+    rng = np.random.default_rng(1)
+    logits = (rng.standard_normal(vocab) * 1.5).astype(np.float32)
+    logits[7] = logits[11]  # equal probabilities stand or fall together
+    T, top_p = 0.9, 0.6
+    p = P.softmax(logits.astype(np.float64) / T)
+    keep = P.top_p_keep(p, top_p)
+    x = dev(np.tile(logits, (draws, 1)))
+    out = K.sample(x, dev(np.full(draws, T)), dev(np.full(draws, top_p)), dev(np.full(draws, 5), torch.int64), dev(np.arange(draws), torch.int32)).cpu().numpy()
+    freq = np.bincount(out, minlength=vocab) / draws
+    assert freq[~keep].sum() == 0 and (freq[keep] > 0).all()
+    q = np.where(keep, p, 0) / p[keep].sum()
+    assert np.abs(freq - q).max() < 4 * np.sqrt(q.max() / draws) + 1e-3
+    # a tiny top_p leaves the most likely token only
+    out = K.sample(x[:50], dev(np.full(50, T)), dev(np.full(50, 1e-6)), dev(np.arange(50), torch.int64), dev(np.arange(50), torch.int32)).cpu().numpy()
+    assert (out == int(np.argmax(logits))).all()
+
+
+def test_add(K):
+    rng = np.random.default_rng(2)
+    a, b = rng.standard_normal((7, 33)).astype(np.float32), rng.standard_normal((7, 33)).astype(np.float32)
+    np.testing.assert_array_equal(host(K.add(dev(a), dev(b))), (a + b).astype(np.float64))
+    np.testing.assert_allclose(host(K.add(dev(a), dev(b, torch.bfloat16))), a + bf16_round(b), atol=1e-6)
+
+
+def test_operands_are_checked_on_the_host(K):
+    from mini_llm_amd.ops.kernels import OperandError
+
+    x = torch.zeros((4, 8), device=DEV)
+    with pytest.raises(OperandError):
+        K.linear(x, torch.zeros((3, 9), device=DEV))  # inner sizes differ
+    with pytest.raises(OperandError):
+        K.linear(torch.zeros((4, 8)), torch.zeros((3, 8)))  # CPU tensors: no CPU path
+    with pytest.raises(OperandError):
+        K.layernorm(x, torch.ones(7, device=DEV), torch.ones(8, device=DEV), 1e-5)
+    with pytest.raises(OperandError):
+        K.linear(x.t(), torch.zeros((3, 4), device=DEV))  # not contiguous
