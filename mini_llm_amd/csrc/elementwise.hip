@@ -52,7 +52,7 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     int source = row_index ? row_index[row] : row;
     const float* in_row = x + (size_t)source * width;
     OutT* out_row = out + (size_t)row * width;
-    float inverse_width = 1.0f / (float)width;
+    const float n = (float)width;  // divided by, not multiplied with its inverse: a constant row has mean exactly itself
 
     if constexpr (ROW_REGS > 0) {
         float values[ROW_REGS];
@@ -63,7 +63,7 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
             values[r] = i < width ? in_row[i] : 0.0f;
             sum += values[r];
         }
-        float mean = wave_sum(sum) * inverse_width;
+        float mean = wave_sum(sum) / n;
         float squares = 0.0f;
 #pragma unroll
         for (int r = 0; r < ROW_REGS; r++) {
@@ -71,7 +71,7 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
             float diff = i < width ? values[r] - mean : 0.0f;
             squares += diff * diff;
         }
-        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) * inverse_width + eps);
+        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) / n + eps);
 #pragma unroll
         for (int r = 0; r < ROW_REGS; r++) {
             int i = lane + r * WAVE;
@@ -81,13 +81,13 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     } else {
         float sum = 0.0f;
         for (int i = lane; i < width; i += WAVE) sum += in_row[i];
-        float mean = wave_sum(sum) * inverse_width;
+        float mean = wave_sum(sum) / n;
         float squares = 0.0f;
         for (int i = lane; i < width; i += WAVE) {
             float diff = in_row[i] - mean;
             squares += diff * diff;
         }
-        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) * inverse_width + eps);
+        float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) / n + eps);
         for (int i = lane; i < width; i += WAVE)
             out_row[i] = from_float<OutT>((in_row[i] - mean) * inverse_stddev * gamma[i] + beta[i]);
     }

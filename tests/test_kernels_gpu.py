@@ -95,11 +95,10 @@ def test_linear_f32(K, m, n, k, activation):
 def test_linear_f32_is_true_32_bit(K):
     # values that a reduced-precision matrix mode (tf32/bf16 inputs) would round away
     m, n, k = 8, 64, 64
-    x = np.full((m, k), 1.0 + 2.0**-20, dtype=np.float32)
-    w = np.full((n, k), 1.0 + 2.0**-21, dtype=np.float32)
+    x = np.full((m, k), 1.0 + 2.0**-12, dtype=np.float32)  # 12 fraction bits: tf32 keeps 10, bf16 7
+    w = np.ones((n, k), dtype=np.float32)
     out = host(K.linear(dev(x), dev(w)))
-    exact = k * (1.0 + 2.0**-20) * (1.0 + 2.0**-21)
-    assert abs(out[0, 0] - exact) < 1e-5 and abs(out[0, 0] - k) > 5e-5
+    assert (out == k * (1.0 + 2.0**-12)).all()  # exact in float32; a reduced mode gives 64.0
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -164,8 +163,8 @@ def test_paged_attention(K, dtype, n_heads, n_kv_heads, head_size, page_size, wi
         k_all, v_all = rnd(total, n_kv_heads * head_size), rnd(total, n_kv_heads * head_size)
         q = rnd(new, n_heads * head_size)
         if r == 0:  # one far key stands out for the last query: a missed tile would show
-            k_all[3] = q[-1].reshape(n_heads, head_size)[:: n_heads // n_kv_heads].reshape(-1) * 4
-            k_all[3], q[-1] = rnd(1)[0] * 0 + bf16_round(k_all[3]) if dtype == torch.bfloat16 else k_all[3], q[-1]
+            far = q[-1].reshape(n_heads, head_size)[:: n_heads // n_kv_heads].reshape(-1) * 4
+            k_all[3] = bf16_round(far) if dtype == torch.bfloat16 else far
         n_blocks = (total + page_size - 1) // page_size
         pages = [order.pop() for _ in range(n_blocks)]
         tables[r, :n_blocks] = pages
