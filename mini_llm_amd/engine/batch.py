@@ -1,0 +1,148 @@
+"""One step's batch: the tokens of several requests laid end to end, with everything the
+kernels need to find each token's request, position, cache rows and pages.
+
+The reference packs the control data of a batched decode into one struct and uploads it with a
+single pinned copy (engine/src/gpt2_gpu_batch.cu:18-24,91-113). The same is done here for mixed
+batches; pages are numbers, not pointers."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+
+
+@dataclass
+class StepEntry:
+    """A request's next tokens (a portion of its prompt, or one decoded token) and the places
+    among them whose logits are wanted."""
+
+    request_id: object
+    tokens: list
+    want: list = field(default_factory=list)
+
+
+@dataclass
+class GroupStepData:
+    block_tables: object   # int32 [n_requests, max_blocks]: pages of each request of the batch
+    slots: object          # int32 [n_tokens]: cache row each token's key/value is written to
+
+
+@dataclass
+class StepBatch:
+    n_tokens: int
+    n_requests: int
+    n_logit_rows: int
+    max_q_len: int          # the longest portion in the batch
+    max_total_len: int      # the longest sequence after this step
+    tokens: object          # int32 [n_tokens]
+    positions: object       # int32 [n_tokens]
+    token_request: object   # int32 [n_tokens]: row of the block tables (index into the batch)
+    q_starts: object        # int32 [n_requests + 1]: first row of each request's portion
+    context_lens: object    # int32 [n_requests]: tokens stored before this step
+    state_slots: object     # int32 [n_requests]
+    logit_rows: object      # int32 [n_logit_rows]: rows whose logits are computed
+    groups: list            # GroupStepData per cache group
+    request_ids: list = field(default_factory=list)
+    host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
+
+
+class BatchStaging:
+    """Pinned host buffers, used in turn, and the device buffer the batch is copied into. A
+    buffer is written again only after the copy out of it has finished."""
+
+    def __init__(self, device, ring: int = 4):
+        self.device, self.ring = device, ring
+        self._host, self._events, self._device = [], [], []
+        self._next = 0
+        self._capacity = 0
+
+    def _grow(self, n_ints: int) -> None:
+        import torch
+
+        torch.cuda.synchronize(self.device)
+        self._capacity = max(1024, 1 << (n_ints - 1).bit_length())
+        self._host = [torch.empty(self._capacity, dtype=torch.int32, pin_memory=True) for _ in range(self.ring)]
+        self._device = [torch.empty(self._capacity, dtype=torch.int32, device=self.device) for _ in range(self.ring)]
+        self._events = [None] * self.ring
+
+    def upload(self, flat: np.ndarray):
+        """flat: int32 numpy array -> device tensor holding it (valid until ``ring`` later uploads)."""
+        import torch
+
+        n = int(flat.shape[0])
+        if n > self._capacity:
+            self._grow(n)
+        i = self._next
+        self._next = (i + 1) % self.ring
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        self._host[i][:n].numpy()[:] = flat
+        self._device[i][:n].copy_(self._host[i][:n], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._events[i] = event
+        return self._device[i][:n]
+
+
+def _aligned(n: int) -> int:
+    return (n + 3) & ~3  # sections start on 16-byte boundaries
+
+
+def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int) -> StepBatch:
+    """Lays out the batch on the host and uploads it in one copy. The entries have been checked
+    and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests)."""
+    n_requests = len(entries)
+    q_lens = [len(e.tokens) for e in entries]
+    n_tokens = sum(q_lens)
+    contexts = [cache.length(e.request_id) for e in entries]
+    n_groups = len(cache.groups)
+    max_total = max(c + q for c, q in zip(contexts, q_lens))
+    table_width = cache.max_blocks() or max(1, -(-max_total // cache.page_size))
+
+    tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(contexts, q_lens)])
+    token_request = np.repeat(np.arange(n_requests, dtype=np.int32), q_lens)
+    q_starts = np.zeros(n_requests + 1, dtype=np.int32)
+    q_starts[1:] = np.cumsum(q_lens)
+    logit_rows = np.asarray([q_starts[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
+    state_slots = np.asarray([cache.requests[e.request_id].state_slot for e in entries], dtype=np.int32)
+    tables, slots = [], []
+    for gi in range(n_groups):
+        table = np.full((n_requests, table_width), -1, dtype=np.int32)
+        slot = np.empty(n_tokens, dtype=np.int32)
+        for i, e in enumerate(entries):
+            pages = np.asarray(cache.block_table(e.request_id, gi), dtype=np.int32)
+            table[i, : len(pages)] = pages
+            pos = positions[q_starts[i] : q_starts[i + 1]]
+            slot[q_starts[i] : q_starts[i + 1]] = pages[pos // cache.page_size] * cache.page_size + pos % cache.page_size
+        tables.append(table)
+        slots.append(slot)
+
+    sections = [tokens, positions, token_request, q_starts, np.asarray(contexts, dtype=np.int32), state_slots, logit_rows]
+    for table, slot in zip(tables, slots):
+        sections += [table.reshape(-1), slot]
+    offsets, total = [], 0
+    for section in sections:
+        offsets.append(total)
+        total += _aligned(len(section))
+    host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts,
+            "context_lens": sections[4], "state_slots": state_slots, "logit_rows": logit_rows,
+            "block_tables": tables, "slots": slots}
+    if staging is None:
+        views = sections
+    else:
+        flat = np.zeros(max(total, 4), dtype=np.int32)
+        for offset, section in zip(offsets, sections):
+            flat[offset : offset + len(section)] = section
+        device = staging.upload(flat)
+        views = [device[o : o + len(s)] for o, s in zip(offsets, sections)]
+    groups = [
+        GroupStepData(block_tables=views[7 + 2 * gi].reshape(n_requests, table_width), slots=views[8 + 2 * gi])
+        for gi in range(n_groups)
+    ]
+    return StepBatch(
+        n_tokens=n_tokens, n_requests=n_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens), max_total_len=max_total,
+        tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
+        state_slots=views[5], logit_rows=views[6], groups=groups, request_ids=[e.request_id for e in entries], host=host,
+    )

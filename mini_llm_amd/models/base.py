@@ -1,0 +1,113 @@
+"""A model as data: parts, distinct layers, and the order in which layers run.
+
+``schedule`` is a list of layer calls. A call names the layer (block) to run and the cache
+layer it uses; the same block may be called twice (shared weights, a cache of its own each
+time), and a call may read a cache layer that an earlier call wrote (``write_cache=False``)."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+from ..parts.base import Block, LayerContext, Norm, Part, PositionEncoding
+from ..parts.embedding import TokenEmbedding
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    block: int               # index into Model.blocks
+    cache: int               # cache layer (and state layer) this call uses
+    write_cache: bool = True
+
+
+@dataclass(frozen=True)
+class CacheGroupSpec:
+    """Cache layers with the same page geometry and the same retention share one pool of page
+    numbers and one block table per request."""
+
+    name: str
+    layers: tuple            # cache layer ids
+    n_kv_heads: int
+    head_size: int
+    window: int | None
+
+
+class Model(Part):
+    def __init__(self, config, precision, *, embedding: TokenEmbedding, position_encoding: PositionEncoding | None,
+                 blocks: list, schedule: list, final_norm: Norm, head, names: dict):
+        self.config, self.precision = config, precision
+        self.embedding, self.position_encoding = embedding, position_encoding
+        self.blocks, self.schedule = list(blocks), list(schedule)
+        self.final_norm, self.head = final_norm, head
+        self._names = names  # prefixes: embedding, position_encoding, block (format with {i}), final_norm
+        written = set()
+        for call in self.schedule:
+            if not 0 <= call.block < len(self.blocks):
+                raise ValueError(f"the schedule names layer {call.block}, but there are {len(self.blocks)}")
+            if call.write_cache:
+                if call.cache in written:
+                    raise ValueError(f"cache layer {call.cache} is written by two layer calls")
+                written.add(call.cache)
+            elif call.cache not in written:
+                raise ValueError(f"a layer call reads cache layer {call.cache} before any call has written it")
+
+    # -- tree ------------------------------------------------------------------------------------
+    def children(self):
+        out = {self._names["embedding"]: self.embedding}
+        if self.position_encoding is not None:
+            out[self._names["position_encoding"]] = self.position_encoding
+        for i, block in enumerate(self.blocks):
+            out[self._names["block"].format(i=i)] = block
+        out[self._names["final_norm"]] = self.final_norm
+        return out
+
+    def canonical_tensor_name(self, name: str) -> str | None:
+        """Name in a file -> name in ``named_tensor_specs`` (None: known and not needed)."""
+        return name
+
+    # -- what the engine asks ----------------------------------------------------------------------
+    @property
+    def vocab_size(self) -> int:
+        return self.embedding.vocab_size
+
+    def max_positions(self) -> int | None:
+        """The longest sequence the model can hold (None: no limit of its own)."""
+        if self.position_encoding is not None and hasattr(self.position_encoding, "max_positions"):
+            return self.position_encoding.max_positions()
+        return None
+
+    def cache_groups(self) -> list[CacheGroupSpec]:
+        groups: dict = {}
+        for call in self.schedule:
+            need = self.blocks[call.block].mixer_part().kv_need()
+            if need is None:
+                continue
+            layers = groups.setdefault((need.n_kv_heads, need.head_size, need.window), [])
+            if call.write_cache:
+                layers.append(call.cache)
+            elif call.cache not in layers:
+                raise ValueError(f"a layer call reads cache layer {call.cache}, whose pages have another shape or window")
+        return [
+            CacheGroupSpec(f"{'window' + str(key[2]) if key[2] else 'full'}_h{key[0]}x{key[1]}", tuple(layers), *key)
+            for key, layers in groups.items()
+        ]
+
+    def state_needs(self) -> dict:
+        """state layer id -> StateNeed, for the mixers that keep state of fixed size."""
+        out = {}
+        for call in self.schedule:
+            need = self.blocks[call.block].mixer_part().state_need()
+            if need is not None and call.write_cache:
+                out[call.cache] = need
+        return out
+
+    def forward(self, batch, cache):
+        """The whole step: embeds the batch's tokens, runs the schedule over the cache, and
+        returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only."""
+        hidden = self.embedding.forward(batch.tokens, batch.positions, self.position_encoding)
+        for call in self.schedule:
+            hidden = self.blocks[call.block].forward(hidden, cache.layer_context(batch, call))
+        if batch.n_logit_rows == 0:
+            return None
+        # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
+        normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
+        return self.head.forward(normed)

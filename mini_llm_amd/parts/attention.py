@@ -1,0 +1,56 @@
+"""Causal multi-head attention over the paged cache, with a fused q/k/v projection.
+
+Formulas in the reference's order: q, k, v are column blocks of one product
+(engine/src/gpt2.c:79-90); head h owns columns [h*hs, (h+1)*hs) (engine/src/attention.c:78-97);
+scores scaled by 1/sqrt(head size), causal, softmax in 32-bit (engine/src/attention.cu:90-123);
+the output projection adds its bias and the residual (engine/src/transformer_block.c:60-62)."""
+
+from __future__ import annotations
+
+import math
+
+from ..ops import kernels
+from .base import KVNeed, LayerContext, Mixer, register_part
+from .linear import Linear
+
+
+class CausalSelfAttention(Mixer):
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int | None = None, head_size: int | None = None,
+                 window: int | None = None, out_std: float = 0.02, qkv_name: str = "c_attn.", out_name: str = "c_proj."):
+        self.width, self.n_heads = width, n_heads
+        self.n_kv_heads = n_heads if n_kv_heads is None else n_kv_heads
+        self.head_size = width // n_heads if head_size is None else head_size
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError(f"{n_heads} heads do not divide into {self.n_kv_heads} key/value heads")
+        if self.head_size % 16 or not 16 <= self.head_size <= 256:
+            raise ValueError(f"head size {self.head_size} is not a multiple of 16 in 16..256")
+        self.window = window
+        self.scale = 1.0 / math.sqrt(self.head_size)
+        self.q_width = self.n_heads * self.head_size
+        self.kv_width = self.n_kv_heads * self.head_size
+        self.qkv = Linear(width, self.q_width + 2 * self.kv_width)
+        self.out = Linear(self.q_width, width, weight_std=out_std)
+        self._names = (qkv_name, out_name)
+
+    def children(self):
+        return {self._names[0]: self.qkv, self._names[1]: self.out}
+
+    def kv_need(self):
+        return KVNeed(self.n_kv_heads, self.head_size, self.window)
+
+    def forward(self, x, residual, ctx: LayerContext):
+        qkv = self.qkv.forward(x)
+        q = qkv[:, : self.q_width]
+        if ctx.write_cache:
+            k = qkv[:, self.q_width : self.q_width + self.kv_width]
+            v = qkv[:, self.q_width + self.kv_width :]
+            kernels.cache_write(k, v, ctx.k_pages, ctx.v_pages, ctx.group.slots, self.n_kv_heads, self.head_size)
+        mixed = kernels.paged_attention(
+            q, ctx.k_pages, ctx.v_pages, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
+            self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
+            max_q_len=ctx.batch.max_q_len,
+        )
+        return self.out.forward(mixed, residual=residual)
+
+
+register_part("mixer", "causal_attention", CausalSelfAttention)

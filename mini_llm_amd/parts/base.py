@@ -1,0 +1,139 @@
+"""The interfaces of the parts a layer is put together from, and one registry per kind.
+
+A part owns its sizes and constants as constructor parameters, declares the tensors it needs
+(``tensor_specs``), receives them (``bind``) and computes (``forward``). No part knows which
+model it is in: the architecture's builder picks parts by name, layer by layer."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+from ..weights.spec import TensorSpec
+
+
+class Part:
+    """A node of the model tree: its own tensors plus named children."""
+
+    def tensor_specs(self) -> dict[str, TensorSpec]:
+        """local tensor name -> spec, for this part's own tensors."""
+        return {}
+
+    def children(self) -> dict[str, "Part"]:
+        """name prefix -> sub-part."""
+        return {}
+
+    def bind(self, tensors: dict) -> None:
+        """Receives this part's own tensors, already on the device in the kept layout."""
+        for name, tensor in tensors.items():
+            setattr(self, name.replace(".", "_"), tensor)
+
+    # -- walking the tree ------------------------------------------------------------------
+    def named_tensor_specs(self, prefix: str = "") -> dict[str, TensorSpec]:
+        out = {prefix + name: spec for name, spec in self.tensor_specs().items()}
+        for child_prefix, child in self.children().items():
+            out.update(child.named_tensor_specs(prefix + child_prefix))
+        return out
+
+    def bind_named(self, tensors: dict, prefix: str = "") -> None:
+        own = {name: tensors[prefix + name] for name in self.tensor_specs()}
+        if own:
+            self.bind(own)
+        for child_prefix, child in self.children().items():
+            child.bind_named(tensors, prefix + child_prefix)
+
+
+# -- what a mixer may ask of the cache manager ---------------------------------------------------
+@dataclass(frozen=True)
+class KVNeed:
+    """Keys and values that grow with the sequence, kept in pages. ``window`` None: every key
+    is kept; an integer w: only the last w keys are ever read, older pages are given back."""
+
+    n_kv_heads: int
+    head_size: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """State of fixed size per request, kept in a slot: zero at admission, updated in place."""
+
+    shape: tuple
+    dtype: object  # torch.dtype
+
+
+@dataclass
+class LayerContext:
+    """What the step function hands a mixer for one layer call."""
+
+    batch: object                 # engine.batch.StepBatch: tokens, positions, requests
+    k_pages: object = None        # [num_pages, n_kv_heads, page_size, head_size] of the call's cache layer
+    v_pages: object = None
+    group: object = None          # cache.GroupStepData: block tables and write slots of the layer's group
+    write_cache: bool = True      # False: the layer reads a cache another layer call has written
+    state: object = None          # [num_slots, *StateNeed.shape] of the call's state layer
+    extra: dict = field(default_factory=dict)
+
+
+class Norm(Part):
+    def forward(self, x, out_dtype, row_index=None):
+        """x: [rows, width] float32 -> [rows or len(row_index), width] of out_dtype."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    """Mixes information between the positions of a sequence (attention here)."""
+
+    def kv_need(self) -> KVNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x, residual, ctx: LayerContext):
+        """x: [rows, width] normed input in the compute dtype; returns residual + mix(x) in
+        float32. Rows belong to several requests and may be a portion of a prompt or one decoded
+        token; what came before is in the cache / the state slot."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, residual):
+        """x: [rows, width] in the compute dtype; returns residual + f(x) in float32."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """How positions enter the model. ``stage`` says where: 'embedding' (added to the token
+    rows) or 'mixer' (applied to queries and keys inside the mixer)."""
+
+    stage = "embedding"
+
+
+class Block(Part):
+    def forward(self, hidden, ctx: LayerContext):
+        """hidden: [rows, width] float32 residual stream -> the same after this layer."""
+        raise NotImplementedError
+
+    def mixer_part(self) -> Mixer:
+        raise NotImplementedError
+
+
+# -- registries -----------------------------------------------------------------------------------
+NORMS: dict[str, type] = {}
+MIXERS: dict[str, type] = {}
+FEED_FORWARDS: dict[str, type] = {}
+POSITION_ENCODINGS: dict[str, type] = {}
+BLOCKS: dict[str, type] = {}
+_KINDS = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS, "position_encoding": POSITION_ENCODINGS, "block": BLOCKS}
+
+
+def register_part(kind: str, name: str, cls: type) -> None:
+    """kind: norm | mixer | feed_forward | position_encoding | block."""
+    _KINDS[kind][name] = cls
+
+
+def make_part(kind: str, name: str, **parameters):
+    table = _KINDS[kind]
+    if name not in table:
+        raise KeyError(f"no {kind} named {name!r}; registered: {', '.join(sorted(table))}")
+    return table[name](**parameters)

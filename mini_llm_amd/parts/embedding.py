@@ -1,0 +1,35 @@
+"""The token table, read at the bottom of the model (gather) and, tied, at the top (head)."""
+
+from __future__ import annotations
+
+from ..ops import kernels
+from ..weights.spec import TABLE, Normal, TensorSpec
+from .base import Part, PositionEncoding
+
+
+class TokenEmbedding(Part):
+    def __init__(self, vocab_size: int, width: int):
+        self.vocab_size, self.width = vocab_size, width
+        self.weight = None
+
+    def tensor_specs(self):
+        return {"weight": TensorSpec((self.vocab_size, self.width), TABLE, Normal(0.02))}
+
+    def forward(self, tokens, positions, position_encoding: PositionEncoding | None):
+        """[rows, width] float32: token rows, with the position rows added when the encoding
+        is one that enters at the embedding."""
+        if position_encoding is None or position_encoding.stage != "embedding":
+            raise NotImplementedError("only encodings added at the embedding have a kernel here")
+        return kernels.embed(tokens, positions, self.weight, position_encoding.weight)
+
+
+class TiedHead(Part):
+    """logits = x . wte^T, no bias, no tensor of its own (engine/src/gpt2.c:244-256)."""
+
+    def __init__(self, embedding: TokenEmbedding):
+        self.embedding = embedding
+
+    def forward(self, x):
+        import torch
+
+        return kernels.linear(x, self.embedding.weight, out_dtype=torch.float32)

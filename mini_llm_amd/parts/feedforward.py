@@ -1,0 +1,30 @@
+"""Dense feed-forward: up projection, activation, down projection, residual sum
+(engine/src/transformer_block.c:64-71). The activation is fused into the up product and the
+residual sum into the down product."""
+
+from __future__ import annotations
+
+from .base import FeedForward, register_part
+from .linear import Linear
+
+ACTIVATIONS = ("gelu_new", "gelu")
+
+
+class DenseMLP(FeedForward):
+    def __init__(self, width: int, inner: int, activation: str, down_std: float = 0.02,
+                 up_name: str = "c_fc.", down_name: str = "c_proj."):
+        if activation not in ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {ACTIVATIONS}")
+        self.width, self.inner, self.activation = width, inner, activation
+        self.up = Linear(width, inner)
+        self.down = Linear(inner, width, weight_std=down_std)
+        self._names = (up_name, down_name)
+
+    def children(self):
+        return {self._names[0]: self.up, self._names[1]: self.down}
+
+    def forward(self, x, residual):
+        return self.down.forward(self.up.forward(x, activation=self.activation), residual=residual)
+
+
+register_part("feed_forward", "dense_mlp", DenseMLP)

@@ -1,0 +1,28 @@
+"""A linear map y = x W + b as a part: weight stored [in, out] (GPT-2's Conv1D) or [out, in],
+kept [out, in] for the matrix kernels, with the epilogue (activation, residual sum) fused."""
+
+from __future__ import annotations
+
+from ..ops import kernels
+from ..weights.spec import MATRIX, VECTOR, Normal, TensorSpec
+from .base import Part
+
+
+class Linear(Part):
+    def __init__(self, in_features: int, out_features: int, *, bias: bool = True, stored_in_out: bool = True,
+                 weight_std: float = 0.02, bias_std: float = 0.01):
+        self.in_features, self.out_features = in_features, out_features
+        self.has_bias, self.stored_in_out = bias, stored_in_out
+        self.weight_std, self.bias_std = weight_std, bias_std
+        self.weight = None
+        self.bias = None
+
+    def tensor_specs(self):
+        shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
+        specs = {"weight": TensorSpec(shape, MATRIX, Normal(self.weight_std), keep_transposed=self.stored_in_out)}
+        if self.has_bias:
+            specs["bias"] = TensorSpec((self.out_features,), VECTOR, Normal(self.bias_std))
+        return specs
+
+    def forward(self, x, activation=None, residual=None, out_dtype=None):
+        return kernels.linear(x, self.weight, self.bias, activation=activation, residual=residual, out_dtype=out_dtype)

@@ -1,0 +1,163 @@
+"""Helpers for the replay tests: traces in the four ways of cutting the work, a driver for
+bin/trace_run, and the plain implementation's logits to compare with."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import numpy as np
+
+import plain_gpt2
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, timeout=600):
+    """Runs bin/trace_run over the steps; returns {step: array [wanted, vocab]}."""
+    out_dir = Path(out_dir)
+    cmd = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
+           "--out", str(out_dir), "--max-tokens", str(max_tokens)]
+    if page_size:
+        cmd += ["--page-size", str(page_size)]
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    done = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=timeout)
+    assert done.returncode == 0, f"trace_run failed ({done.returncode}):\n{done.stderr[-3000:]}"
+    assert [l for l in done.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    vocab = json.loads((Path(model_dir) / "config.json").read_text())["vocab_size"]
+    out = {}
+    for s in steps:
+        wanted = sum(len(e.get("want", [])) for e in s["entries"])
+        path = out_dir / f"{s['step']}.f32"
+        if wanted:
+            out[s["step"]] = np.fromfile(path, dtype="<f4").reshape(wanted, vocab)
+        else:
+            assert not path.exists()
+    return out
+
+
+class Collector:
+    """Gathers, per request, the logits of each position from the steps' outputs."""
+
+    def __init__(self):
+        self.steps = []
+        self.where = []  # per step: list of (request, position) in output order
+        self.fed = {}
+
+    def add(self, entries, end=()):
+        """entries: [(request, tokens, want)]; positions follow from what was fed before."""
+        places, recs = [], []
+        for request, tokens, want in entries:
+            start = self.fed.get(request, 0)
+            recs.append({"id": request, "tokens": [int(t) for t in tokens], "want": [int(w) for w in want]})
+            places += [(request, start + w) for w in want]
+            self.fed[request] = start + len(tokens)
+        self.steps.append({"step": len(self.steps), "entries": recs, "end": list(end)})
+        self.where.append(places)
+        for request in end:
+            self.fed.pop(request, None)
+
+    def gather(self, outputs):
+        """{request: {position: logits row}}"""
+        got = {}
+        for step, places in zip(self.steps, self.where):
+            if places:
+                rows = outputs[step["step"]]
+                for row, (request, position) in zip(rows, places):
+                    got.setdefault(request, {})[position] = row
+        return got
+
+
+def whole(requests):
+    """Each request alone, all its tokens in one step, every position wanted."""
+    c = Collector()
+    for name, tokens in requests.items():
+        c.add([(name, tokens, range(len(tokens)))], end=[name])
+    return c
+
+
+def prefill_then_decode(requests, tail=32):
+    """All but the last ``tail`` tokens in one step, then the rest one by one."""
+    c = Collector()
+    for name, tokens in requests.items():
+        head = max(1, len(tokens) - tail)
+        c.add([(name, tokens[:head], range(head))])
+        for i in range(head, len(tokens)):
+            c.add([(name, tokens[i : i + 1], [0])], end=[name] if i == len(tokens) - 1 else [])
+        if head == len(tokens):
+            c.add([], end=[name])
+    return c
+
+
+def chunked(requests, sizes=(7, 2, 16, 3, 2, 33, 5, 2, 64, 11)):
+    """Portions of changing size, down to two tokens."""
+    c = Collector()
+    for name, tokens in requests.items():
+        at, i = 0, 0
+        while at < len(tokens):
+            n = min(sizes[i % len(sizes)], len(tokens) - at)
+            i += 1
+            last = at + n == len(tokens)
+            c.add([(name, tokens[at : at + n], range(n))], end=[name] if last else [])
+            at += n
+    return c
+
+
+def mixed(requests, seed=0, max_live=4, tail=12):
+    """Up to ``max_live`` live requests: portions of some beside single decoded tokens of
+    others; a request is sometimes left out of a step; requests join as others end."""
+    rng = np.random.default_rng(seed)
+    c = Collector()
+    waiting = list(requests.items())
+    live = {}  # name -> [tokens, fed]
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            name, tokens = waiting.pop(0)
+            live[name] = [tokens, 0]
+        entries, ended = [], []
+        for name, (tokens, fed) in list(live.items()):
+            if len(live) > 1 and rng.random() < 0.2:
+                continue  # left out of this step
+            left = len(tokens) - fed
+            if left <= tail:
+                n = 1  # the last tokens go one by one, as decoded tokens would
+            else:
+                n = int(min(left - tail, rng.choice([2, 3, 5, 8, 13, 21, 40])))
+            entries.append((name, tokens[fed : fed + n], range(n)))
+            live[name][1] = fed + n
+            if fed + n == len(tokens):
+                ended.append(name)
+                del live[name]
+        if entries:
+            c.add(entries, end=ended)
+    return c
+
+
+def peak_tokens(collector, page=64):
+    """The most tokens live requests hold at any time, each rounded up to a multiple of ``page``."""
+    held, peak = {}, 0
+    for step in collector.steps:
+        for e in step["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        peak = max(peak, sum(-(-n // page) * page for n in held.values()))
+        for name in step["end"]:
+            held.pop(name, None)
+    return peak
+
+
+def plain_logits(config, weights, requests, dtype=np.float64):
+    return {name: plain_gpt2.forward(config, weights, tokens, dtype) for name, tokens in requests.items()}
+
+
+def compare(got, ref, atol, rtol):
+    """Every position of every request; on a mismatch names the first wrong place."""
+    for name, rows in ref.items():
+        assert set(got[name]) == set(range(len(rows))), f"{name}: positions {sorted(set(range(len(rows))) - set(got[name]))} missing"
+        for position in range(len(rows)):
+            a, b = got[name][position].astype(np.float64), rows[position]
+            err = np.abs(a - b)
+            bad = err > atol + rtol * np.abs(b)
+            assert not bad.any(), (
+                f"request {name!r} position {position}: {int(bad.sum())} logits differ, max error {err.max():.3e} "
+                f"(allowed {atol:g} + {rtol:g}*|ref|); first wrong position of this request"
+            )
