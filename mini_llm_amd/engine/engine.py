@@ -1,0 +1,224 @@
+"""The Python entry point: a model folder (or a configuration and a seed) in, tokens out.
+
+Named after the reference's binding (pytorch/src/mini_llm/native.py): ``EngineOptions``, an
+engine object that is a context manager, ``forward_last``, sessions with ``prefill`` /
+``decode``, and the four calls its scheduler drives (``try_take_cache``, ``release_cache``,
+``prefill_greedy``, ``decode_batch``: pytorch/src/mini_llm/batch_api.py:33-70). Above them sits
+this framework's own scheduler with ``submit`` / ``step`` / ``generate``."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+from ..cache import OutOfPages
+from ..sampling import SamplingParams
+from .batch import StepEntry
+from .loading import DEFAULT_PAGE_SIZE, load_model, make_cache, random_model
+from .scheduler import Request, Scheduler
+from .step import ModelRunner, StepError
+
+
+@dataclass(frozen=True)
+class EngineOptions:
+    """How the engine is sized. ``max_sessions`` is the reference's name for the number of
+    requests that can be live at once (native.py:31-38)."""
+
+    dtype: str = "bfloat16"
+    max_sessions: int = 64
+    max_tokens: int | None = None        # cache capacity in tokens; None: max_sessions full contexts
+    page_size: int = DEFAULT_PAGE_SIZE
+    max_tokens_per_step: int = 2048      # token budget of one scheduler step
+    device: str = "cuda:0"
+
+
+class _Executor:
+    """The scheduler's view of the runner, the cache and the sampler."""
+
+    def __init__(self, engine: "Engine"):
+        self._engine = engine
+        self.page_size = engine.cache.page_size
+
+    def max_positions(self):
+        return self._engine.model.max_positions()
+
+    def check_prompt(self, tokens):
+        limit, vocab = self.max_positions(), self._engine.model.vocab_size
+        if limit is not None and len(tokens) > limit:
+            raise ValueError(f"the prompt has {len(tokens)} tokens; the model holds {limit}")
+        for token in tokens:
+            if not 0 <= int(token) < vocab:
+                raise ValueError(f"token {token} is outside the vocabulary [0, {vocab})")
+
+    def can_open(self):
+        return self._engine.cache.can_open()
+
+    def open(self, request_id):
+        self._engine.cache.open(("scheduled", request_id))
+
+    def close(self, request_id):
+        self._engine.cache.close(("scheduled", request_id))
+
+    def length(self, request_id):
+        return self._engine.cache.length(("scheduled", request_id))
+
+    def fits(self, wanted):
+        return self._engine.cache.can_reserve([(("scheduled", r), n) for r, n in wanted])
+
+    def run(self, entries, sampling, steps):
+        entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want) for e in entries]
+        logits = self._engine.runner.step(entries)
+        if logits is None:
+            return []
+        return self._engine.sampler.sample(logits, sampling, steps).cpu().tolist()
+
+
+class Session:
+    """One sequence driven by hand: prefill a prompt (in one or several portions), then decode
+    token by token; each call returns the logits after its last token (the reference's
+    CachedSession, native.py:88-166)."""
+
+    def __init__(self, engine: "Engine", handle):
+        self._engine, self._handle = engine, handle
+
+    def _active(self):
+        if self._engine is None:
+            raise RuntimeError("the session is closed")
+        return self._engine
+
+    def prefill(self, token_ids) -> np.ndarray:
+        tokens = [int(t) for t in token_ids]
+        logits = self._active().runner.step([StepEntry(self._handle, tokens, [len(tokens) - 1])])
+        return logits[0].cpu().numpy()
+
+    def decode(self, token_id: int) -> np.ndarray:
+        return self.prefill([token_id])
+
+    def length(self) -> int:
+        return self._active().cache.length(self._handle)
+
+    def close(self) -> None:
+        if self._engine is not None:
+            self._engine.release_cache(self._handle)
+            self._engine = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *_):
+        self.close()
+
+
+class Engine:
+    def __init__(self, model_dir=None, options: EngineOptions = EngineOptions(), *, model=None):
+        """model_dir: folder with config.json and model.safetensors. ``model``: an already
+        loaded model instead (see ``from_random``)."""
+        from ..ops import library
+        from ..sampling import Sampler
+
+        library()  # fails loudly here if the kernels are missing
+        self.options = options
+        self.model = model if model is not None else load_model(model_dir, options.dtype, options.device)
+        limit = self.model.max_positions() or 4096
+        max_tokens = options.max_tokens or options.max_sessions * limit
+        self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
+                                max_requests=options.max_sessions, device=options.device)
+        self.runner = ModelRunner(self.model, self.cache, options.device)
+        self.sampler = Sampler(self.runner.staging)
+        self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step)
+        self._next_handle = 0
+
+    @classmethod
+    def from_random(cls, config, seed: int, options: EngineOptions = EngineOptions()):
+        """An engine over random weights of the given typed configuration."""
+        return cls(options=options, model=random_model(config, seed, options.dtype, options.device))
+
+    @property
+    def config(self):
+        return self.model.config
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *_):
+        self.close()
+
+    def close(self) -> None:
+        if self.scheduler.is_running():
+            self.scheduler.stop()
+
+    # --- one sequence at a time (native.py) ---------------------------------------------------------
+    def forward_last(self, token_ids) -> np.ndarray:
+        """Logits after the last token of a whole sequence; nothing is kept."""
+        with self.open_session() as session:
+            return session.prefill(token_ids)
+
+    def open_session(self) -> Session:
+        handle = self.try_take_cache()
+        if handle is None:
+            raise RuntimeError("all sessions are taken")
+        return Session(self, handle)
+
+    # --- the calls the reference's scheduler drives (batch_api.py) --------------------------------------
+    def try_take_cache(self):
+        """A handle for a new sequence, or None when all are taken. Never waits."""
+        if not self.cache.can_open():
+            return None
+        handle = ("session", self._next_handle)
+        self._next_handle += 1
+        self.cache.open(handle)
+        return handle
+
+    def release_cache(self, handle) -> None:
+        self.cache.close(handle)
+
+    def prefill_greedy(self, handle, token_ids) -> int:
+        tokens = [int(t) for t in token_ids]
+        if not tokens:
+            raise RuntimeError("the prompt has no tokens")
+        logits = self.runner.step([StepEntry(handle, tokens, [len(tokens) - 1])])
+        return int(self.sampler.sample(logits, [SamplingParams()], [0]).cpu()[0])
+
+    def decode_batch(self, handles, tokens) -> list[int]:
+        if len(handles) != len(tokens) or not handles:
+            raise RuntimeError("a batch has one token per sequence and at least one sequence")
+        logits = self.runner.step([StepEntry(h, [int(t)], [0]) for h, t in zip(handles, tokens)])
+        return self.sampler.sample(logits, [SamplingParams()] * len(handles), [0] * len(handles)).cpu().tolist()
+
+    # --- continuous batching ------------------------------------------------------------------------------
+    def submit(self, request: Request) -> None:
+        self.scheduler.submit(request)
+
+    def step(self) -> bool:
+        return self.scheduler.step()
+
+    def stats(self) -> dict:
+        return self.scheduler.stats()
+
+    def generate(self, prompts, max_new_tokens: int = 64, temperature: float = 0.0, top_p: float = 1.0,
+                 seed: int = 0, eos_token_id: int | None = None) -> list[list[int]]:
+        """Continues every prompt (a list of token ids) through the scheduler; returns the new
+        tokens of each. A prompt too long for the model is cut from the left so that the new
+        tokens fit, as the reference's script does (scripts/complete.py:92-110)."""
+        limit = self.model.max_positions()
+        outputs: list[list[int]] = [[] for _ in prompts]
+        errors: list[str | None] = [None] * len(prompts)
+        for i, prompt in enumerate(prompts):
+            tokens = [int(t) for t in prompt]
+            if limit is not None and len(tokens) > max(1, limit - max_new_tokens):
+                tokens = tokens[-max(1, limit - max_new_tokens):]
+
+            def emit(token, finish, i=i):
+                outputs[i].append(token)
+
+            def fail(message, i=i):
+                errors[i] = message
+
+            self.submit(Request(tokens, max_new_tokens, eos_token_id, emit, fail,
+                                SamplingParams(temperature=temperature, top_p=top_p, seed=seed + i)))
+        self.scheduler.run_until_idle()
+        failed = [f"prompt {i}: {e}" for i, e in enumerate(errors) if e is not None]
+        if failed:
+            raise RuntimeError("generation failed: " + "; ".join(failed))
+        return outputs

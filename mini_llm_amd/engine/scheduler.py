@@ -1,0 +1,361 @@
+"""Continuous batching over the step function.
+
+The reference's scheduler (pytorch/src/mini_llm/scheduler.py) admits a waiting request when a
+cache is free, prefills its whole prompt in a call of its own, and decodes all running requests
+in one batched step. This one keeps its queues, its finish reasons and their order, its error
+scopes and its statistics, and differs where the engine below differs: prompts are cut into
+portions under a token budget and run in the same step as the decodes, the currency of
+admission is pages, and a decision is made for the case that pages run out.
+
+Every iteration (`step`):
+1. cancelled requests leave;
+2. plan: running requests past their prompt bring one token each; what is left of the token
+   budget goes to prompts, first those already running, then newly admitted ones in arrival
+   order (no request overtakes the head of the queue; a request is admitted when the pages for
+   its whole prompt are free, though it is fed in portions);
+3. when pages run out for a running request, the request admitted last is preempted: it gives
+   everything back and returns to the FRONT of the queue with its prompt extended by what it has
+   generated, to be recomputed when there is room. A request that does not fit an empty pool
+   fails;
+4. one step of the engine; each request whose prompt is complete gets one new token, sampled
+   on the device; `emit(token, finish)`; a finished request leaves at once and frees its pages.
+"""
+
+from __future__ import annotations
+
+import collections
+import logging
+import threading
+from dataclasses import dataclass, field
+from typing import Callable, Literal, Protocol
+
+from ..cache import OutOfPages
+from ..sampling import SamplingParams
+from .batch import StepEntry
+
+logger = logging.getLogger(__name__)
+
+FinishReason = Literal["stop", "length", "context"]
+
+
+class StepExecutor(Protocol):
+    """What the scheduler needs from the engine below it."""
+
+    page_size: int
+
+    def max_positions(self) -> int | None: ...
+    def check_prompt(self, tokens: list[int]) -> None: ...          # raises if it can never run
+    def can_open(self) -> bool: ...
+    def open(self, request_id) -> None: ...
+    def close(self, request_id) -> None: ...
+    def length(self, request_id) -> int: ...
+    def fits(self, wanted: list) -> bool: ...                        # [(request_id, n_new)] all at once
+    def run(self, entries: list, sampling: list, steps: list) -> list[int]: ...
+
+
+@dataclass
+class Request:
+    """The reference's Request (scheduler.py:41-53) plus how to sample."""
+
+    tokens: list
+    max_new_tokens: int | None
+    eos_token_id: int | None
+    # emit(token, finish): finish is None for every token but the last one.
+    emit: Callable[[int, FinishReason | None], None]
+    fail: Callable[[str], None]
+    sampling: SamplingParams = field(default_factory=SamplingParams)
+    cancelled: bool = field(default=False, init=False)
+
+    def cancel(self) -> None:
+        self.cancelled = True
+
+
+@dataclass
+class _Running:
+    request: Request
+    request_id: int
+    pending: list              # tokens not yet fed: the rest of the prompt, or the last sampled token
+    history: list = field(default_factory=list)   # tokens fed since it was (re)admitted: what its pages hold
+    generated: int = 0
+    prompt_len: int = 0        # of the original prompt (a preempted request's recompute does not count)
+    order: int = 0             # admission order; the largest is preempted first
+    finished: bool = False
+
+
+class Scheduler:
+    def __init__(self, executor: StepExecutor, max_batch: int = 16, max_tokens_per_step: int = 2048,
+                 max_prefills_per_step: int | None = None):
+        if max_batch < 1 or max_tokens_per_step < 1:
+            raise ValueError("max_batch and max_tokens_per_step must be at least 1")
+        if max_prefills_per_step is not None and max_prefills_per_step < 1:
+            raise ValueError("max_prefills_per_step must be at least 1")
+        self._executor = executor
+        self._max_batch, self._budget, self._max_prefills = max_batch, max_tokens_per_step, max_prefills_per_step
+        self._waiting: collections.deque = collections.deque()   # Request, or _Running that was preempted
+        self._running: list[_Running] = []
+        self._wake = threading.Condition()
+        self._stopping = False
+        self._thread: threading.Thread | None = None
+        self._next_id = 0
+        self._order = 0
+        self._steps = self._decode_steps = self._tokens = self._prefills = 0
+        self._batch_sizes = self._step_tokens = self._preemptions = 0
+
+    # --- called from other threads -------------------------------------------------------------
+    def submit(self, request: Request) -> None:
+        with self._wake:
+            self._waiting.append(request)
+            self._wake.notify()
+
+    def stats(self) -> dict:
+        steps = self._decode_steps
+        return {
+            "decode_steps": steps,
+            "tokens": self._tokens,
+            "prefills": self._prefills,
+            "mean_batch_size": self._batch_sizes / steps if steps else 0.0,
+            "running": len(self._running),
+            "waiting": len(self._waiting),
+            "steps": self._steps,
+            "tokens_per_step": self._step_tokens / self._steps if self._steps else 0.0,
+            "preemptions": self._preemptions,
+        }
+
+    def start(self) -> None:
+        self._thread = threading.Thread(target=self._loop, name="scheduler", daemon=True)
+        self._thread.start()
+
+    def stop(self) -> None:
+        with self._wake:
+            self._stopping = True
+            self._wake.notify()
+        if self._thread is not None:
+            self._thread.join()
+        self._fail_everything("the engine is shutting down")
+
+    def is_running(self) -> bool:
+        return self._thread is not None and self._thread.is_alive()
+
+    def has_work(self) -> bool:
+        with self._wake:
+            return bool(self._running) or bool(self._waiting)
+
+    def run_until_idle(self) -> None:
+        while self.step():
+            pass
+
+    # --- the scheduler thread ------------------------------------------------------------------
+    def _loop(self) -> None:
+        while True:
+            with self._wake:
+                while not self._stopping and not self._running and not self._waiting:
+                    self._wake.wait()
+                if self._stopping:
+                    return
+            self.step()
+
+    def step(self) -> bool:
+        """One iteration. Returns False if there was nothing to do."""
+        try:
+            self._drop_cancelled()
+            entries, owners = self._plan()
+            if entries:
+                self._run(entries, owners)
+        except Exception as error:  # the engine is shared: every running request is affected
+            logger.exception("engine error")
+            self._fail_running(str(error))
+            return True
+        return bool(entries) or self.has_work()
+
+    # --- planning ------------------------------------------------------------------------------
+    def _drop_cancelled(self) -> None:
+        for running in [r for r in self._running if r.request.cancelled]:
+            self._executor.close(running.request_id)
+            self._running.remove(running)
+
+    def _portion_that_fits(self, running: _Running, wanted_so_far: list, most: int) -> int:
+        """The largest portion <= most whose pages can be had beside what is planned already."""
+        n = most
+        while n >= 1 and not self._executor.fits(wanted_so_far + [(running.request_id, n)]):
+            # shrink to the end of the page before the last one the portion touches
+            length = self._executor.length(running.request_id)
+            page = self._executor.page_size
+            n = min(n - 1, ((length + n - 1) // page) * page - length)
+        return max(n, 0)
+
+    def _preempt(self, victim: _Running) -> None:
+        """The victim gives everything back and waits at the front of the queue; what it has been
+        fed so far becomes prompt again, so that it is recomputed and goes on where it was."""
+        self._executor.close(victim.request_id)
+        self._running.remove(victim)
+        victim.pending = victim.history + victim.pending
+        victim.history = []
+        self._preemptions += 1
+        with self._wake:
+            self._waiting.appendleft(victim)
+
+    def _plan(self):
+        entries, owners, wanted = [], [], []
+        budget = self._budget
+        preempted = False
+        # Running requests first, in admission order: decodes bring one token, prompts a portion.
+        # Requests are planned oldest first and preempted youngest first, so a victim never has
+        # an entry in the plan yet.
+        for running in sorted(self._running, key=lambda r: r.order):
+            if running not in self._running:
+                continue  # preempted while an older request was planned
+            if budget < 1:
+                break
+            most = min(len(running.pending), budget)
+            n = self._portion_that_fits(running, wanted, most)
+            while n == 0:
+                victim = max(self._running, key=lambda r: r.order)
+                preempted = True
+                if victim is running:
+                    if len(self._running) == 1:
+                        # alone, with every other page free, and still no room
+                        self._executor.close(running.request_id)
+                        self._running.remove(running)
+                        running.request.fail("the request needs more cache pages than the pool has")
+                    else:
+                        self._preempt(running)
+                    break
+                self._preempt(victim)
+                n = self._portion_that_fits(running, wanted, most)
+            if n == 0:
+                continue
+            self._add_entry(entries, owners, wanted, running, n)
+            budget -= n
+        # Then admissions, in arrival order; the head of the queue is never overtaken. None in a
+        # step that had to preempt: the preempted request would come straight back.
+        admitted = 0
+        while not preempted and budget >= 1 and len(self._running) < self._max_batch:
+            if self._max_prefills is not None and admitted >= self._max_prefills:
+                break
+            item = self._pop_waiting()
+            if item is None:
+                break
+            running = self._admit(item, wanted, budget)
+            if running is None:
+                continue          # cancelled or failed: the next one gets its turn
+            if running is False:
+                self._push_front(item)
+                break             # no room yet: wait for a running request to end
+            n = self._portion_that_fits(running, wanted, min(len(running.pending), budget))
+            self._add_entry(entries, owners, wanted, running, n)
+            budget -= n
+            admitted += 1
+        return entries, owners
+
+    def _add_entry(self, entries, owners, wanted, running, n) -> None:
+        completes = n == len(running.pending)
+        entries.append(StepEntry(running.request_id, list(running.pending[:n]), [n - 1] if completes else []))
+        owners.append(running)
+        wanted.append((running.request_id, n))
+
+    def _admit(self, item, wanted, budget):
+        """None: the request is gone (cancelled / failed). False: no room now. Else the _Running."""
+        request = item.request if isinstance(item, _Running) else item
+        if request.cancelled:
+            return None
+        if isinstance(item, _Running):
+            running = item
+        else:
+            try:
+                if not request.tokens:
+                    raise ValueError("the prompt has no tokens")
+                self._executor.check_prompt(list(request.tokens))
+            except Exception as error:  # a bad prompt is the problem of this request only
+                logger.warning("request refused: %s", error)
+                request.fail(str(error))
+                return None
+            running = _Running(request, -1, list(request.tokens), prompt_len=len(request.tokens))
+        if not self._executor.can_open():
+            return False
+        request_id = self._next_id
+        self._executor.open(request_id)
+        # Admitted only if its whole prompt has room beside what is planned: a request that could
+        # take a first portion and then stall would only be preempted again.
+        if not self._executor.fits(wanted + [(request_id, len(running.pending))]):
+            self._executor.close(request_id)
+            if not self._running and not wanted:
+                request.fail("the request needs more cache pages than the pool has")
+                return None
+            return False
+        self._next_id += 1
+        running.request_id = request_id
+        running.order = self._order
+        self._order += 1
+        self._running.append(running)
+        return running
+
+    def _pop_waiting(self):
+        with self._wake:
+            return self._waiting.popleft() if self._waiting else None
+
+    def _push_front(self, item) -> None:
+        with self._wake:
+            self._waiting.appendleft(item)
+
+    # --- running and delivering ----------------------------------------------------------------
+    def _run(self, entries, owners) -> None:
+        sampled_owners = [o for o, e in zip(owners, entries) if e.want]
+        sampling = [o.request.sampling for o in sampled_owners]
+        steps = [o.generated for o in sampled_owners]
+        tokens = self._executor.run(entries, sampling, steps)
+        self._steps += 1
+        self._step_tokens += sum(len(e.tokens) for e in entries)
+        decodes = sum(1 for o, e in zip(owners, entries) if o.generated > 0 and len(e.tokens) == 1)
+        if decodes:
+            self._decode_steps += 1
+            self._batch_sizes += decodes
+        for owner, entry in zip(owners, entries):
+            owner.history.extend(entry.tokens)
+            del owner.pending[: len(entry.tokens)]
+        for owner, token in zip(sampled_owners, tokens):
+            if owner.generated == 0:
+                self._prefills += 1
+            owner.generated += 1
+            owner.pending = [int(token)]
+            self._deliver(owner, int(token))
+        self._running = [r for r in self._running if not r.finished]
+
+    def _finish_reason(self, running: _Running, token: int) -> FinishReason | None:
+        # the order of the reference's checks (scheduler.py:185-196)
+        request = running.request
+        if request.eos_token_id is not None and token == request.eos_token_id:
+            return "stop"
+        limit = self._executor.max_positions()
+        if limit is not None and running.prompt_len + running.generated >= limit:
+            return "context"
+        if request.max_new_tokens is not None and running.generated >= request.max_new_tokens:
+            return "length"
+        return None
+
+    def _deliver(self, running: _Running, token: int) -> None:
+        """Hands one token to its request. If that ends the request, its pages are given back."""
+        reason = self._finish_reason(running, token)
+        self._tokens += 1
+        try:
+            running.request.emit(token, reason)
+        except Exception:
+            # The consumer is gone. That is the problem of this request only.
+            logger.exception("emit failed, dropping the request")
+            reason = "stop"
+        if reason is not None:
+            self._executor.close(running.request_id)
+            running.finished = True
+
+    def _fail_running(self, message: str) -> None:
+        running, self._running = self._running, []
+        for item in running:
+            try:
+                self._executor.close(item.request_id)
+            except Exception:
+                logger.exception("closing a request after an engine error failed")
+            item.request.fail(message)
+
+    def _fail_everything(self, message: str) -> None:
+        self._fail_running(message)
+        while (item := self._pop_waiting()) is not None:
+            (item.request if isinstance(item, _Running) else item).fail(message)
