@@ -1,0 +1,200 @@
+"""Decode and prefill throughput of the engine on one MI355X, GPT-2 small with random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--batch 8]
+
+A step is one decode step: every live sequence gets one new token (greedy, sampled on the
+device and fed back). Sequences start from 512-token uniform-random prompts and decode towards
+1,024 tokens; when they are full they are given back and prefilled again outside the timed
+region, so that exactly K steps are timed. Prints one JSON line. The reference's counterpart is
+engine/bench/bench_batch.c (batched decode at a context) and engine/bench/bench.c."""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+sys.path.insert(0, str(Path(__file__).resolve().parent))
+
+# MI355X's published peaks
+HBM_GBS = 8000.0
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+SMALL = {"architectures": ["GPT2LMHeadModel"], "n_layer": 12, "n_embd": 768, "n_head": 12, "n_inner": 3072,
+         "vocab_size": 50257, "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+PROMPT_LEN, CONTEXT, SEED = 512, 1024, 5
+
+
+def element_size(dtype: str) -> int:
+    return 2 if dtype == "bfloat16" else 4
+
+
+def matrix_elements(c) -> int:
+    per_layer = c.n_embd * 3 * c.n_embd + c.n_embd * c.n_embd + 2 * c.n_embd * c.n_inner
+    return c.n_layer * per_layer
+
+
+def decode_bytes(c, dtype: str, context_lens) -> float:
+    """What a decode step has to read: every weight it uses once, and the live requests' cache."""
+    e = element_size(dtype)
+    weights = (matrix_elements(c) + c.vocab_size * c.n_embd) * e          # matrices and the tied head
+    vectors = c.n_layer * (9 * c.n_embd + c.n_inner) * 4 + 2 * c.n_embd * 4   # biases and norms, 32-bit
+    cache = sum(context_lens) * 2 * c.n_embd * c.n_layer * e
+    return float(weights + vectors + cache)
+
+
+def prefill_flops(c, lengths, wanted_rows: int) -> float:
+    tokens = sum(lengths)
+    linear = 2.0 * tokens * matrix_elements(c)
+    attention = sum(2.0 * 2.0 * (n * (n + 1) / 2) * c.n_embd * c.n_layer for n in lengths)  # QK^T and PV, causal
+    head = 2.0 * wanted_rows * c.vocab_size * c.n_embd
+    return linear + attention + head
+
+
+class DecodeBench:
+    def __init__(self, engine, batch: int):
+        import numpy as np
+
+        self.engine, self.batch = engine, batch
+        rng = np.random.default_rng(SEED + 1)
+        self.prompts = [rng.integers(0, engine.config.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
+        self.handles, self.last, self.length = [], [], 0
+
+    def start(self):
+        """Takes the sequences and prefills their prompts (a few at a time, untimed)."""
+        from mini_llm_amd.engine import StepEntry
+        from mini_llm_amd.sampling import SamplingParams
+
+        self.stop()
+        self.handles = [self.engine.try_take_cache() for _ in range(self.batch)]
+        self.last = []
+        for i in range(0, self.batch, 4):
+            entries = [StepEntry(h, p, [PROMPT_LEN - 1]) for h, p in zip(self.handles[i : i + 4], self.prompts[i : i + 4])]
+            logits = self.engine.runner.step(entries)
+            self.last += self.engine.sampler.sample(logits, [SamplingParams()] * len(entries), [0] * len(entries)).cpu().tolist()
+        self.length = PROMPT_LEN
+
+    def stop(self):
+        for handle in self.handles:
+            self.engine.release_cache(handle)
+        self.handles = []
+
+    def run(self, steps: int, warmup: int):
+        """(seconds, bytes a step had to read on average) over exactly ``steps`` timed steps."""
+        import torch
+
+        self.start()
+        for _ in range(warmup):
+            if self.length >= CONTEXT:
+                self.start()
+            self.last = self.engine.decode_batch(self.handles, self.last)
+            self.length += 1
+        seconds, bytes_read, done = 0.0, 0.0, 0
+        config, dtype = self.engine.config, self.engine.options.dtype
+        while done < steps:
+            if self.length >= CONTEXT:
+                self.start()
+            n = min(steps - done, CONTEXT - self.length)
+            torch.cuda.synchronize()
+            begin = time.perf_counter()
+            for _ in range(n):
+                self.last = self.engine.decode_batch(self.handles, self.last)
+            torch.cuda.synchronize()
+            seconds += time.perf_counter() - begin
+            for k in range(n):
+                bytes_read += decode_bytes(config, dtype, [self.length + k + 1] * self.batch)
+            self.length += n
+            done += n
+        self.stop()
+        return seconds, bytes_read / steps
+
+
+def measure_prefill(engine, runs: int = 5):
+    import numpy as np
+    import torch
+
+    from mini_llm_amd.engine import StepEntry
+
+    rng = np.random.default_rng(SEED + 2)
+    lengths = [CONTEXT, CONTEXT]
+    prompts = [rng.integers(0, engine.config.vocab_size, n).tolist() for n in lengths]
+    times = []
+    for _ in range(runs + 2):
+        handles = [engine.try_take_cache() for _ in prompts]
+        entries = [StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)]
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        engine.runner.step(entries)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - begin)
+        for h in handles:
+            engine.release_cache(h)
+    seconds = float(np.median(times[2:]))
+    tokens = sum(lengths)
+    flops = prefill_flops(engine.config, lengths, len(prompts))
+    return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(seconds * 1e3, 3),
+            "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=256)
+    parser.add_argument("--warmup", type=int, default=16)
+    parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})")
+        return 2
+
+    from mini_llm_amd.config import config_from_dict
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    layers = args.layers or SMALL["n_layer"]
+    config = config_from_dict(dict(SMALL, n_layer=layers))
+    largest = max(args.batch, 1 if args.no_points else 64)
+    engine = Engine.from_random(config, SEED, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
+
+    seconds, step_bytes = DecodeBench(engine, args.batch).run(args.steps, args.warmup)
+    ms_per_step = seconds / args.steps * 1e3
+    achieved = step_bytes / (seconds / args.steps) / 1e9
+    record = {
+        "metric": f"decode tokens/s at batch {args.batch}, GPT-2 small, 512-token prompts decoding towards 1024",
+        "value": round(args.batch * args.steps / seconds, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded random weights, uniform-random token ids",
+        "config": {
+            "model": "gpt2-small", "n_layer": SMALL["n_layer"], "layers_run": layers, "n_embd": config.n_embd,
+            "n_head": config.n_head, "n_inner": config.n_inner, "vocab_size": config.vocab_size,
+            "n_positions": config.n_positions, "activation_function": config.activation_function,
+            "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "page_size": engine.cache.page_size,
+            "kv_cache_dtype": args.dtype, "sampling": "greedy", "parallelism": "single-gpu", "seed": SEED,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
+    }
+    if not args.no_points:
+        record["prefill"] = measure_prefill(engine)
+        points = {}
+        for batch, steps in ((1, 128), (64, 64)):
+            s, _ = DecodeBench(engine, batch).run(steps, 8)
+            points[f"decode_b{batch}"] = round(batch * steps / s, 1)
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,240 @@
+"""Generation through the entry point, the step function's checks, cache reuse, long decoding,
+the first tokens of a sequence: the engine against the plain implementation."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gpt2
+from conftest import random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def engines(model_dirs):
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    cache = {}
+
+    def get(name, dtype="float32", **options):
+        key = (name, dtype, tuple(sorted(options.items())))
+        if key not in cache:
+            cache[key] = Engine(model_dirs[name][0], EngineOptions(dtype=dtype, **options))
+        return cache[key]
+
+    return get
+
+
+def plain_check_greedy(config, weights, prompt, generated, margin):
+    """Every generated token must be (within margin) the plain implementation's argmax."""
+    tokens = list(prompt)
+    for token in generated:
+        logits = plain_gpt2.forward(config, weights, tokens)[-1]
+        assert logits[token] >= logits.max() - margin, f"token {token} at length {len(tokens)}: {logits[token]} < {logits.max()}"
+        tokens.append(token)
+
+
+def test_greedy_generation_matches_plain_f32(model_dirs, engines):
+    # three requests with prompts of 5, 17 and 33 ids, 16 greedy tokens each
+    _, config, weights = model_dirs["A"]
+    prompts = [random_tokens(1 + i, n, config["vocab_size"]) for i, n in enumerate((5, 17, 33))]
+    out = engines("A").generate(prompts, max_new_tokens=16)
+    for prompt, generated in zip(prompts, out):
+        assert generated == plain_gpt2.greedy(config, weights, prompt, 16)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_bf16(model_dirs, engines, name):
+    _, config, weights = model_dirs[name]
+    rounded = {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
+    prompts = [random_tokens(1 + i, n, config["vocab_size"]) for i, n in enumerate((5, 17, 33))]
+    out = engines(name, "bfloat16").generate(prompts, max_new_tokens=16)
+    for prompt, generated in zip(prompts, out):
+        assert len(generated) == 16
+        plain_check_greedy(config, rounded, prompt, generated, margin=0.05)
+
+
+def host_uniform(seed, step, index):
+    """The sampler's counter-based generator, on the host (mini_llm_amd/csrc/sampling.hip)."""
+    m = (1 << 64) - 1
+    z = (seed + 0x9E3779B97F4A7C15 * (step + 1) + 0xD1B54A32D192ED03 * (index + 1)) & m
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+    z = z ^ (z >> 31)
+    return ((z >> 40) + 0.5) / 16777216.0
+
+
+def test_temperature_sampling_in_chunks_beside_decodes(model_dirs, engines):
+    # prompts of 1, 9 and 40 ids prefilled in 8-token portions beside ongoing decodes, 20 new
+    # tokens each at temperature 0.8; every draw is checked against the generator on the host
+    _, config, weights = model_dirs["B"]
+    vocab = config["vocab_size"]
+    prompts = [random_tokens(3 + i, n, vocab) for i, n in enumerate((1, 9, 40))]
+    engine = engines("B", "float32", max_tokens_per_step=8)
+    out = engine.generate(prompts, max_new_tokens=20, temperature=0.8, seed=4)
+    assert engine.stats()["tokens_per_step"] <= 8
+    assert out != engines("B").generate(prompts, max_new_tokens=20)  # it really samples
+    for i, (prompt, generated) in enumerate(zip(prompts, out)):
+        assert len(generated) == 20
+        tokens = list(prompt)
+        for step, token in enumerate(generated):
+            logits = plain_gpt2.forward(config, weights, tokens)[-1]
+            noise = np.array([-math.log(-math.log(host_uniform(4 + i, step, v))) for v in range(vocab)])
+            score = (logits - logits.max()) / 0.8 + noise
+            assert score[token] >= score.max() - 1e-3, f"request {i} step {step}: token {token} is not the draw"
+            tokens.append(token)
+    # the same seeds give the same tokens in another batch composition
+    alone = engines("B").generate([prompts[2]], max_new_tokens=20, temperature=0.8, seed=6)
+    assert alone[0] == out[2]
+
+
+def test_top_p_generation_stays_in_the_nucleus(model_dirs, engines):
+    _, config, weights = model_dirs["A"]
+    prompt = random_tokens(9, 12, config["vocab_size"])
+    (generated,) = engines("A").generate([prompt], max_new_tokens=12, temperature=1.5, top_p=0.3, seed=11)
+    tokens = list(prompt)
+    for token in generated:
+        p = plain_gpt2.softmax(plain_gpt2.forward(config, weights, tokens)[-1] / 1.5)
+        # kept if the mass of strictly more likely tokens is below top_p (a little slack for rounding)
+        assert p[p > p[token] * (1 + 1e-4)].sum() < 0.3 + 1e-4
+        tokens.append(token)
+
+
+def test_eos_and_context_limits(model_dirs, engines):
+    _, config, weights = model_dirs["B"]
+    prompt = random_tokens(5, 10, config["vocab_size"])
+    free = plain_gpt2.greedy(config, weights, prompt, 6)
+    (out,) = engines("B").generate([prompt], max_new_tokens=6, eos_token_id=free[3])
+    assert out == free[: free.index(free[3]) + 1]
+    # 60 + 4 = n_positions: generation stops at the context's end; a longer prompt is cut from the left
+    long_prompt = random_tokens(6, 60, config["vocab_size"])
+    (out,) = engines("B").generate([long_prompt], max_new_tokens=50)
+    assert len(out) == 50 and len(long_prompt[-14:]) + 50 == 64
+    (out,) = engines("B").generate([long_prompt[:60]], max_new_tokens=4)
+    assert out == plain_gpt2.greedy(config, weights, long_prompt[:60], 4)
+
+
+def test_sessions_and_forward_last(model_dirs, engines):
+    _, config, weights = model_dirs["A"]
+    engine = engines("A")
+    tokens = random_tokens(7, 30, config["vocab_size"])
+    ref = plain_gpt2.forward(config, weights, tokens)
+    np.testing.assert_allclose(engine.forward_last(tokens), ref[-1], atol=2e-5, rtol=1e-4)
+    with engine.open_session() as session:
+        np.testing.assert_allclose(session.prefill(tokens[:1]), ref[0], atol=2e-5, rtol=1e-4)   # the very first token
+        np.testing.assert_allclose(session.decode(tokens[1]), ref[1], atol=2e-5, rtol=1e-4)
+        np.testing.assert_allclose(session.prefill(tokens[2:20]), ref[19], atol=2e-5, rtol=1e-4)
+        for i in range(20, 30):
+            np.testing.assert_allclose(session.decode(tokens[i]), ref[i], atol=2e-5, rtol=1e-4)
+        assert session.length() == 30
+    with pytest.raises(RuntimeError, match="closed"):
+        session.decode(1)
+
+
+def test_the_reference_schedulers_four_calls(model_dirs, engines):
+    # try_take_cache / prefill_greedy / decode_batch / release_cache (pytorch/src/mini_llm/batch_api.py)
+    _, config, weights = model_dirs["A"]
+    engine = engines("A", "float32", max_sessions=3)
+    prompts = [random_tokens(20 + i, n, config["vocab_size"]) for i, n in enumerate((3, 11, 26))]
+    handles = [engine.try_take_cache() for _ in prompts]
+    assert engine.try_take_cache() is None  # all taken: None, no waiting
+    last = [engine.prefill_greedy(h, p) for h, p in zip(handles, prompts)]
+    got = [[t] for t in last]
+    for _ in range(7):
+        last = engine.decode_batch(handles, last)
+        for g, t in zip(got, last):
+            g.append(t)
+    for h in handles:
+        engine.release_cache(h)
+    assert got == [plain_gpt2.greedy(config, weights, p, 8) for p in prompts]
+    assert engine.try_take_cache() is not None
+
+
+def test_step_checks_everything_before_it_changes_anything(model_dirs, engines):
+    from mini_llm_amd.cache import OutOfPages
+    from mini_llm_amd.engine import StepEntry, StepError
+
+    engine = engines("B", "float32", max_sessions=4, max_tokens=64)  # one page
+    a, b = engine.try_take_cache(), engine.try_take_cache()
+    engine.runner.step([StepEntry(a, [1, 2, 3], [2])])
+    free = engine.cache.free_pages()
+    bad = [
+        [StepEntry(a, [4], [0]), StepEntry(b, [1000], [0])],      # a token outside the vocabulary
+        [StepEntry(a, [4], [0]), StepEntry(a, [5], [0])],         # a request twice
+        [StepEntry(a, [4], [0]), StepEntry("nobody", [5], [0])],  # an unknown request
+        [StepEntry(a, [4] * 62, [0])],                            # 3 + 62 > n_positions
+        [StepEntry(a, [], [])],                                   # no tokens
+        [StepEntry(a, [4, 5], [2])],                              # a wanted place that is not there
+        [],
+    ]
+    for entries in bad:
+        with pytest.raises(StepError):
+            engine.runner.step(entries)
+        assert engine.cache.length(a) == 3 and engine.cache.length(b) == 0 and engine.cache.free_pages() == free
+    # a holds the only page: a's next token fits on it, b's does not, and neither is taken
+    with pytest.raises(OutOfPages):
+        engine.runner.step([StepEntry(a, [4], [0]), StepEntry(b, [5] * 5, [0])])
+    assert engine.cache.length(a) == 3 and engine.cache.free_pages() == free
+    engine.cache.check_invariants()
+    engine.release_cache(a); engine.release_cache(b)
+
+
+def test_used_pages_give_the_same_bits_as_fresh_ones(model_dirs, engines):
+    # the reference's reset test: a cache used by a longer sequence gives bit-equal results
+    # (engine/tests/test_gpt2_gpu.c:266-289)
+    _, config, _ = model_dirs["A"]
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    tokens = random_tokens(30, 70, config["vocab_size"])
+    fresh = Engine(model_dirs["A"][0], EngineOptions(dtype="float32", max_sessions=2, max_tokens=128))
+    first = fresh.forward_last(tokens)
+    other = fresh.forward_last(random_tokens(31, 128, config["vocab_size"]))  # fills every page with something else
+    again = fresh.forward_last(tokens)
+    assert (first == again).all() and not (first == other).all()
+
+
+def test_long_decoding_and_page_edges(model_dirs, tmp_path):
+    # 40 tokens at once, then 540 one by one across nine page edges, against the whole sequence
+    import replay
+
+    folder, config, weights = model_dirs["C"]
+    requests = {"long": random_tokens(40, 580, config["vocab_size"])}
+    collector = replay.prefill_then_decode(requests, tail=540)
+    for dtype, tol in (("float32", dict(atol=2e-5, rtol=1e-4)), ("bfloat16", dict(atol=4e-2, rtol=4e-2))):
+        got = collector.gather(replay.run_trace(folder, dtype, collector.steps, tmp_path / dtype, 640))
+        w = weights if dtype == "float32" else {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
+        replay.compare(got, replay.plain_logits(config, w, requests), **tol)
+
+
+@pytest.mark.parametrize("page_size", [16, 32, 128])
+def test_other_page_sizes(model_dirs, tmp_path, page_size):
+    import replay
+
+    folder, config, weights = model_dirs["A"]
+    requests = {f"r{i}": random_tokens(50 + i, n, config["vocab_size"]) for i, n in enumerate((33, 128, 17, 65))}
+    collector = replay.mixed(requests, seed=page_size)
+    max_tokens = replay.peak_tokens(collector, page=max(64, page_size))
+    got = collector.gather(replay.run_trace(folder, "float32", collector.steps, tmp_path / "o", max_tokens, page_size=page_size))
+    replay.compare(got, replay.plain_logits(config, weights, requests), atol=2e-5, rtol=1e-4)
+
+
+def test_trace_run_refuses_bad_folders(tmp_path, model_dirs):
+    import json
+    import subprocess
+    import sys
+
+    import replay
+
+    folder, config, weights = model_dirs["A"]
+    broken = tmp_path / "broken"
+    broken.mkdir()
+    (broken / "config.json").write_text(json.dumps(config))
+    w = dict(weights)
+    del w["h.0.ln_1.bias"]
+    plain_gpt2.write_safetensors(broken / "model.safetensors", w)
+    cmd = [sys.executable, str(replay.ROOT / "bin" / "trace_run"), "--model", str(broken), "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "64"]
+    done = subprocess.run(cmd, input="", capture_output=True, text=True, timeout=300)
+    assert done.returncode != 0 and "missing (1): h.0.ln_1.bias" in done.stderr
