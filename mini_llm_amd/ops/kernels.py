@@ -153,11 +153,18 @@ def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
     check(library().mllm_cache_write(_ptr(k_src), _ptr(v_src), k_src.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(slots), n, n_kv_heads, head_size, page_size, _code(k_pages.dtype), _stream()))
 
 
-def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, out=None):
+DECODE_MAX_Q_LEN = 8        # portions up to this many tokens take the split-key kernel
+DECODE_TARGET_WAVES = 2048  # enough waves to fill 256 compute units several times over
+DECODE_MIN_SPLIT = 64       # keys
+
+
+def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, out=None):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
-    row of block_tables that holds the request's pages (negative: padding row, output zero)."""
+    row of block_tables that holds the request's pages (negative: padding row, output zero).
+    ``max_q_len`` (the longest portion in the batch) picks the kernel; ``max_len`` (the longest
+    sequence after this step) only balances the split of the keys over waves."""
     _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     page_size = k_pages.shape[2]
     width = n_heads * head_size
@@ -172,7 +179,23 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         out = torch.empty((n, width), dtype=q.dtype, device=q.device)
     _device_tensor(out, "out", q.dtype, 2)
     _require(tuple(out.shape) == (n, width), "out has the wrong shape")
-    check(library().mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
+    lib = library()
+    if n == 0:
+        return out
+    rows_aligned = q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0  # 16-byte loads of q
+    if (max_q_len is not None and max_q_len <= DECODE_MAX_Q_LEN and rows_aligned
+            and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))):
+        # decoding and short portions: the keys of each (token, head) are split over waves
+        reach = block_tables.shape[1] * page_size if max_len is None else max(1, min(max_len, block_tables.shape[1] * page_size))
+        n_splits = max(1, min(DECODE_TARGET_WAVES // (n * n_heads), -(-reach // DECODE_MIN_SPLIT)))
+        keys_per_split = -(-reach // n_splits)
+        keys_per_split = -(-keys_per_split // DECODE_MIN_SPLIT) * DECODE_MIN_SPLIT
+        n_splits = -(-reach // keys_per_split)
+        floats = lib.mllm_attention_decode_scratch(n, n_heads, head_size, n_splits)
+        scratch = torch.empty((floats,), dtype=torch.float32, device=q.device)
+        check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(scratch), floats, _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), keys_per_split, n_splits, _code(q.dtype), _stream()))
+        return out
+    check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
     return out
 
 

@@ -21,6 +21,8 @@ _SIGNATURES = {
     "mllm_gemm": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_longlong, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
+    "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P],
 }
 
@@ -48,6 +50,8 @@ def library() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = c_int
+        lib.mllm_attention_decode_scratch.argtypes = [c_int, c_int, c_int, c_int]
+        lib.mllm_attention_decode_scratch.restype = c_longlong
         lib.mllm_last_error.restype = ctypes.c_char_p
         lib.mllm_last_error.argtypes = []
         lib.path = path

@@ -48,7 +48,7 @@ class CausalSelfAttention(Mixer):
         mixed = kernels.paged_attention(
             q, ctx.k_pages, ctx.v_pages, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
             self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
-            max_q_len=ctx.batch.max_q_len,
+            max_q_len=ctx.batch.max_q_len, max_len=ctx.batch.max_total_len,
         )
         return self.out.forward(mixed, residual=residual)
 

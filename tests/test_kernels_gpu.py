@@ -140,13 +140,19 @@ def plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window):
     return out[total - nq :]
 
 
+@pytest.mark.parametrize("path", ["general", "split_keys", "split_keys_balanced"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize(
     "n_heads,n_kv_heads,head_size,page_size,window",
     [(4, 4, 16, 16, 0), (3, 3, 32, 64, 0), (5, 5, 48, 32, 0), (6, 2, 64, 16, 0), (2, 1, 80, 64, 0),
-     (2, 2, 128, 64, 0), (4, 2, 32, 16, 37), (1, 1, 256, 16, 0)],
+     (2, 2, 128, 64, 0), (4, 2, 32, 16, 37), (1, 1, 256, 16, 0), (12, 12, 64, 64, 0), (2, 2, 64, 128, 100)],
 )
-def test_paged_attention(K, dtype, n_heads, n_kv_heads, head_size, page_size, window):
+def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_size, window):
+    # general: a wave per (token, head). split_keys: the decode kernel (forced for every row by
+    # promising short portions; it treats rows independently, so the promise costs only speed),
+    # with the splits laid over the tables' whole reach or balanced over the longest sequence.
+    if path != "general" and head_size not in (16, 32, 64, 128, 256):
+        pytest.skip("the split-key kernel takes power-of-two head sizes; others go the general way")
     rng = np.random.default_rng(n_heads * 100 + head_size)
     # three requests: (cached context, new tokens); pages handed out in a scrambled order
     shapes = [(0, 70), (150, 1), (61, 9)]
@@ -185,6 +191,7 @@ def test_paged_attention(K, dtype, n_heads, n_kv_heads, head_size, page_size, wi
     out = K.paged_attention(
         dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
         n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window,
+        max_q_len=None if path == "general" else 1, max_len=151 if path == "split_keys_balanced" else None,
     )
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
