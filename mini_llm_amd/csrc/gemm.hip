@@ -179,13 +179,128 @@ __global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, cons
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Few rows (decoding, short portions): M <= 64. The product is bound by reading W once, so the
+// work is cut along N and K, not M: a block owns 16 output columns, its waves take turns along
+// K, and W streams straight from memory into MFMA operands (a lane loads 16 bytes of one of the
+// 16 rows; the x rows of the same k come through the cache). out^T = W . x^T, so that W is the
+// 16-row operand. The waves' partial sums meet in LDS, where the epilogue runs.
+// ------------------------------------------------------------------------------------------------
+template <typename T, typename OutT, int MT, int KSPLIT>
+__global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
+    const T* __restrict__ A, const T* __restrict__ W, const float* __restrict__ bias,
+    const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue) {
+    constexpr int VEC = Tile<T>::VEC;
+    constexpr int KSTEP = 4 * VEC;  // k covered by one load of the wave: 4 lane groups x 16 bytes
+    constexpr int UNROLL = 4;
+    __shared__ float sums[KSPLIT][MT * 4][WAVE];
+
+    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+    const int row16 = lane % 16, quad = lane / 16;
+    const int n0 = blockIdx.x * 16;
+    const int n = n0 + row16;
+    const bool n_valid = n < N;
+    const T* w_row = W + (size_t)(n_valid ? n : 0) * K;
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const T* x_row[MT];
+    bool x_valid[MT];
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+        int t = i * 16 + row16;
+        x_valid[i] = t < M;
+        x_row[i] = A + (size_t)(x_valid[i] ? t : 0) * K;
+    }
+
+    // wave w takes k-steps w, w + KSPLIT, ... in groups of UNROLL
+    const int n_steps = (K + KSTEP - 1) / KSTEP;
+    for (int step0 = wave * UNROLL; step0 < n_steps; step0 += KSPLIT * UNROLL) {
+        Vec16 w_piece[UNROLL], x_piece[UNROLL][MT];
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            int k = (step0 + u) * KSTEP + quad * VEC;
+            bool k_valid = k < K;  // K is a multiple of VEC: a piece is whole or absent
+            w_piece[u] = Vec16{{0u, 0u, 0u, 0u}};
+            if (k_valid && n_valid) w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + k);
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                x_piece[u][i] = Vec16{{0u, 0u, 0u, 0u}};
+                if (k_valid && x_valid[i]) x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + k);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            if constexpr (sizeof(T) == 2) {
+                bf16x8 a = *reinterpret_cast<bf16x8*>(&w_piece[u]);
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, *reinterpret_cast<bf16x8*>(&x_piece[u][i]), acc[i], 0, 0, 0);
+            } else {
+                f32x4 a = *reinterpret_cast<f32x4*>(&w_piece[u]);
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+#pragma unroll
+                    for (int i = 0; i < MT; i++)
+                        acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], (*reinterpret_cast<f32x4*>(&x_piece[u][i]))[c], acc[i], 0, 0, 0);
+            }
+        }
+    }
+
+    // acc[i][r] is out[token i*16 + lane%16][column n0 + 4*(lane/16) + r]
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) sums[wave][i * 4 + r][lane] = acc[i][r];
+    __syncthreads();
+    for (int index = threadIdx.x; index < MT * 4 * WAVE; index += WAVE * KSPLIT) {
+        int l = index % WAVE, ir = index / WAVE;
+        int token = (ir / 4) * 16 + l % 16;
+        int col = n0 + 4 * (l / 16) + ir % 4;
+        if (token >= M || col >= N) continue;
+        float value = 0.0f;
+#pragma unroll
+        for (int w = 0; w < KSPLIT; w++) value += sums[w][ir][l];  // the same order for every element
+        if (bias) value += bias[col];
+        if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
+        else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+        size_t at = (size_t)token * N + col;
+        if (residual) value = residual[at] + value;
+        out[at] = from_float<OutT>(value);
+    }
+}
+
+template <typename T, typename OutT, int MT>
+void launch_skinny(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M,
+                   int N, int K, int epilogue, hipStream_t stream) {
+    constexpr int KSTEP = 4 * Tile<T>::VEC;
+    int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
+    int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
+    while (split < 8 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
+    dim3 grid(tiles);
+    if (split == 1)
+        gemm_skinny_kernel<T, OutT, MT, 1><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    else if (split == 2)
+        gemm_skinny_kernel<T, OutT, MT, 2><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    else if (split == 4)
+        gemm_skinny_kernel<T, OutT, MT, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    else
+        gemm_skinny_kernel<T, OutT, MT, 8><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+}
+
 template <typename T, typename OutT>
 void launch_gemm(const void* A, const void* W, const float* bias, const float* residual, void* out,
                  int M, int N, int K, int epilogue, hipStream_t stream) {
     const T* a = (const T*)A;
     const T* w = (const T*)W;
     OutT* o = (OutT*)out;
-    if (M <= 32) {
+    if (M <= 64 && K % Tile<T>::VEC == 0) {
+        if (M <= 16) launch_skinny<T, OutT, 1>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+        else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+        else launch_skinny<T, OutT, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+    } else if (M <= 32) {
         dim3 grid(ceil_div(N, 128), ceil_div(M, 32));
         gemm_kernel<T, OutT, 32, 128, 1, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
     } else if (M <= 64 || (long long)ceil_div(M, 128) * ceil_div(N, 128) < 128) {
