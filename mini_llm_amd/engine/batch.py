@@ -66,8 +66,9 @@ class BatchStaging:
         self._device = [torch.empty(self._capacity, dtype=torch.int32, device=self.device) for _ in range(self.ring)]
         self._events = [None] * self.ring
 
-    def upload(self, flat: np.ndarray):
-        """flat: int32 numpy array -> device tensor holding it (valid until ``ring`` later uploads)."""
+    def upload(self, flat: np.ndarray, into=None):
+        """flat: int32 numpy array -> device tensor holding it (valid until ``ring`` later
+        uploads), or copied into the device tensor ``into`` if one is given."""
         import torch
 
         n = int(flat.shape[0])
@@ -78,20 +79,34 @@ class BatchStaging:
         if self._events[i] is not None:
             self._events[i].synchronize()
         self._host[i][:n].numpy()[:] = flat
-        self._device[i][:n].copy_(self._host[i][:n], non_blocking=True)
+        target = self._device[i][:n] if into is None else into[:n]
+        target.copy_(self._host[i][:n], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
         self._events[i] = event
-        return self._device[i][:n]
+        return target
 
 
 def _aligned(n: int) -> int:
     return (n + 3) & ~3  # sections start on 16-byte boundaries
 
 
-def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int) -> StepBatch:
+def _pad(array: np.ndarray, length: int, fill: int) -> np.ndarray:
+    if len(array) >= length:
+        return array
+    out = np.full(length, fill, dtype=np.int32)
+    out[: len(array)] = array
+    return out
+
+
+def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int, capacity: int | None = None,
+                     device_buffer=None) -> StepBatch:
     """Lays out the batch on the host and uploads it in one copy. The entries have been checked
-    and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests)."""
+    and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests).
+
+    ``capacity`` pads the batch to that many tokens and requests with rows that do nothing (token
+    -1, request -1, slot -1), so that the layout depends on the capacity alone; ``device_buffer``
+    then is the fixed device buffer the batch is copied into (a captured graph reads it)."""
     n_requests = len(entries)
     q_lens = [len(e.tokens) for e in entries]
     n_tokens = sum(q_lens)
@@ -99,18 +114,23 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     n_groups = len(cache.groups)
     max_total = max(c + q for c, q in zip(contexts, q_lens))
     table_width = cache.max_blocks() or max(1, -(-max_total // cache.page_size))
+    cap_tokens = n_tokens if capacity is None else capacity
+    cap_requests = n_requests if capacity is None else capacity
+    if n_tokens > cap_tokens or n_requests > cap_requests:
+        raise ValueError("the batch exceeds the capacity it is laid out for")
 
     tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
     positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(contexts, q_lens)])
     token_request = np.repeat(np.arange(n_requests, dtype=np.int32), q_lens)
-    q_starts = np.zeros(n_requests + 1, dtype=np.int32)
-    q_starts[1:] = np.cumsum(q_lens)
+    q_starts = np.full(cap_requests + 1, n_tokens, dtype=np.int32)
+    q_starts[0] = 0
+    q_starts[1 : n_requests + 1] = np.cumsum(q_lens)
     logit_rows = np.asarray([q_starts[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
     state_slots = np.asarray([cache.requests[e.request_id].state_slot for e in entries], dtype=np.int32)
     tables, slots = [], []
     for gi in range(n_groups):
-        table = np.full((n_requests, table_width), -1, dtype=np.int32)
-        slot = np.empty(n_tokens, dtype=np.int32)
+        table = np.full((cap_requests, table_width), -1, dtype=np.int32)
+        slot = np.full(cap_tokens, -1, dtype=np.int32)
         for i, e in enumerate(entries):
             pages = np.asarray(cache.block_table(e.request_id, gi), dtype=np.int32)
             table[i, : len(pages)] = pages
@@ -118,16 +138,20 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
             slot[q_starts[i] : q_starts[i + 1]] = pages[pos // cache.page_size] * cache.page_size + pos % cache.page_size
         tables.append(table)
         slots.append(slot)
+    n_logit_rows = len(logit_rows)
+    if capacity is not None:
+        logit_rows = _pad(logit_rows, cap_tokens, 0)
 
-    sections = [tokens, positions, token_request, q_starts, np.asarray(contexts, dtype=np.int32), state_slots, logit_rows]
+    sections = [_pad(tokens, cap_tokens, -1), _pad(positions, cap_tokens, 0), _pad(token_request, cap_tokens, -1), q_starts,
+                _pad(np.asarray(contexts, dtype=np.int32), cap_requests, 0), _pad(state_slots, cap_requests, 0), logit_rows]
     for table, slot in zip(tables, slots):
         sections += [table.reshape(-1), slot]
     offsets, total = [], 0
     for section in sections:
         offsets.append(total)
         total += _aligned(len(section))
-    host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts,
-            "context_lens": sections[4], "state_slots": state_slots, "logit_rows": logit_rows,
+    host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts[: n_requests + 1],
+            "context_lens": sections[4][:n_requests], "state_slots": state_slots, "logit_rows": logit_rows[:n_logit_rows],
             "block_tables": tables, "slots": slots}
     if staging is None:
         views = sections
@@ -135,14 +159,24 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         flat = np.zeros(max(total, 4), dtype=np.int32)
         for offset, section in zip(offsets, sections):
             flat[offset : offset + len(section)] = section
-        device = staging.upload(flat)
+        device = staging.upload(flat, into=device_buffer)
         views = [device[o : o + len(s)] for o, s in zip(offsets, sections)]
     groups = [
-        GroupStepData(block_tables=views[7 + 2 * gi].reshape(n_requests, table_width), slots=views[8 + 2 * gi])
+        GroupStepData(block_tables=views[7 + 2 * gi].reshape(cap_requests, table_width), slots=views[8 + 2 * gi])
         for gi in range(n_groups)
     ]
     return StepBatch(
-        n_tokens=n_tokens, n_requests=n_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens), max_total_len=max_total,
+        n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
+        max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], groups=groups, request_ids=[e.request_id for e in entries], host=host,
     )
+
+
+def padded_size(cache, capacity: int) -> int:
+    """int32 elements of a batch laid out for ``capacity`` tokens and requests."""
+    table_width = cache.max_blocks()
+    lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 3
+    for _ in cache.groups:
+        lengths += [capacity * table_width, capacity]
+    return sum(_aligned(n) for n in lengths)

@@ -30,6 +30,7 @@ class EngineOptions:
     max_tokens: int | None = None        # cache capacity in tokens; None: max_sessions full contexts
     page_size: int = DEFAULT_PAGE_SIZE
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
+    use_graphs: bool = True              # replay decode steps from captured HIP graphs
     device: str = "cuda:0"
 
 
@@ -124,7 +125,7 @@ class Engine:
         max_tokens = options.max_tokens or options.max_sessions * limit
         self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
                                 max_requests=options.max_sessions, device=options.device)
-        self.runner = ModelRunner(self.model, self.cache, options.device)
+        self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs)
         self.sampler = Sampler(self.runner.staging)
         self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step)
         self._next_handle = 0

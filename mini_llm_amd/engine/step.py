@@ -5,24 +5,67 @@ batched decode: engine/include/gpt2_gpu.h:64-68,89-90,161-165). Here there is on
 prompts beside single decoded tokens, cut anywhere, run as one batch from the cache, with logits
 returned only at the wanted places. Like the reference's calls it checks everything before it
 changes anything (engine/src/gpt2_gpu_batch.cu:67-88), and a request's stored length grows only
-after the step has been launched (engine/src/gpt2_gpu.cu:364)."""
+after the step has been launched (engine/src/gpt2_gpu.cu:364).
+
+A step in which every request brings one token and wants its logits (a decode step) is
+launch-bound, as the reference found (docs/kernels/007_fewer_launches.md): it is captured once
+per batch-size bucket in a HIP graph and replayed; the batch's metadata lies in a fixed device
+buffer per bucket that is overwritten before each replay."""
 
 from __future__ import annotations
 
 from ..cache import CacheManager, OutOfPages
-from .batch import BatchStaging, StepBatch, StepEntry, build_step_batch
+from .batch import BatchStaging, StepBatch, StepEntry, build_step_batch, padded_size
+
+GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
 
 class StepError(ValueError):
     """The batch cannot be run; nothing has been changed."""
 
 
+class _DecodeGraph:
+    """One captured decode step for up to ``capacity`` requests."""
+
+    def __init__(self, runner: "ModelRunner", capacity: int):
+        import torch
+
+        self.runner, self.capacity = runner, capacity
+        self.buffer = torch.zeros(padded_size(runner.cache, capacity), dtype=torch.int32, device=runner.device)
+        self.graph = None
+        self.logits = None
+
+    def run(self, entries):
+        import torch
+
+        runner = self.runner
+        batch = build_step_batch(entries, runner.cache, runner.staging, vocab_size=runner.model.vocab_size,
+                                 capacity=self.capacity, device_buffer=self.buffer)
+        if self.graph is None:
+            # once eagerly (on a side stream, as capture needs), then the capture itself
+            side = torch.cuda.Stream(device=runner.device)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                runner.model.forward(batch, runner.cache)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize(runner.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = runner.model.forward(batch, runner.cache)
+            self.graph = graph
+        self.graph.replay()
+        return batch, self.logits[: len(entries)]
+
+
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, device):
+    def __init__(self, model, cache: CacheManager, device, use_graphs: bool = True):
         self.model, self.cache, self.device = model, cache, device
         self.staging = BatchStaging(device) if device is not None else None
         self.steps_run = 0
+        self.graph_steps = 0
         self.last_batch: StepBatch | None = None
+        self.use_graphs = bool(use_graphs and device is not None and cache.max_length is not None and model.all_graph_safe())
+        self._graphs: dict = {}
 
     def validate(self, entries) -> None:
         if not entries:
@@ -50,10 +93,21 @@ class ModelRunner:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
 
+    def _graph_for(self, entries):
+        if not self.use_graphs or len(entries) > GRAPH_BUCKETS[-1]:
+            return None
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return None
+        capacity = next(b for b in GRAPH_BUCKETS if b >= len(entries))
+        if capacity not in self._graphs:
+            self._graphs[capacity] = _DecodeGraph(self, capacity)
+        return self._graphs[capacity]
+
     def step(self, entries: list[StepEntry]):
         """Runs the entries as one batch. Returns float32 logits [wanted places, vocab] on the
-        device (None if nothing is wanted), in the order of the entries and of each ``want``.
-        Raises StepError / OutOfPages before anything has changed."""
+        device (None if nothing is wanted), in the order of the entries and of each ``want``;
+        they are valid until the next step. Raises StepError / OutOfPages before anything has
+        changed."""
         self.validate(entries)
         reserved = []
         try:
@@ -65,8 +119,13 @@ class ModelRunner:
                 self.cache.rollback(request_id)
             raise
         try:
-            batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size)
-            logits = self.model.forward(batch, self.cache)
+            graph = self._graph_for(entries)
+            if graph is not None:
+                batch, logits = graph.run(entries)
+                self.graph_steps += 1
+            else:
+                batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size)
+                logits = self.model.forward(batch, self.cache)
         except Exception:
             for request_id in reserved:
                 self.cache.rollback(request_id)

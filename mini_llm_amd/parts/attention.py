@@ -15,6 +15,8 @@ from .linear import Linear
 
 
 class CausalSelfAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, width: int, n_heads: int, n_kv_heads: int | None = None, head_size: int | None = None,
                  window: int | None = None, out_std: float = 0.02, qkv_name: str = "c_attn.", out_name: str = "c_proj."):
         self.width, self.n_heads = width, n_heads

@@ -14,6 +14,11 @@ from ..weights.spec import TensorSpec
 class Part:
     """A node of the model tree: its own tensors plus named children."""
 
+    # True if ``forward`` only launches kernels whose arguments are device tensors and numbers
+    # fixed by the batch's capacity: then a decode step may be captured in a HIP graph and
+    # replayed. A part that plans on the host from the batch's contents says False.
+    graph_safe = True
+
     def tensor_specs(self) -> dict[str, TensorSpec]:
         """local tensor name -> spec, for this part's own tensors."""
         return {}
@@ -33,6 +38,9 @@ class Part:
         for child_prefix, child in self.children().items():
             out.update(child.named_tensor_specs(prefix + child_prefix))
         return out
+
+    def all_graph_safe(self) -> bool:
+        return self.graph_safe and all(child.all_graph_safe() for child in self.children().values())
 
     def bind_named(self, tensors: dict, prefix: str = "") -> None:
         own = {name: tensors[prefix + name] for name in self.tensor_specs()}
@@ -82,6 +90,8 @@ class Norm(Part):
 
 class Mixer(Part):
     """Mixes information between the positions of a sequence (attention here)."""
+
+    graph_safe = False  # a mixer says so itself
 
     def kv_need(self) -> KVNeed | None:
         return None

@@ -238,3 +238,54 @@ def test_trace_run_refuses_bad_folders(tmp_path, model_dirs):
     cmd = [sys.executable, str(replay.ROOT / "bin" / "trace_run"), "--model", str(broken), "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "64"]
     done = subprocess.run(cmd, input="", capture_output=True, text=True, timeout=300)
     assert done.returncode != 0 and "missing (1): h.0.ln_1.bias" in done.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_match_eager_steps(model_dirs, dtype):
+    # decode steps replayed from a captured graph, with eager steps (prompt portions, other batch
+    # sizes) and synchronisations between the replays; every replay is checked against the same
+    # step run without graphs and against the plain implementation
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    folder, config, weights = model_dirs["C"]
+    vocab = config["vocab_size"]
+    seqs = {name: random_tokens(60 + i, n, vocab) for i, (name, n) in enumerate((("a", 150), ("b", 90), ("c", 131), ("d", 70)))}
+    if dtype == "bfloat16":
+        weights = {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
+    ref = {name: plain_gpt2.forward(config, weights, t) for name, t in seqs.items()}
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=4e-2, rtol=4e-2)
+    results = {}
+    for use_graphs in (True, False):
+        engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=8, max_tokens=1024, use_graphs=use_graphs))
+        handles = {name: engine.try_take_cache() for name in seqs}
+        fed = {name: 0 for name in seqs}
+        got = {name: {} for name in seqs}
+
+        def run(step):
+            entries = [StepEntry(handles[name], seqs[name][fed[name] : fed[name] + n], [n - 1]) for name, n in step]
+            logits = engine.runner.step(entries).cpu().numpy()
+            for row, (name, n) in zip(logits, step):
+                fed[name] += n
+                got[name][fed[name] - 1] = row
+
+        run([("a", 100), ("b", 40)])
+        for i in range(30):
+            run([("a", 1), ("b", 1)])                     # bucket of 2, replayed
+            if i == 5:
+                run([("c", 77)])                          # an eager step in between
+            if i > 5:
+                run([("c", 1)])                           # bucket of 1
+            if i % 7 == 0:
+                torch.cuda.synchronize()
+            if i == 12:
+                run([("d", 50), ("a", 1)])                # mixed: eager
+            if i > 12 and i % 2:
+                run([("a", 1), ("b", 1), ("c", 1)])       # bucket of 4 with a padding row
+        assert (engine.runner.graph_steps > 0) == use_graphs
+        results[use_graphs] = got
+        for name in seqs:
+            for position, row in got[name].items():
+                np.testing.assert_allclose(row, ref[name][position], err_msg=f"{name} {position} graphs={use_graphs}", **tol)
+    for name in seqs:
+        assert results[True][name].keys() == results[False][name].keys()
