@@ -419,3 +419,291 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }
+
+// ------------------------------------------------------------------------------------------------
+// Prompt portions: a block per (request, head, tile of queries), a wave per 32 queries, keys in
+// tiles of 64 through LDS, both products on the matrix cores, softmax statistics carried from
+// tile to tile in 32-bit.
+//
+// The scores are computed transposed, S^T = K . Q^T (keys are the rows): a lane then holds one
+// query's scores for 32 of the 64 keys, so the row maximum and sum need one exchange with the
+// lane 32 further on and nothing else, and the same registers are the B operand of
+// O^T = V^T . P^T with no shuffle. The order of the keys inside an MFMA's k index is free as long
+// as both operands agree; V^T is read from LDS in the order the score registers have.
+// bfloat16: V is transposed on its way into LDS (two keys packed per 32-bit word).
+// float32: the 32-bit MFMA takes single elements, V is read as stored.
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int PF_KEYS = 64;  // keys per tile
+
+template <typename T, int HD_PAD>
+struct PrefillLds {
+    static constexpr bool HALF = sizeof(T) == 2;
+    static constexpr int K_STRIDE = HD_PAD + (HALF ? 8 : 4);            // elements per key row
+    static constexpr int V_STRIDE = HALF ? PF_KEYS + 4 : HD_PAD + 4;    // bf16: [d][key]; f32: [key][d]
+    static constexpr int V_ROWS = HALF ? HD_PAD : PF_KEYS;
+};
+
+template <typename T, int HD_PAD, int NW>
+__global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
+    const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
+    const int* __restrict__ q_starts, const int* __restrict__ context_lens,
+    const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
+    int head_size, int page_size, int window, float scale) {
+    typedef PrefillLds<T, HD_PAD> L;
+    constexpr bool HALF = L::HALF;
+    constexpr int VEC = HALF ? 8 : 4;
+    constexpr int THREADS = 64 * NW;
+    constexpr int QSTEPS = HALF ? HD_PAD / 16 : HD_PAD / 8;   // k-steps of the score product
+    constexpr int DT = HD_PAD / 32;                           // 32-row tiles of the output's head dimension
+    __shared__ __attribute__((aligned(16))) T k_tile[PF_KEYS * L::K_STRIDE];
+    __shared__ __attribute__((aligned(16))) T v_tile[L::V_ROWS * L::V_STRIDE];
+
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int lane32 = lane % 32, half = lane / 32;
+    const int request = blockIdx.z, head = blockIdx.y;
+    const int q_first = q_starts[request];
+    const int q_len = q_starts[request + 1] - q_first;
+    const int tile_q0 = (gridDim.x - 1 - blockIdx.x) * (32 * NW);  // long tiles first
+    if (tile_q0 >= q_len) return;
+    const int context = context_lens[request];
+    const int kv_head = head / (n_heads / n_kv_heads);
+    const int* table = block_tables + (size_t)request * max_blocks;
+
+    // this lane's query
+    const int q_local = tile_q0 + wave * 32 + lane32;
+    const bool q_valid = q_local < q_len;
+    const int q_position = context + q_local;
+    const int wave_first_position = context + tile_q0 + wave * 32;
+    const int wave_last_position = context + min(tile_q0 + wave * 32 + 31, q_len - 1);
+    const bool wave_active = tile_q0 + wave * 32 < q_len;
+
+    // Q^T operand, kept in registers: dims (step, half, element)
+    Vec16 q_reg[QSTEPS];
+    {
+        const T* q_row = q + (size_t)(q_first + (q_valid ? q_local : 0)) * q_stride + head * head_size;
+#pragma unroll
+        for (int s = 0; s < QSTEPS; s++) {
+            int d = s * (2 * VEC) + half * VEC;
+            q_reg[s] = Vec16{{0u, 0u, 0u, 0u}};
+            if (q_valid && d < head_size) q_reg[s] = *reinterpret_cast<const Vec16*>(q_row + d);
+        }
+    }
+
+    f32x16 acc_o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc_o[i][v] = 0.0f;
+    float running_max = -INFINITY, running_sum = 0.0f;
+
+    const int block_last_position = context + min(tile_q0 + 32 * NW, q_len) - 1;
+    const int block_first_key = window > 0 ? max(0, context + tile_q0 - window + 1) : 0;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float score_scale = HALF ? scale * LOG2E : scale;  // bfloat16 runs take 2^x of a prescaled score
+
+    constexpr int PIECES_PER_ROW = HD_PAD / VEC;
+    for (int k0 = (block_first_key / PF_KEYS) * PF_KEYS; k0 <= block_last_position; k0 += PF_KEYS) {
+        __syncthreads();  // the previous tile has been consumed
+        // ---- stage K (as stored) and V (transposed for bfloat16) ----
+        if constexpr (HALF) {
+            constexpr int PAIRS = (PF_KEYS / 2) * PIECES_PER_ROW;  // two keys of the same dims per thread step
+            for (int pair = tid; pair < PAIRS; pair += THREADS) {
+                int c = pair % PIECES_PER_ROW, row = (pair / PIECES_PER_ROW) * 2;
+                Vec16 k_piece[2], v_piece[2];
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    int key = k0 + row + e;
+                    k_piece[e] = Vec16{{0u, 0u, 0u, 0u}};
+                    v_piece[e] = Vec16{{0u, 0u, 0u, 0u}};
+                    if (key >= block_first_key && key <= block_last_position && c * VEC < head_size) {  // pages before a window may be gone
+                        int page = table[key / page_size];
+                        size_t at = (((size_t)page * n_kv_heads + kv_head) * page_size + key % page_size) * head_size + c * VEC;
+                        k_piece[e] = *reinterpret_cast<const Vec16*>(k_pages + at);
+                        v_piece[e] = *reinterpret_cast<const Vec16*>(v_pages + at);
+                    }
+                    *reinterpret_cast<Vec16*>(&k_tile[(row + e) * L::K_STRIDE + c * VEC]) = k_piece[e];
+                }
+                const uint16_t* v0 = reinterpret_cast<const uint16_t*>(&v_piece[0]);
+                const uint16_t* v1 = reinterpret_cast<const uint16_t*>(&v_piece[1]);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) {
+                    uint32_t packed = (uint32_t)v0[i] | ((uint32_t)v1[i] << 16);
+                    *reinterpret_cast<uint32_t*>(&v_tile[(c * VEC + i) * L::V_STRIDE + row]) = packed;
+                }
+            }
+        } else {
+            constexpr int PIECES = PF_KEYS * PIECES_PER_ROW;
+            for (int piece = tid; piece < PIECES; piece += THREADS) {
+                int c = piece % PIECES_PER_ROW, row = piece / PIECES_PER_ROW;
+                int key = k0 + row;
+                Vec16 k_piece = Vec16{{0u, 0u, 0u, 0u}}, v_piece = Vec16{{0u, 0u, 0u, 0u}};
+                if (key >= block_first_key && key <= block_last_position && c * VEC < head_size) {  // pages before a window may be gone
+                    int page = table[key / page_size];
+                    size_t at = (((size_t)page * n_kv_heads + kv_head) * page_size + key % page_size) * head_size + c * VEC;
+                    k_piece = *reinterpret_cast<const Vec16*>(k_pages + at);
+                    v_piece = *reinterpret_cast<const Vec16*>(v_pages + at);
+                }
+                *reinterpret_cast<Vec16*>(&k_tile[row * L::K_STRIDE + c * VEC]) = k_piece;
+                *reinterpret_cast<Vec16*>(&v_tile[row * L::V_STRIDE + c * VEC]) = v_piece;
+            }
+        }
+        __syncthreads();
+        // a wave whose queries all lie before this tile, or whose windows have all passed it, has nothing to add
+        if (!wave_active || k0 > wave_last_position) continue;
+        if (window > 0 && k0 + PF_KEYS - 1 < wave_first_position - window + 1) continue;
+
+        // ---- S^T = K . Q^T : two 32-key tiles ----
+        f32x16 s_acc[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) s_acc[j][v] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < QSTEPS; s++) {
+                const T* k_at = &k_tile[(j * 32 + lane32) * L::K_STRIDE + s * (2 * VEC) + half * VEC];
+                if constexpr (HALF) {
+                    s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(k_at),
+                                                                       *reinterpret_cast<const bf16x8*>(&q_reg[s]), s_acc[j], 0, 0, 0);
+                } else {
+                    f32x4 a = *reinterpret_cast<const f32x4*>(k_at);
+                    f32x4 b = *reinterpret_cast<const f32x4*>(&q_reg[s]);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) s_acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[c], b[c], s_acc[j], 0, 0, 0);
+                }
+            }
+        }
+        // ---- mask, running maximum ----
+        const int first_allowed = window > 0 ? q_position - window + 1 : 0;
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                int key = k0 + j * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                bool allowed = q_valid && key <= q_position && key >= first_allowed;
+                float s = allowed ? s_acc[j][v] * score_scale : -INFINITY;
+                s_acc[j][v] = s;
+                tile_max = fmaxf(tile_max, s);
+            }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
+        float new_max = fmaxf(running_max, tile_max);
+        float safe_max = new_max == -INFINITY ? 0.0f : new_max;  // a query with no key yet
+        float rescale = HALF ? __builtin_amdgcn_exp2f(running_max - safe_max) : expf(running_max - safe_max);
+        running_max = new_max;
+        running_sum *= rescale;
+#pragma unroll
+        for (int i = 0; i < DT; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_o[i][v] *= rescale;
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float p = HALF ? __builtin_amdgcn_exp2f(s_acc[j][v] - safe_max) : expf(s_acc[j][v] - safe_max);
+                s_acc[j][v] = p;
+                running_sum += p;
+            }
+        // ---- O^T += V^T . P^T ----
+        if constexpr (HALF) {
+#pragma unroll
+            for (int slab = 0; slab < 4; slab++) {  // 16 keys each: score registers 8*(slab%2) .. +7 of tile slab/2
+                bf16x8 p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) p[e] = static_cast<bf16_t>(s_acc[slab / 2][8 * (slab % 2) + e]);
+#pragma unroll
+                for (int i = 0; i < DT; i++) {
+                    const T* v_at = &v_tile[(i * 32 + lane32) * L::V_STRIDE + 16 * slab + 4 * half];
+                    bf16x4 lo = *reinterpret_cast<const bf16x4*>(v_at);
+                    bf16x4 hi = *reinterpret_cast<const bf16x4*>(v_at + 8);
+                    bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p, acc_o[i], 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    int key = j * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+#pragma unroll
+                    for (int i = 0; i < DT; i++)
+                        acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(v_tile[key * L::V_STRIDE + i * 32 + lane32], s_acc[j][v], acc_o[i], 0, 0, 0);
+                }
+        }
+    }
+
+    running_sum += __shfl_xor(running_sum, 32, WAVE);
+    if (!q_valid) return;
+    float inverse = 1.0f / running_sum;  // every query sees at least its own key
+    T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * head_size;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            int d = i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+            if (d < head_size) out_row[d] = from_float<T>(acc_o[i][v] * inverse);
+        }
+}
+
+template <typename T, int HD_PAD>
+void launch_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride,
+                    const int* q_starts, const int* context_lens, const int* block_tables, int max_blocks,
+                    int n_requests, int max_q_len, int n_heads, int n_kv_heads, int head_size, int page_size,
+                    int window, float scale, hipStream_t stream) {
+    // 128 queries per block when that still fills the chip, else 64
+    long long blocks4 = (long long)ceil_div(max_q_len, 128) * n_heads * n_requests;
+    if (blocks4 >= 512) {
+        dim3 grid(ceil_div(max_q_len, 128), n_heads, n_requests);
+        attention_prefill_kernel<T, HD_PAD, 4><<<grid, 256, 0, stream>>>(
+            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
+            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_size, window, scale);
+    } else {
+        dim3 grid(ceil_div(max_q_len, 64), n_heads, n_requests);
+        attention_prefill_kernel<T, HD_PAD, 2><<<grid, 128, 0, stream>>>(
+            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
+            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_size, window, scale);
+    }
+}
+
+}  // namespace
+
+// 1 if the matrix-core prefill kernel takes this head size.
+MLLM_API int mllm_attention_prefill_supported(int head_size) {
+    return head_size >= 16 && head_size <= 128 && head_size % 16 == 0 ? 1 : 0;
+}
+
+MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
+                                    int out_stride, const int* q_starts, const int* context_lens,
+                                    const int* block_tables, int max_blocks, int n_requests, int max_q_len,
+                                    int n_heads, int n_kv_heads, int head_size, int page_size, int window,
+                                    float scale, int dtype, hipStream_t stream) {
+    MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
+    MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_prefill: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
+    MLLM_REQUIRE(mllm_attention_prefill_supported(head_size), "attention_prefill: head size %d is not a multiple of 16 in 16..128", head_size);
+    MLLM_REQUIRE(page_size > 0 && window >= 0, "attention_prefill: bad page size or window");
+    MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_prefill: rows are too short for the heads");
+    MLLM_REQUIRE(n_requests <= 65535 && n_heads <= 65535, "attention_prefill: too many requests or heads for one launch");
+    if (n_requests == 0 || max_q_len == 0) return 0;
+    int padded = ceil_div(head_size, 32) * 32;
+#define MLLM_PREFILL_CASE(T, PAD)                                                                                      \
+    launch_prefill<T, PAD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,      \
+                           max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_size, window, scale, stream)
+    if (dtype == MLLM_F32) {
+        if (padded == 32) MLLM_PREFILL_CASE(float, 32);
+        else if (padded == 64) MLLM_PREFILL_CASE(float, 64);
+        else if (padded == 96) MLLM_PREFILL_CASE(float, 96);
+        else MLLM_PREFILL_CASE(float, 128);
+    } else if (dtype == MLLM_BF16) {
+        if (padded == 32) MLLM_PREFILL_CASE(bf16_t, 32);
+        else if (padded == 64) MLLM_PREFILL_CASE(bf16_t, 64);
+        else if (padded == 96) MLLM_PREFILL_CASE(bf16_t, 96);
+        else MLLM_PREFILL_CASE(bf16_t, 128);
+    } else {
+        MLLM_REQUIRE(false, "attention_prefill: unknown dtype %d", dtype);
+    }
+#undef MLLM_PREFILL_CASE
+    return mllm_check_launch("attention_prefill");
+}

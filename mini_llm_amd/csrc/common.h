@@ -27,6 +27,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int WAVE = 64;
 
+// 16 bytes moved as one piece, whatever they hold.
+struct alignas(16) Vec16 {
+    uint32_t w[4];
+};
+
 void mllm_set_error(const char* format, ...);
 int mllm_check_launch(const char* what);
 

@@ -25,10 +25,6 @@ struct Tile<bf16_t> {
     static constexpr int PAD = 8;
 };
 
-struct alignas(16) Vec16 {
-    uint32_t w[4];
-};
-
 // One 16-byte piece of a row, zero where the matrix ends. `aligned` says that every row starts
 // on a 16-byte boundary (K a multiple of VEC), else the piece is gathered element by element.
 template <typename T>

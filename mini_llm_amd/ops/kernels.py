@@ -158,13 +158,16 @@ DECODE_TARGET_WAVES = 2048  # enough waves to fill 256 compute units several tim
 DECODE_MIN_SPLIT = 64       # keys
 
 
-def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, out=None):
+def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
     row of block_tables that holds the request's pages (negative: padding row, output zero).
     ``max_q_len`` (the longest portion in the batch) picks the kernel; ``max_len`` (the longest
-    sequence after this step) only balances the split of the keys over waves."""
+    sequence after this step) only balances the split of the keys over waves. ``q_starts``
+    ([requests + 1], first row of each request's portion; its rows are contiguous) and
+    ``context_lens`` ([requests], keys stored before this step) let long portions take the
+    matrix-core kernel, which walks tiles of one request's queries."""
     _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     page_size = k_pages.shape[2]
     width = n_heads * head_size
@@ -194,6 +197,15 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         floats = lib.mllm_attention_decode_scratch(n, n_heads, head_size, n_splits)
         scratch = torch.empty((floats,), dtype=torch.float32, device=q.device)
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(scratch), floats, _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), keys_per_split, n_splits, _code(q.dtype), _stream()))
+        return out
+    if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
+            and rows_aligned and lib.mllm_attention_prefill_supported(head_size)):
+        _device_tensor(q_starts, "q_starts", torch.int32, 1)
+        _device_tensor(context_lens, "context_lens", torch.int32, 1)
+        n_requests = context_lens.shape[0]
+        _require(q_starts.shape[0] == n_requests + 1, "q_starts must have one entry more than context_lens")
+        _require(block_tables.shape[0] >= n_requests, "fewer block tables than requests")
+        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
         return out
     check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
     return out

@@ -51,6 +51,7 @@ class CausalSelfAttention(Mixer):
             q, ctx.k_pages, ctx.v_pages, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
             self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
             max_q_len=ctx.batch.max_q_len, max_len=ctx.batch.max_total_len,
+            q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens,
         )
         return self.out.forward(mixed, residual=residual)
 

@@ -140,7 +140,7 @@ def plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window):
     return out[total - nq :]
 
 
-@pytest.mark.parametrize("path", ["general", "split_keys", "split_keys_balanced"])
+@pytest.mark.parametrize("path", ["general", "split_keys", "split_keys_balanced", "matrix_cores"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize(
     "n_heads,n_kv_heads,head_size,page_size,window",
@@ -151,8 +151,11 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     # general: a wave per (token, head). split_keys: the decode kernel (forced for every row by
     # promising short portions; it treats rows independently, so the promise costs only speed),
     # with the splits laid over the tables' whole reach or balanced over the longest sequence.
-    if path != "general" and head_size not in (16, 32, 64, 128, 256):
+    # matrix_cores: the prefill kernel, a block per tile of one request's queries.
+    if path.startswith("split") and head_size not in (16, 32, 64, 128, 256):
         pytest.skip("the split-key kernel takes power-of-two head sizes; others go the general way")
+    if path == "matrix_cores" and head_size > 128:
+        pytest.skip("the matrix-core kernel takes head sizes up to 128; larger go the general way")
     rng = np.random.default_rng(n_heads * 100 + head_size)
     # three requests: (cached context, new tokens); pages handed out in a scrambled order
     shapes = [(0, 70), (150, 1), (61, 9)]
@@ -183,15 +186,19 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
         treq += [r] * new
         tpos += list(range(ctx, total))
         refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window or None))
-    # a padding row in the middle
-    q_rows.insert(1, np.zeros((1, n_heads * head_size)))
-    treq.insert(shapes[0][1], -1)
-    tpos.insert(shapes[0][1], 0)
-    refs.insert(1, np.zeros((1, n_heads * head_size)))
+    extra = {}
+    if path == "matrix_cores":
+        starts = np.cumsum([0] + [new for _, new in shapes])
+        extra = dict(q_starts=dev(starts, torch.int32), context_lens=dev([c for c, _ in shapes], torch.int32))
+    else:  # a padding row in the middle
+        q_rows.insert(1, np.zeros((1, n_heads * head_size)))
+        treq.insert(shapes[0][1], -1)
+        tpos.insert(shapes[0][1], 0)
+        refs.insert(1, np.zeros((1, n_heads * head_size)))
     out = K.paged_attention(
         dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
         n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window,
-        max_q_len=None if path == "general" else 1, max_len=151 if path == "split_keys_balanced" else None,
+        max_q_len={"general": None, "matrix_cores": 70}.get(path, 1), max_len=151 if path == "split_keys_balanced" else None, **extra,
     )
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
