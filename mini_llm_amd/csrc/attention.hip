@@ -252,12 +252,12 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
         for (int u = 0; u < UNROLL; u++) {
             int key = base + u * RPI + group;
             valid[u] = key < end;
-            if (valid[u]) {
-                int page = table[key / page_size];
-                size_t row = ((size_t)page * n_kv_heads + kv_head) * page_size + key % page_size;
-                kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
-                vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
-            }
+            // unconditional loads from a clamped key: no branch between them, all in flight together
+            int safe_key = min(key, end - 1);
+            int page = table[safe_key / page_size];
+            size_t row = ((size_t)page * n_kv_heads + kv_head) * page_size + safe_key % page_size;
+            kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
+            vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
         }
         float score[UNROLL];
         float tile_max = -INFINITY;
@@ -421,9 +421,11 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
 }
 
 // ------------------------------------------------------------------------------------------------
-// Prompt portions: a block per (request, head, tile of queries), a wave per 32 queries, keys in
-// tiles of 64 through LDS, both products on the matrix cores, softmax statistics carried from
-// tile to tile in 32-bit.
+// Prompt portions: a block per (request, head, tile of 32*QG queries). A wave owns 32 queries and
+// every KS-th tile of 64 keys: the block stages KS key tiles at a time in LDS, the KS waves of a
+// query group work on them side by side (the chain of dependent softmax updates is KS times
+// shorter than the sequence), and their (max, sum, output) triples are merged at the end. Both
+// products run on the matrix cores, the softmax statistics in 32-bit.
 //
 // The scores are computed transposed, S^T = K . Q^T (keys are the rows): a lane then holds one
 // query's scores for 32 of the 64 keys, so the row maximum and sum need one exchange with the
@@ -435,50 +437,71 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-constexpr int PF_KEYS = 64;  // keys per tile
+constexpr int PF_KEYS = 64;     // keys per tile
+constexpr int PF_TABLE = 1024;  // block table entries a block keeps in LDS (longer tables are read from memory)
 
-template <typename T, int HD_PAD>
+template <typename T, int HD_PAD, int QG, int KS>
 struct PrefillLds {
     static constexpr bool HALF = sizeof(T) == 2;
     static constexpr int K_STRIDE = HD_PAD + (HALF ? 8 : 4);            // elements per key row
     static constexpr int V_STRIDE = HALF ? PF_KEYS + 4 : HD_PAD + 4;    // bf16: [d][key]; f32: [key][d]
     static constexpr int V_ROWS = HALF ? HD_PAD : PF_KEYS;
+    static constexpr int K_ELEMS = PF_KEYS * K_STRIDE, V_ELEMS = V_ROWS * V_STRIDE;
+    static constexpr int TILE_BYTES = KS * (K_ELEMS + V_ELEMS) * (int)sizeof(T);
+    // merge: every wave but the first of its query group leaves 16*DT + 2 floats per lane
+    static constexpr int MERGE_BYTES = QG * (KS - 1) * WAVE * (16 * (HD_PAD / 32) + 2) * 4;
+    static constexpr int BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
+    // bfloat16 V^T: the group of four keys g of row d lies at group g ^ swizzle(d). The rows a wave
+    // writes at once are 8 apart, which without this would all fall on the same banks.
+    static __device__ __forceinline__ int swizzle(int d) { return ((d >> 4) & 3) << 2; }
 };
 
-template <typename T, int HD_PAD, int NW>
-__global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
+template <bool HALF>
+__device__ __forceinline__ float softmax_exp(float x) {
+    if constexpr (HALF) return __builtin_amdgcn_exp2f(x);  // scores are prescaled by log2(e)
+    else return expf(x);
+}
+
+template <typename T, int HD_PAD, int QG, int KS>
+__global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ q_starts, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int head_size, int page_size, int window, float scale) {
-    typedef PrefillLds<T, HD_PAD> L;
+    int head_size, int page_shift, int window, float scale) {
+    typedef PrefillLds<T, HD_PAD, QG, KS> L;
     constexpr bool HALF = L::HALF;
     constexpr int VEC = HALF ? 8 : 4;
-    constexpr int THREADS = 64 * NW;
+    constexpr int THREADS = 64 * QG * KS;
     constexpr int QSTEPS = HALF ? HD_PAD / 16 : HD_PAD / 8;   // k-steps of the score product
     constexpr int DT = HD_PAD / 32;                           // 32-row tiles of the output's head dimension
-    __shared__ __attribute__((aligned(16))) T k_tile[PF_KEYS * L::K_STRIDE];
-    __shared__ __attribute__((aligned(16))) T v_tile[L::V_ROWS * L::V_STRIDE];
+    constexpr int SPAN = KS * PF_KEYS;                        // keys the block covers per iteration
+    __shared__ __attribute__((aligned(16))) unsigned char lds_raw[L::BYTES];
+    __shared__ int table_lds[PF_TABLE];
+    T* const k_tiles = reinterpret_cast<T*>(lds_raw);
+    T* const v_tiles = k_tiles + KS * L::K_ELEMS;
 
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int lane32 = lane % 32, half = lane / 32;
+    const int query_group = wave % QG, key_split = wave / QG;
     const int request = blockIdx.z, head = blockIdx.y;
     const int q_first = q_starts[request];
     const int q_len = q_starts[request + 1] - q_first;
-    const int tile_q0 = (gridDim.x - 1 - blockIdx.x) * (32 * NW);  // long tiles first
+    const int tile_q0 = (gridDim.x - 1 - blockIdx.x) * (32 * QG);  // long tiles first
     if (tile_q0 >= q_len) return;
     const int context = context_lens[request];
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
+    const int page_mask = (1 << page_shift) - 1;
 
     // this lane's query
-    const int q_local = tile_q0 + wave * 32 + lane32;
+    const int q_local = tile_q0 + query_group * 32 + lane32;
     const bool q_valid = q_local < q_len;
     const int q_position = context + q_local;
-    const int wave_first_position = context + tile_q0 + wave * 32;
-    const int wave_last_position = context + min(tile_q0 + wave * 32 + 31, q_len - 1);
-    const bool wave_active = tile_q0 + wave * 32 < q_len;
+    const int wave_first_position = context + tile_q0 + query_group * 32;
+    const int wave_last_position = context + min(tile_q0 + query_group * 32 + 31, q_len - 1);
+    const bool wave_active = tile_q0 + query_group * 32 < q_len;
+    const bool wave_full = tile_q0 + query_group * 32 + 31 < q_len;
 
     // Q^T operand, kept in registers: dims (step, half, element)
     Vec16 q_reg[QSTEPS];
@@ -487,8 +510,8 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
 #pragma unroll
         for (int s = 0; s < QSTEPS; s++) {
             int d = s * (2 * VEC) + half * VEC;
-            q_reg[s] = Vec16{{0u, 0u, 0u, 0u}};
-            if (q_valid && d < head_size) q_reg[s] = *reinterpret_cast<const Vec16*>(q_row + d);
+            q_reg[s] = *reinterpret_cast<const Vec16*>(q_row + min(d, head_size - VEC));
+            if (!(q_valid && d < head_size)) q_reg[s] = Vec16{{0u, 0u, 0u, 0u}};
         }
     }
 
@@ -499,59 +522,85 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
         for (int v = 0; v < 16; v++) acc_o[i][v] = 0.0f;
     float running_max = -INFINITY, running_sum = 0.0f;
 
-    const int block_last_position = context + min(tile_q0 + 32 * NW, q_len) - 1;
+    const int block_last_position = context + min(tile_q0 + 32 * QG, q_len) - 1;
     const int block_first_key = window > 0 ? max(0, context + tile_q0 - window + 1) : 0;
+    // the pages this block walks, copied to LDS once: a tile's loads then do not wait for a lookup in memory
+    const int first_page = block_first_key >> page_shift, last_page = block_last_position >> page_shift;
+    const bool table_in_lds = last_page - first_page < PF_TABLE;
+    if (table_in_lds)
+        for (int i = tid; i <= last_page - first_page; i += THREADS) table_lds[i] = table[first_page + i];
+    __syncthreads();
     constexpr float LOG2E = 1.4426950408889634f;
     const float score_scale = HALF ? scale * LOG2E : scale;  // bfloat16 runs take 2^x of a prescaled score
 
+    // K and V tiles go memory -> registers -> LDS; the loads of the next tiles are issued before the
+    // products of the current ones, so their latency hides behind the matrix cores.
     constexpr int PIECES_PER_ROW = HD_PAD / VEC;
-    for (int k0 = (block_first_key / PF_KEYS) * PF_KEYS; k0 <= block_last_position; k0 += PF_KEYS) {
-        __syncthreads();  // the previous tile has been consumed
-        // ---- stage K (as stored) and V (transposed for bfloat16) ----
-        if constexpr (HALF) {
-            constexpr int PAIRS = (PF_KEYS / 2) * PIECES_PER_ROW;  // two keys of the same dims per thread step
-            for (int pair = tid; pair < PAIRS; pair += THREADS) {
-                int c = pair % PIECES_PER_ROW, row = (pair / PIECES_PER_ROW) * 2;
-                Vec16 k_piece[2], v_piece[2];
+    constexpr int ROWS_PER_UNIT = HALF ? 2 : 1;  // bfloat16 takes two keys per step, to pack V^T words
+    constexpr int UNITS = (SPAN / ROWS_PER_UNIT) * PIECES_PER_ROW;
+    constexpr int UNITS_PER_THREAD = (UNITS + THREADS - 1) / THREADS;
+    Vec16 k_regs[UNITS_PER_THREAD][ROWS_PER_UNIT], v_regs[UNITS_PER_THREAD][ROWS_PER_UNIT];
+    auto fetch = [&](int k_base) {
 #pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    int key = k0 + row + e;
-                    k_piece[e] = Vec16{{0u, 0u, 0u, 0u}};
-                    v_piece[e] = Vec16{{0u, 0u, 0u, 0u}};
-                    if (key >= block_first_key && key <= block_last_position && c * VEC < head_size) {  // pages before a window may be gone
-                        int page = table[key / page_size];
-                        size_t at = (((size_t)page * n_kv_heads + kv_head) * page_size + key % page_size) * head_size + c * VEC;
-                        k_piece[e] = *reinterpret_cast<const Vec16*>(k_pages + at);
-                        v_piece[e] = *reinterpret_cast<const Vec16*>(v_pages + at);
-                    }
-                    *reinterpret_cast<Vec16*>(&k_tile[(row + e) * L::K_STRIDE + c * VEC]) = k_piece[e];
-                }
-                const uint16_t* v0 = reinterpret_cast<const uint16_t*>(&v_piece[0]);
-                const uint16_t* v1 = reinterpret_cast<const uint16_t*>(&v_piece[1]);
+        for (int i = 0; i < UNITS_PER_THREAD; i++) {
+            int unit = min(tid + i * THREADS, UNITS - 1);
+            int c = unit % PIECES_PER_ROW, row = (unit / PIECES_PER_ROW) * ROWS_PER_UNIT;
 #pragma unroll
-                for (int i = 0; i < VEC; i++) {
-                    uint32_t packed = (uint32_t)v0[i] | ((uint32_t)v1[i] << 16);
-                    *reinterpret_cast<uint32_t*>(&v_tile[(c * VEC + i) * L::V_STRIDE + row]) = packed;
+            for (int e = 0; e < ROWS_PER_UNIT; e++) {
+                int key = k_base + row + e;
+                // pages before a window may be gone, keys beyond the last query are not stored yet:
+                // the load goes to a clamped key and column, the result is zeroed afterwards
+                bool valid = key >= block_first_key && key <= block_last_position && c * VEC < head_size;
+                int safe_key = min(max(key, block_first_key), block_last_position);
+                int page = table_in_lds ? table_lds[(safe_key >> page_shift) - first_page] : table[safe_key >> page_shift];
+                size_t at = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask)) * head_size + min(c * VEC, head_size - VEC);
+                k_regs[i][e] = *reinterpret_cast<const Vec16*>(k_pages + at);
+                v_regs[i][e] = *reinterpret_cast<const Vec16*>(v_pages + at);
+                if (!valid) {
+                    k_regs[i][e] = Vec16{{0u, 0u, 0u, 0u}};
+                    v_regs[i][e] = Vec16{{0u, 0u, 0u, 0u}};
                 }
-            }
-        } else {
-            constexpr int PIECES = PF_KEYS * PIECES_PER_ROW;
-            for (int piece = tid; piece < PIECES; piece += THREADS) {
-                int c = piece % PIECES_PER_ROW, row = piece / PIECES_PER_ROW;
-                int key = k0 + row;
-                Vec16 k_piece = Vec16{{0u, 0u, 0u, 0u}}, v_piece = Vec16{{0u, 0u, 0u, 0u}};
-                if (key >= block_first_key && key <= block_last_position && c * VEC < head_size) {  // pages before a window may be gone
-                    int page = table[key / page_size];
-                    size_t at = (((size_t)page * n_kv_heads + kv_head) * page_size + key % page_size) * head_size + c * VEC;
-                    k_piece = *reinterpret_cast<const Vec16*>(k_pages + at);
-                    v_piece = *reinterpret_cast<const Vec16*>(v_pages + at);
-                }
-                *reinterpret_cast<Vec16*>(&k_tile[row * L::K_STRIDE + c * VEC]) = k_piece;
-                *reinterpret_cast<Vec16*>(&v_tile[row * L::V_STRIDE + c * VEC]) = v_piece;
             }
         }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int i = 0; i < UNITS_PER_THREAD; i++) {
+            int unit = tid + i * THREADS;
+            if (unit >= UNITS) continue;
+            int c = unit % PIECES_PER_ROW, row = (unit / PIECES_PER_ROW) * ROWS_PER_UNIT;
+            int tile = row / PF_KEYS, in_tile = row % PF_KEYS;
+            T* k_tile = k_tiles + tile * L::K_ELEMS;
+            T* v_tile = v_tiles + tile * L::V_ELEMS;
+#pragma unroll
+            for (int e = 0; e < ROWS_PER_UNIT; e++)
+                *reinterpret_cast<Vec16*>(&k_tile[(in_tile + e) * L::K_STRIDE + c * VEC]) = k_regs[i][e];
+            if constexpr (HALF) {
+                const uint16_t* v0 = reinterpret_cast<const uint16_t*>(&v_regs[i][0]);
+                const uint16_t* v1 = reinterpret_cast<const uint16_t*>(&v_regs[i][ROWS_PER_UNIT - 1]);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) {
+                    uint32_t packed = (uint32_t)v0[j] | ((uint32_t)v1[j] << 16);
+                    int d = c * VEC + j;
+                    *reinterpret_cast<uint32_t*>(&v_tile[d * L::V_STRIDE + (((in_tile >> 2) ^ L::swizzle(d)) << 2) + (in_tile & 3)]) = packed;
+                }
+            } else {
+                *reinterpret_cast<Vec16*>(&v_tile[in_tile * L::V_STRIDE + c * VEC]) = v_regs[i][0];
+            }
+        }
+    };
+
+    const T* const k_tile = k_tiles + key_split * L::K_ELEMS;
+    const T* const v_tile = v_tiles + key_split * L::V_ELEMS;
+    const int first_base = (block_first_key / PF_KEYS) * PF_KEYS;
+    fetch(first_base);
+    for (int k_base = first_base; k_base <= block_last_position; k_base += SPAN) {
+        __syncthreads();  // the previous tiles have been consumed
+        stage();
         __syncthreads();
-        // a wave whose queries all lie before this tile, or whose windows have all passed it, has nothing to add
+        if (k_base + SPAN <= block_last_position) fetch(k_base + SPAN);
+        const int k0 = k_base + key_split * PF_KEYS;
+        // a wave whose queries all lie before its tile, or whose windows have all passed it, has nothing to add
         if (!wave_active || k0 > wave_last_position) continue;
         if (window > 0 && k0 + PF_KEYS - 1 < wave_first_position - window + 1) continue;
 
@@ -575,23 +624,34 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
                 }
             }
         }
-        // ---- mask, running maximum ----
-        const int first_allowed = window > 0 ? q_position - window + 1 : 0;
+        // ---- scale, mask (only where the tile touches the diagonal, a window or the tile's end), maximum ----
         float tile_max = -INFINITY;
+        const bool interior = wave_full && window == 0 && k0 + PF_KEYS - 1 <= wave_first_position;
+        if (interior) {
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                int key = k0 + j * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-                bool allowed = q_valid && key <= q_position && key >= first_allowed;
-                float s = allowed ? s_acc[j][v] * score_scale : -INFINITY;
-                s_acc[j][v] = s;
-                tile_max = fmaxf(tile_max, s);
-            }
+                for (int v = 0; v < 16; v++) {
+                    s_acc[j][v] *= score_scale;
+                    tile_max = fmaxf(tile_max, s_acc[j][v]);
+                }
+        } else {
+            const int first_allowed = window > 0 ? q_position - window + 1 : 0;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    int key = k0 + j * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                    bool allowed = q_valid && key <= q_position && key >= first_allowed;
+                    float s = allowed ? s_acc[j][v] * score_scale : -INFINITY;
+                    s_acc[j][v] = s;
+                    tile_max = fmaxf(tile_max, s);
+                }
+        }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, WAVE));
         float new_max = fmaxf(running_max, tile_max);
         float safe_max = new_max == -INFINITY ? 0.0f : new_max;  // a query with no key yet
-        float rescale = HALF ? __builtin_amdgcn_exp2f(running_max - safe_max) : expf(running_max - safe_max);
+        float rescale = softmax_exp<HALF>(running_max - safe_max);
         running_max = new_max;
         running_sum *= rescale;
 #pragma unroll
@@ -602,7 +662,7 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                float p = HALF ? __builtin_amdgcn_exp2f(s_acc[j][v] - safe_max) : expf(s_acc[j][v] - safe_max);
+                float p = softmax_exp<HALF>(s_acc[j][v] - safe_max);
                 s_acc[j][v] = p;
                 running_sum += p;
             }
@@ -615,9 +675,10 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
                 for (int e = 0; e < 8; e++) p[e] = static_cast<bf16_t>(s_acc[slab / 2][8 * (slab % 2) + e]);
 #pragma unroll
                 for (int i = 0; i < DT; i++) {
-                    const T* v_at = &v_tile[(i * 32 + lane32) * L::V_STRIDE + 16 * slab + 4 * half];
-                    bf16x4 lo = *reinterpret_cast<const bf16x4*>(v_at);
-                    bf16x4 hi = *reinterpret_cast<const bf16x4*>(v_at + 8);
+                    const int d = i * 32 + lane32, group = 4 * slab + half;
+                    const T* v_row = &v_tile[d * L::V_STRIDE];
+                    bf16x4 lo = *reinterpret_cast<const bf16x4*>(v_row + ((group ^ L::swizzle(d)) << 2));
+                    bf16x4 hi = *reinterpret_cast<const bf16x4*>(v_row + (((group + 2) ^ L::swizzle(d)) << 2));
                     bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p, acc_o[i], 0, 0, 0);
                 }
@@ -636,6 +697,46 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
     }
 
     running_sum += __shfl_xor(running_sum, 32, WAVE);
+
+    // ---- merge the key splits of each query group: the first wave of the group gathers ----
+    if constexpr (KS > 1) {
+        constexpr int PER_LANE = 16 * DT + 2;
+        float* merge = reinterpret_cast<float*>(lds_raw);
+        __syncthreads();  // the tiles are no longer read
+        if (key_split > 0) {
+            float* mine = merge + (((key_split - 1) * QG + query_group) * WAVE + lane) * PER_LANE;
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) mine[i * 16 + v] = acc_o[i][v];
+            mine[16 * DT] = running_max;
+            mine[16 * DT + 1] = running_sum;
+        }
+        __syncthreads();
+        if (key_split > 0) return;
+        float total_max = running_max;
+#pragma unroll
+        for (int s = 1; s < KS; s++)
+            total_max = fmaxf(total_max, merge[(((s - 1) * QG + query_group) * WAVE + lane) * PER_LANE + 16 * DT]);
+        float safe_max = total_max == -INFINITY ? 0.0f : total_max;
+        float weight = softmax_exp<HALF>(running_max - safe_max);
+        running_sum *= weight;
+#pragma unroll
+        for (int i = 0; i < DT; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_o[i][v] *= weight;
+#pragma unroll
+        for (int s = 1; s < KS; s++) {
+            const float* other = merge + (((s - 1) * QG + query_group) * WAVE + lane) * PER_LANE;
+            float w = softmax_exp<HALF>(other[16 * DT] - safe_max);
+            running_sum += other[16 * DT + 1] * w;
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc_o[i][v] += other[i * 16 + v] * w;
+        }
+    }
+
     if (!q_valid) return;
     float inverse = 1.0f / running_sum;  // every query sees at least its own key
     T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * head_size;
@@ -648,31 +749,50 @@ __global__ __launch_bounds__(64 * NW) void attention_prefill_kernel(
         }
 }
 
+int g_prefill_shape = 0;  // 0: chosen by size; set by mllm_attention_prefill_force_shape for tuning runs
+
 template <typename T, int HD_PAD>
 void launch_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride,
                     const int* q_starts, const int* context_lens, const int* block_tables, int max_blocks,
-                    int n_requests, int max_q_len, int n_heads, int n_kv_heads, int head_size, int page_size,
+                    int n_requests, int max_q_len, int n_heads, int n_kv_heads, int head_size, int page_shift,
                     int window, float scale, hipStream_t stream) {
-    // 128 queries per block when that still fills the chip, else 64
-    long long blocks4 = (long long)ceil_div(max_q_len, 128) * n_heads * n_requests;
-    if (blocks4 >= 512) {
-        dim3 grid(ceil_div(max_q_len, 128), n_heads, n_requests);
-        attention_prefill_kernel<T, HD_PAD, 4><<<grid, 256, 0, stream>>>(
-            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
-            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_size, window, scale);
-    } else {
-        dim3 grid(ceil_div(max_q_len, 64), n_heads, n_requests);
-        attention_prefill_kernel<T, HD_PAD, 2><<<grid, 128, 0, stream>>>(
-            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
-            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_size, window, scale);
+    // Queries per block (32*QG) set how often keys and values are read again from the cache;
+    // waves along the keys (KS) set the length of the chain of dependent softmax updates.
+    constexpr bool ROOMY = PrefillLds<T, HD_PAD, 1, 4>::TILE_BYTES <= 80 * 1024;
+    // Measured on MI355X (two 1,024-token prompts, 12 heads of 64): 128 queries per block run 2.5
+    // times faster than 32, because every block reads its keys and values again from the cache.
+    int shape = g_prefill_shape;
+    if (shape == 0) shape = max_q_len > 64 ? 3 : (max_q_len > 32 ? 5 : (ROOMY ? 1 : 4));
+#define MLLM_PREFILL_LAUNCH(QG, KS)                                                                                   \
+    {                                                                                                                  \
+        dim3 grid(ceil_div(max_q_len, 32 * QG), n_heads, n_requests);                                                  \
+        attention_prefill_kernel<T, HD_PAD, QG, KS><<<grid, 64 * QG * KS, 0, stream>>>(                                \
+            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens, \
+            block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_shift, window, scale);                      \
     }
+    if constexpr (ROOMY) {
+        if (shape == 1) MLLM_PREFILL_LAUNCH(1, 4)
+        else if (shape == 2) MLLM_PREFILL_LAUNCH(2, 4)
+        else if (shape == 3) MLLM_PREFILL_LAUNCH(4, 2)
+        else if (shape == 4) MLLM_PREFILL_LAUNCH(1, 2)
+        else MLLM_PREFILL_LAUNCH(2, 2)
+    } else {
+        if (shape == 3) MLLM_PREFILL_LAUNCH(4, 2)
+        else if (shape == 5) MLLM_PREFILL_LAUNCH(2, 2)
+        else MLLM_PREFILL_LAUNCH(1, 2)
+    }
+#undef MLLM_PREFILL_LAUNCH
 }
 
 }  // namespace
 
-// 1 if the matrix-core prefill kernel takes this head size.
-MLLM_API int mllm_attention_prefill_supported(int head_size) {
-    return head_size >= 16 && head_size <= 128 && head_size % 16 == 0 ? 1 : 0;
+// Tuning aid: forces one block shape of the prefill kernel (0 gives the choice back to the sizes).
+MLLM_API void mllm_attention_prefill_force_shape(int shape) { g_prefill_shape = shape; }
+
+// 1 if the matrix-core prefill kernel takes this head size and page size.
+MLLM_API int mllm_attention_prefill_supported(int head_size, int page_size) {
+    bool page_ok = page_size > 0 && (page_size & (page_size - 1)) == 0;
+    return head_size >= 16 && head_size <= 128 && head_size % 16 == 0 && page_ok ? 1 : 0;
 }
 
 MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
@@ -682,15 +802,18 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
                                     float scale, int dtype, hipStream_t stream) {
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_prefill: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
-    MLLM_REQUIRE(mllm_attention_prefill_supported(head_size), "attention_prefill: head size %d is not a multiple of 16 in 16..128", head_size);
-    MLLM_REQUIRE(page_size > 0 && window >= 0, "attention_prefill: bad page size or window");
+    MLLM_REQUIRE(mllm_attention_prefill_supported(head_size, page_size),
+                 "attention_prefill: head size %d is not a multiple of 16 in 16..128, or page size %d is no power of two", head_size, page_size);
+    MLLM_REQUIRE(window >= 0, "attention_prefill: bad window");
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_prefill: rows are too short for the heads");
     MLLM_REQUIRE(n_requests <= 65535 && n_heads <= 65535, "attention_prefill: too many requests or heads for one launch");
     if (n_requests == 0 || max_q_len == 0) return 0;
     int padded = ceil_div(head_size, 32) * 32;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) page_shift++;
 #define MLLM_PREFILL_CASE(T, PAD)                                                                                      \
     launch_prefill<T, PAD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,      \
-                           max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_size, window, scale, stream)
+                           max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_shift, window, scale, stream)
     if (dtype == MLLM_F32) {
         if (padded == 32) MLLM_PREFILL_CASE(float, 32);
         else if (padded == 64) MLLM_PREFILL_CASE(float, 64);

@@ -14,40 +14,49 @@ template <typename T>
 struct Tile;
 template <>
 struct Tile<float> {
-    static constexpr int BK = 16;   // k elements per LDS tile
+    static constexpr int BK = 32;   // k elements per LDS tile
     static constexpr int VEC = 4;   // elements per 16-byte vector
     static constexpr int PAD = 4;
 };
 template <>
 struct Tile<bf16_t> {
-    static constexpr int BK = 32;
+    static constexpr int BK = 64;
     static constexpr int VEC = 8;
     static constexpr int PAD = 8;
 };
 
-// One 16-byte piece of a row, zero where the matrix ends. `aligned` says that every row starts
-// on a 16-byte boundary (K a multiple of VEC), else the piece is gathered element by element.
-template <typename T>
-__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k,
-                                            int K, bool aligned) {
+// One 16-byte piece of a row, zero where the matrix ends. With ALIGNED (K a multiple of VEC, so
+// every row starts on a 16-byte boundary and a piece is whole or absent) the load is
+// unconditional from a clamped address and the result is selected afterwards: no branch stands
+// between the loads of a tile, so they are all in flight together. Otherwise the piece is
+// gathered element by element.
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k, int K) {
     constexpr int VEC = Tile<T>::VEC;
-    Vec16 v = {{0u, 0u, 0u, 0u}};
-    if (row >= n_rows || k >= K) return v;
-    const T* p = base + (size_t)row * K + k;
-    if (aligned && k + VEC <= K) {
-        v = *reinterpret_cast<const Vec16*>(p);
+    if constexpr (ALIGNED) {
+        bool valid = row < n_rows && k < K;
+        int safe_row = min(row, n_rows - 1), safe_k = min(k, K - VEC);
+        Vec16 v = *reinterpret_cast<const Vec16*>(base + (size_t)safe_row * K + safe_k);
+        if (!valid) v = Vec16{{0u, 0u, 0u, 0u}};
+        return v;
     } else {
+        Vec16 v = {{0u, 0u, 0u, 0u}};
+        if (row >= n_rows || k >= K) return v;
+        const T* p = base + (size_t)row * K + k;
         T* e = reinterpret_cast<T*>(&v);
 #pragma unroll
         for (int i = 0; i < VEC; i++)
             if (k + i < K) e[i] = p[i];
+        return v;
     }
-    return v;
 }
 
 // Block tile BM x BN, 4 waves laid out WAVES_M x WAVES_N, each wave TM x TN tiles of 32x32.
-template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, const T* __restrict__ W,
+// Tiles of A and W go memory -> registers -> LDS; the loads run two tiles ahead of the products
+// (two register sets used in turn), so that one block per compute unit still hides the memory
+// latency: these products are small enough that the grid often is no more than that.
+template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                    const float* __restrict__ bias,
                                                    const float* __restrict__ residual,
                                                    OutT* __restrict__ out, int M, int N, int K,
@@ -56,8 +65,9 @@ __global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, cons
     constexpr int LDK = BK + PAD;
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
     constexpr int VPR = BK / VEC;  // 16-byte pieces per tile row
-    constexpr int A_PIECES = (BM * VPR + 255) / 256, W_PIECES = (BN * VPR + 255) / 256;
-    static_assert(WAVES_M * WAVES_N == 4 && TM >= 1 && TN >= 1, "tile layout");
+    constexpr int THREADS = 64 * WAVES_M * WAVES_N;
+    constexpr int A_PIECES = (BM * VPR + THREADS - 1) / THREADS, W_PIECES = (BN * VPR + THREADS - 1) / THREADS;
+    static_assert(TM >= 1 && TN >= 1, "tile layout");
 
     __shared__ __attribute__((aligned(16))) T a_tile[BM * LDK];
     __shared__ __attribute__((aligned(16))) T w_tile[BN * LDK];
@@ -65,7 +75,6 @@ __global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, cons
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const bool aligned = (K % VEC) == 0;
     const int half = lane / 32, lane32 = lane % 32;
 
     f32x16 acc[TM][TN];
@@ -76,39 +85,32 @@ __global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, cons
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    Vec16 a_next[A_PIECES], w_next[W_PIECES];
-    auto fetch = [&](int k0) {
+    Vec16 a_regs[2][A_PIECES], w_regs[2][W_PIECES];
+    auto fetch = [&](int set, int k0) {
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
-            int piece = tid + i * 256;
-            if (piece < BM * VPR) a_next[i] = load_piece<T>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K, aligned);
+            int piece = tid + i * THREADS;
+            if (piece < BM * VPR) a_regs[set][i] = load_piece<T, ALIGNED>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K);
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
-            int piece = tid + i * 256;
-            if (piece < BN * VPR) w_next[i] = load_piece<T>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, aligned);
+            int piece = tid + i * THREADS;
+            if (piece < BN * VPR) w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K);
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](int set) {
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
-            int piece = tid + i * 256;
-            if (piece < BM * VPR) *reinterpret_cast<Vec16*>(&a_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = a_next[i];
+            int piece = tid + i * THREADS;
+            if (piece < BM * VPR) *reinterpret_cast<Vec16*>(&a_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = a_regs[set][i];
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
-            int piece = tid + i * 256;
-            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = w_next[i];
+            int piece = tid + i * THREADS;
+            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = w_regs[set][i];
         }
     };
-
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        __syncthreads();  // the previous tile has been consumed
-        stage();
-        __syncthreads();
-        if (k0 + BK < K) fetch(k0 + BK);
-
+    auto products = [&]() {
         if constexpr (sizeof(T) == 2) {
 #pragma unroll
             for (int kk = 0; kk < BK / 16; kk++) {
@@ -150,6 +152,22 @@ __global__ __launch_bounds__(256) void gemm_kernel(const T* __restrict__ A, cons
                             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][c], b[j][c], acc[i][j], 0, 0, 0);
             }
         }
+    };
+
+    fetch(0, 0);
+    if (BK < K) fetch(1, BK);
+    for (int k0 = 0; k0 < K; k0 += 2 * BK) {
+        __syncthreads();  // the previous tile has been consumed
+        stage(0);
+        __syncthreads();
+        if (k0 + 2 * BK < K) fetch(0, k0 + 2 * BK);
+        products();
+        if (k0 + BK >= K) break;
+        __syncthreads();
+        stage(1);
+        __syncthreads();
+        if (k0 + 3 * BK < K) fetch(1, k0 + 3 * BK);
+        products();
     }
 
     // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
@@ -219,12 +237,13 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         for (int u = 0; u < UNROLL; u++) {
             int k = (step0 + u) * KSTEP + quad * VEC;
             bool k_valid = k < K;  // K is a multiple of VEC: a piece is whole or absent
-            w_piece[u] = Vec16{{0u, 0u, 0u, 0u}};
-            if (k_valid && n_valid) w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + k);
+            int safe_k = min(k, K - VEC);  // loads are unconditional, from a clamped address: no branch between them
+            w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + safe_k);
+            if (!(k_valid && n_valid)) w_piece[u] = Vec16{{0u, 0u, 0u, 0u}};
 #pragma unroll
             for (int i = 0; i < MT; i++) {
-                x_piece[u][i] = Vec16{{0u, 0u, 0u, 0u}};
-                if (k_valid && x_valid[i]) x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + k);
+                x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + safe_k);
+                if (!(k_valid && x_valid[i])) x_piece[u][i] = Vec16{{0u, 0u, 0u, 0u}};
             }
         }
 #pragma unroll
@@ -286,6 +305,36 @@ void launch_skinny(const T* a, const T* w, const float* bias, const float* resid
         gemm_skinny_kernel<T, OutT, MT, 8><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
 }
 
+int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
+
+template <typename T, typename OutT, bool ALIGNED, int BM, int BN, int WAVES_M, int WAVES_N>
+void launch_tile(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M, int N,
+                 int K, int epilogue, hipStream_t stream) {
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
+    gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+}
+
+template <typename T, typename OutT, bool ALIGNED>
+void launch_tiled(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M, int N,
+                  int K, int epilogue, hipStream_t stream) {
+    int tile = g_forced_tile;
+    if (tile == 0) {
+        // measured on MI355X at GPT-2 sizes: many waves per block hide latency best
+        if (M <= 32) tile = 1;
+        else if (M <= 64) tile = 2;
+        else tile = 7;
+    }
+    switch (tile) {
+        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+    }
+}
+
 template <typename T, typename OutT>
 void launch_gemm(const void* A, const void* W, const float* bias, const float* residual, void* out,
                  int M, int N, int K, int epilogue, hipStream_t stream) {
@@ -296,19 +345,17 @@ void launch_gemm(const void* A, const void* W, const float* bias, const float* r
         if (M <= 16) launch_skinny<T, OutT, 1>(a, w, bias, residual, o, M, N, K, epilogue, stream);
         else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream);
         else launch_skinny<T, OutT, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream);
-    } else if (M <= 32) {
-        dim3 grid(ceil_div(N, 128), ceil_div(M, 32));
-        gemm_kernel<T, OutT, 32, 128, 1, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
-    } else if (M <= 64 || (long long)ceil_div(M, 128) * ceil_div(N, 128) < 128) {
-        dim3 grid(ceil_div(N, 64), ceil_div(M, 64));
-        gemm_kernel<T, OutT, 64, 64, 2, 2><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    } else if (K % Tile<T>::VEC == 0) {
+        launch_tiled<T, OutT, true>(a, w, bias, residual, o, M, N, K, epilogue, stream);
     } else {
-        dim3 grid(ceil_div(N, 128), ceil_div(M, 128));
-        gemm_kernel<T, OutT, 128, 128, 2, 2><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+        launch_tiled<T, OutT, false>(a, w, bias, residual, o, M, N, K, epilogue, stream);
     }
 }
 
 }  // namespace
+
+// Tuning aid: forces one tile shape of the tiled kernel (0 gives the choice back to the sizes).
+MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
 MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const float* residual,
                        void* out, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,

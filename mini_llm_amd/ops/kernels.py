@@ -199,7 +199,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(scratch), floats, _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), keys_per_split, n_splits, _code(q.dtype), _stream()))
         return out
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
-            and rows_aligned and lib.mllm_attention_prefill_supported(head_size)):
+            and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _device_tensor(q_starts, "q_starts", torch.int32, 1)
         _device_tensor(context_lens, "context_lens", torch.int32, 1)
         n_requests = context_lens.shape[0]

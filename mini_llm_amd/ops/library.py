@@ -24,7 +24,7 @@ _SIGNATURES = {
     "mllm_attention_decode": [P, c_int, P, P, P, c_longlong, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
-    "mllm_attention_prefill_supported": [c_int],
+    "mllm_attention_prefill_supported": [c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P],
 }
 
