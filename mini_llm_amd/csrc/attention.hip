@@ -164,14 +164,14 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decoding and short portions: a wave per (token, head, split of the keys).
+// Decoding and short portions: a block per (token, head), a wave per share of the keys.
 //
 // The rows of one head inside a page lie together, so a wave reads them as one contiguous
 // stream: each lane loads 16 bytes, LPR = head bytes / 16 lanes share a row, and one load
 // instruction covers 64 / LPR consecutive keys. A lane therefore holds a slice of the head
 // dimensions of several keys; the dot products are finished with shuffles inside the LPR lanes,
-// and the value sums stay per lane until the end. Each split writes (max, sum, unnormalised
-// output) to a scratch buffer; a second kernel merges the splits.
+// and the value sums stay per lane until the end. The waves of a block take equal shares of
+// one token's keys; their (max, sum, unnormalised output) triples are merged in LDS.
 // ------------------------------------------------------------------------------------------------
 namespace {
 
@@ -190,182 +190,140 @@ struct Chunk<bf16_t> {
     static __device__ __forceinline__ float get(const Raw& r, int i) { return static_cast<float>(r[i]); }
 };
 
+constexpr int DECODE_MAX_SPLITS = 16;
+
+// A block per (token, head); its waves (blockDim.x / 64 of them, a power of two up to 16) split
+// the token's keys evenly among themselves, and their partial results meet in LDS.
 template <typename T, int HD>
-__global__ __launch_bounds__(256) void attention_decode_kernel(
+__global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
-    const T* __restrict__ v_pages, float* __restrict__ partial,
+    const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int page_size, int window, float scale, int keys_per_split, int n_splits) {
+    int page_shift, int window, float scale) {
     constexpr int VEC = Chunk<T>::VEC;
     constexpr int LPR = HD / VEC;          // lanes that share a row
     constexpr int RPI = WAVE / LPR;        // rows one load instruction covers
     constexpr int UNROLL = 8;
     constexpr int KPI = RPI * UNROLL;      // keys per iteration
     static_assert(HD % VEC == 0 && (LPR & (LPR - 1)) == 0 && LPR <= WAVE, "head size must be a power of two");
+    __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
 
-    const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-    const int split = blockIdx.x * 4 + wave;
-    const int head = blockIdx.y, token = blockIdx.z;
-    if (split >= n_splits) return;
+    const int lane = threadIdx.x % WAVE, split = threadIdx.x / WAVE, n_splits = blockDim.x / WAVE;
+    const int head = blockIdx.x, token = blockIdx.y;
     const int request = token_request[token];
-    if (request < 0) return;  // a padding row: the merge kernel writes its zeros
-    float* out = partial + (((size_t)token * n_heads + head) * n_splits + split) * (HD + 2);
-
-    const int position = positions[token];
-    const int first_key = window > 0 ? max(0, position - window + 1) : 0;
-    const int begin = max(first_key, split * keys_per_split);
-    // exclusive; the last split takes whatever lies beyond the splits' nominal reach
-    const int end = split == n_splits - 1 ? position + 1 : min(position + 1, (split + 1) * keys_per_split);
-    const int sub = lane % LPR, group = lane / LPR;
-    if (begin >= end) {
-        if (lane < LPR) {
-#pragma unroll
-            for (int i = 0; i < VEC; i++) out[sub * VEC + i] = 0.0f;
-        }
-        if (lane == 0) {
-            out[HD] = -INFINITY;
-            out[HD + 1] = 0.0f;
-        }
+    T* out_row = out + (size_t)token * out_stride + head * HD;
+    if (request < 0) {  // a padding row; the whole block leaves together
+        for (int d = threadIdx.x; d < HD; d += blockDim.x) out_row[d] = from_float<T>(0.0f);
         return;
     }
+    const int position = positions[token];
+    const int first_key = window > 0 ? max(0, position - window + 1) : 0;
+    const int n_keys = position + 1 - first_key;
+    const int chunk = (((n_keys + n_splits - 1) / n_splits + RPI - 1) / RPI) * RPI;  // keys per wave
+    const int begin = first_key + split * chunk;
+    const int end = min(position + 1, begin + chunk);  // exclusive
+    const int sub = lane % LPR, group = lane / LPR;
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
+    const int page_mask = (1 << page_shift) - 1;
 
     typedef typename Chunk<T>::Raw Raw;
-    float qf[VEC];
-    {
-        Raw raw = *reinterpret_cast<const Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
-#pragma unroll
-        for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
-    }
-
     float o[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; i++) o[i] = 0.0f;
     float running_max = -INFINITY, running_sum = 0.0f;  // the sum is this lane's share
 
-    for (int base = begin; base < end; base += KPI) {
-        Raw kf[UNROLL], vf[UNROLL];  // kept as loaded: converted where they are used
-        bool valid[UNROLL];
+    if (begin < end) {
+        float qf[VEC];
+        {
+            Raw raw = *reinterpret_cast<const Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            int key = base + u * RPI + group;
-            valid[u] = key < end;
-            // unconditional loads from a clamped key: no branch between them, all in flight together
-            int safe_key = min(key, end - 1);
-            int page = table[safe_key / page_size];
-            size_t row = ((size_t)page * n_kv_heads + kv_head) * page_size + safe_key % page_size;
-            kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
-            vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
+            for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
         }
-        float score[UNROLL];
-        float tile_max = -INFINITY;
+        for (int base = begin; base < end; base += KPI) {
+            Raw kf[UNROLL], vf[UNROLL];  // kept as loaded: converted where they are used
+            bool valid[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            float dot = 0.0f;
-            if (valid[u]) {
+            for (int u = 0; u < UNROLL; u++) {
+                int key = base + u * RPI + group;
+                valid[u] = key < end;
+                // unconditional loads from a clamped key: no branch between them, all in flight together
+                int safe_key = min(key, end - 1);
+                int page = table[safe_key >> page_shift];
+                size_t row = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask));
+                kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
+                vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
+            }
+            float score[UNROLL];
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                float dot = 0.0f;
 #pragma unroll
                 for (int i = 0; i < VEC; i++) dot += qf[i] * Chunk<T>::get(kf[u], i);
+#pragma unroll
+                for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
+                score[u] = valid[u] ? dot : -INFINITY;
+                tile_max = fmaxf(tile_max, score[u]);
             }
 #pragma unroll
-            for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
-            score[u] = valid[u] ? dot : -INFINITY;
-            tile_max = fmaxf(tile_max, score[u]);
-        }
+            for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
+            float new_max = fmaxf(running_max, tile_max);  // finite: the first key of the tile is valid
+            float rescale = expf(running_max - new_max);
+            running_sum *= rescale;
 #pragma unroll
-        for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
-        float new_max = fmaxf(running_max, tile_max);  // finite: the first key of the tile is valid
-        float rescale = expf(running_max - new_max);
-        running_sum *= rescale;
+            for (int i = 0; i < VEC; i++) o[i] *= rescale;
 #pragma unroll
-        for (int i = 0; i < VEC; i++) o[i] *= rescale;
-#pragma unroll
-        for (int u = 0; u < UNROLL; u++) {
-            if (valid[u]) {
-                float p = expf(score[u] - new_max);
+            for (int u = 0; u < UNROLL; u++) {
+                float p = valid[u] ? expf(score[u] - new_max) : 0.0f;
                 running_sum += p;
 #pragma unroll
                 for (int i = 0; i < VEC; i++) o[i] += p * Chunk<T>::get(vf[u], i);
             }
+            running_max = new_max;
         }
-        running_max = new_max;
-    }
-    // every lane of a row group counted the same keys: merge across the groups only
+        // every lane of a row group counted the same keys: merge across the groups only
 #pragma unroll
-    for (int offset = LPR; offset < WAVE; offset <<= 1) {
-        running_sum += __shfl_xor(running_sum, offset, WAVE);
+        for (int offset = LPR; offset < WAVE; offset <<= 1) {
+            running_sum += __shfl_xor(running_sum, offset, WAVE);
 #pragma unroll
-        for (int i = 0; i < VEC; i++) o[i] += __shfl_xor(o[i], offset, WAVE);
+            for (int i = 0; i < VEC; i++) o[i] += __shfl_xor(o[i], offset, WAVE);
+        }
     }
     if (lane < LPR) {
 #pragma unroll
-        for (int i = 0; i < VEC; i++) out[sub * VEC + i] = o[i];
+        for (int i = 0; i < VEC; i++) partial[split][sub * VEC + i] = o[i];
     }
     if (lane == 0) {
-        out[HD] = running_max;
-        out[HD + 1] = running_sum;
+        partial[split][HD] = running_max;
+        partial[split][HD + 1] = running_sum;
     }
-}
-
-// Merges the splits of each (token, head): out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M).
-template <typename T>
-__global__ __launch_bounds__(256) void attention_merge_kernel(
-    const float* __restrict__ partial, T* __restrict__ out, int out_stride,
-    const int* __restrict__ token_request, int n_tokens, int n_heads, int head_size, int n_splits) {
-    const int lane = threadIdx.x % WAVE;
-    const int pair = blockIdx.x * 4 + threadIdx.x / WAVE;
-    if (pair >= n_tokens * n_heads) return;
-    const int token = pair / n_heads, head = pair % n_heads;
-    T* out_row = out + (size_t)token * out_stride + head * head_size;
-    if (token_request[token] < 0) {
-        for (int d = lane; d < head_size; d += WAVE) out_row[d] = from_float<T>(0.0f);
-        return;
-    }
-    const float* base = partial + (size_t)pair * n_splits * (head_size + 2);
+    __syncthreads();
+    // out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M); a wave without keys has m = -inf, l = 0
     float total_max = -INFINITY;
-    for (int s = 0; s < n_splits; s++) total_max = fmaxf(total_max, base[s * (head_size + 2) + head_size]);
+    for (int s = 0; s < n_splits; s++) total_max = fmaxf(total_max, partial[s][HD]);
     float total = 0.0f;
-    for (int s = 0; s < n_splits; s++) {
-        const float* p = base + s * (head_size + 2);
-        total += p[head_size + 1] * expf(p[head_size] - total_max);
-    }
+    for (int s = 0; s < n_splits; s++) total += partial[s][HD + 1] * expf(partial[s][HD] - total_max);
     float inverse = 1.0f / total;
-    for (int d = lane; d < head_size; d += WAVE) {
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
         float value = 0.0f;
-        for (int s = 0; s < n_splits; s++) {
-            const float* p = base + s * (head_size + 2);
-            value += p[d] * expf(p[head_size] - total_max);
-        }
+        for (int s = 0; s < n_splits; s++) value += partial[s][d] * expf(partial[s][HD] - total_max);
         out_row[d] = from_float<T>(value * inverse);
     }
 }
 
-template <typename T, int HD>
-void launch_decode(const void* q, int q_stride, const void* k_pages, const void* v_pages, float* partial,
-                   void* out, int out_stride, const int* token_request, const int* positions,
-                   const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
-                   int page_size, int window, float scale, int keys_per_split, int n_splits,
-                   hipStream_t stream) {
-    dim3 grid(ceil_div(n_splits, 4), n_heads, n_tokens);
-    attention_decode_kernel<T, HD><<<grid, 256, 0, stream>>>(
-        (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, partial, token_request, positions,
-        block_tables, max_blocks, n_heads, n_kv_heads, page_size, window, scale, keys_per_split, n_splits);
-    attention_merge_kernel<T><<<ceil_div(n_tokens * n_heads, 4), 256, 0, stream>>>(
-        partial, (T*)out, out_stride, token_request, n_tokens, n_heads, HD, n_splits);
-}
-
 template <typename T>
 int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pages, const void* v_pages,
-                    float* partial, void* out, int out_stride, const int* token_request,
-                    const int* positions, const int* block_tables, int max_blocks, int n_tokens,
-                    int n_heads, int n_kv_heads, int page_size, int window, float scale,
-                    int keys_per_split, int n_splits, hipStream_t stream) {
-#define MLLM_DECODE_CASE(HD)                                                                         \
-    case HD:                                                                                         \
-        launch_decode<T, HD>(q, q_stride, k_pages, v_pages, partial, out, out_stride, token_request, \
-                             positions, block_tables, max_blocks, n_tokens, n_heads, n_kv_heads,     \
-                             page_size, window, scale, keys_per_split, n_splits, stream);            \
+                    void* out, int out_stride, const int* token_request, const int* positions,
+                    const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
+                    int page_shift, int window, float scale, int n_splits, hipStream_t stream) {
+    dim3 grid(n_heads, n_tokens), block(WAVE * n_splits);
+#define MLLM_DECODE_CASE(HD)                                                                                   \
+    case HD:                                                                                                   \
+        attention_decode_kernel<T, HD><<<grid, block, 0, stream>>>(                                            \
+            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
+            positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);              \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
@@ -383,39 +341,34 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
 // 1 if the split-key decode kernel takes this head size and page size for this element type.
 MLLM_API int mllm_attention_decode_supported(int head_size, int page_size, int dtype) {
     if (head_size != 16 && head_size != 32 && head_size != 64 && head_size != 128 && head_size != 256) return 0;
-    int vec = dtype == MLLM_F32 ? 4 : 8;
-    int rows_per_load = WAVE / (head_size / vec);
-    return rows_per_load >= 1 && page_size > 0 ? 1 : 0;
-}
-
-// Floats of scratch that mllm_attention_decode needs for this many tokens, heads and splits.
-MLLM_API long long mllm_attention_decode_scratch(int n_tokens, int n_heads, int head_size, int n_splits) {
-    return (long long)n_tokens * n_heads * n_splits * (head_size + 2);
+    if (dtype != MLLM_F32 && dtype != MLLM_BF16) return 0;
+    return page_size > 0 && (page_size & (page_size - 1)) == 0 ? 1 : 0;
 }
 
 MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pages, const void* v_pages,
-                                   float* scratch, long long scratch_floats, void* out, int out_stride,
-                                   const int* token_request, const int* positions, const int* block_tables,
-                                   int max_blocks, int n_tokens, int n_heads, int n_kv_heads, int head_size,
-                                   int page_size, int window, float scale, int keys_per_split, int n_splits,
-                                   int dtype, hipStream_t stream) {
+                                   void* out, int out_stride, const int* token_request, const int* positions,
+                                   const int* block_tables, int max_blocks, int n_tokens, int n_heads,
+                                   int n_kv_heads, int head_size, int page_size, int window, float scale,
+                                   int n_splits, int dtype, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
-                 "attention_decode: head size %d is not one of 16, 32, 64, 128, 256", head_size);
-    MLLM_REQUIRE(window >= 0 && keys_per_split > 0 && n_splits > 0, "attention_decode: bad window or splits");
-    MLLM_REQUIRE(scratch_floats >= mllm_attention_decode_scratch(n_tokens, n_heads, head_size, n_splits),
-                 "attention_decode: the scratch buffer is too small");
+                 "attention_decode: head size %d is not one of 16, 32, 64, 128, 256, or page size %d is no power of two", head_size, page_size);
+    MLLM_REQUIRE(window >= 0, "attention_decode: bad window");
+    MLLM_REQUIRE(n_splits >= 1 && n_splits <= DECODE_MAX_SPLITS && (n_splits & (n_splits - 1)) == 0,
+                 "attention_decode: %d splits is not a power of two in 1..%d", n_splits, DECODE_MAX_SPLITS);
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_decode: rows are too short for the heads");
-    MLLM_REQUIRE(n_tokens <= 65535 && n_heads <= 65535, "attention_decode: too many tokens or heads for one launch");
+    MLLM_REQUIRE(n_tokens <= 65535, "attention_decode: too many tokens for one launch");
     if (n_tokens == 0) return 0;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) page_shift++;
     int refused = 1;
     if (dtype == MLLM_F32)
-        refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, scratch, out, out_stride, token_request, positions,
-                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_size, window, scale, keys_per_split, n_splits, stream);
-    else if (dtype == MLLM_BF16)
-        refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, scratch, out, out_stride, token_request, positions,
-                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_size, window, scale, keys_per_split, n_splits, stream);
+        refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
+                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, stream);
+    else
+        refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
+                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, stream);
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }

@@ -55,12 +55,20 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     const float n = (float)width;  // divided by, not multiplied with its inverse: a constant row has mean exactly itself
 
     if constexpr (ROW_REGS > 0) {
-        float values[ROW_REGS];
+        // the row, the gains and the offsets are all asked for before anything is reduced, so the
+        // kernel waits for memory once
+        float values[ROW_REGS], gains[ROW_REGS], offsets[ROW_REGS];
+#pragma unroll
+        for (int r = 0; r < ROW_REGS; r++) {
+            int i = min(lane + r * WAVE, width - 1);
+            values[r] = in_row[i];
+            gains[r] = gamma[i];
+            offsets[r] = beta[i];
+        }
         float sum = 0.0f;
 #pragma unroll
         for (int r = 0; r < ROW_REGS; r++) {
-            int i = lane + r * WAVE;
-            values[r] = i < width ? in_row[i] : 0.0f;
+            if (lane + r * WAVE >= width) values[r] = 0.0f;
             sum += values[r];
         }
         float mean = wave_sum(sum) / n;
@@ -76,7 +84,7 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
         for (int r = 0; r < ROW_REGS; r++) {
             int i = lane + r * WAVE;
             if (i < width)
-                out_row[i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gamma[i] + beta[i]);
+                out_row[i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gains[r] + offsets[r]);
         }
     } else {
         float sum = 0.0f;
@@ -102,6 +110,8 @@ static void launch_layernorm(const float* x, const int* row_index, const float* 
     OutT* o = (OutT*)out;
     if (width <= 4 * WAVE)
         layernorm_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+    else if (width <= 12 * WAVE)
+        layernorm_kernel<OutT, 12><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
     else if (width <= 16 * WAVE)
         layernorm_kernel<OutT, 16><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
     else if (width <= 32 * WAVE)

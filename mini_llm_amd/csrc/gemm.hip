@@ -10,6 +10,16 @@
 
 namespace {
 
+// For a fused q/k/v projection whose key and value columns go straight into the cache pages
+// ([num_pages, n_kv_heads, page_size, head_size]) instead of the output matrix.
+struct CacheScatter {
+    void* k_pages;
+    void* v_pages;
+    const int* slots;  // per row: page * page_size + offset, negative = padding row
+    int q_width, kv_width, n_kv_heads, head_size, page_shift;
+    int enabled;
+};
+
 template <typename T>
 struct Tile;
 template <>
@@ -203,7 +213,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 template <typename T, typename OutT, int MT, int KSPLIT>
 __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     const T* __restrict__ A, const T* __restrict__ W, const float* __restrict__ bias,
-    const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue) {
+    const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue,
+    CacheScatter scatter) {
     constexpr int VEC = Tile<T>::VEC;
     constexpr int KSTEP = 4 * VEC;  // k covered by one load of the wave: 4 lane groups x 16 bytes
     constexpr int UNROLL = 4;
@@ -281,6 +292,21 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         if (bias) value += bias[col];
         if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
         else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+        if (scatter.enabled) {
+            if (col < scatter.q_width) {
+                out[(size_t)token * scatter.q_width + col] = from_float<OutT>(value);
+            } else {
+                int slot = scatter.slots[token];
+                if (slot < 0) continue;
+                int c = col - scatter.q_width;
+                OutT* pages = (OutT*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
+                if (c >= scatter.kv_width) c -= scatter.kv_width;
+                int kv_head = c / scatter.head_size, d = c % scatter.head_size;
+                int page = slot >> scatter.page_shift, offset = slot & ((1 << scatter.page_shift) - 1);
+                pages[((((size_t)page * scatter.n_kv_heads + kv_head) << scatter.page_shift) + offset) * scatter.head_size + d] = from_float<OutT>(value);
+            }
+            continue;
+        }
         size_t at = (size_t)token * N + col;
         if (residual) value = residual[at] + value;
         out[at] = from_float<OutT>(value);
@@ -289,20 +315,20 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 
 template <typename T, typename OutT, int MT>
 void launch_skinny(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M,
-                   int N, int K, int epilogue, hipStream_t stream) {
+                   int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}) {
     constexpr int KSTEP = 4 * Tile<T>::VEC;
     int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
     int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
     while (split < 8 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
     dim3 grid(tiles);
     if (split == 1)
-        gemm_skinny_kernel<T, OutT, MT, 1><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+        gemm_skinny_kernel<T, OutT, MT, 1><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
     else if (split == 2)
-        gemm_skinny_kernel<T, OutT, MT, 2><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+        gemm_skinny_kernel<T, OutT, MT, 2><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
     else if (split == 4)
-        gemm_skinny_kernel<T, OutT, MT, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+        gemm_skinny_kernel<T, OutT, MT, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
     else
-        gemm_skinny_kernel<T, OutT, MT, 8><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+        gemm_skinny_kernel<T, OutT, MT, 8><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
 }
 
 int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
@@ -373,4 +399,28 @@ MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const fl
     else
         MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
     return mllm_check_launch("gemm");
+}
+
+// The fused q/k/v projection of a decode step or a short portion (M <= 64 rows): q columns go
+// to out_q [M, q_width], key and value columns straight into the cache pages at slots[row]
+// (what the reference's decode block does with its fused matvec: engine/src/transformer_block.cu:223-242).
+MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, const float* bias, void* out_q, void* k_pages,
+                                 void* v_pages, const int* slots, int M, int K, int q_width, int kv_width,
+                                 int n_kv_heads, int head_size, int page_size, int dtype, hipStream_t stream) {
+    MLLM_REQUIRE(M >= 0 && M <= 64, "gemm_qkv_cache: %d rows; this entry takes up to 64", M);
+    MLLM_REQUIRE(K > 0 && q_width > 0 && kv_width == n_kv_heads * head_size && head_size > 0, "gemm_qkv_cache: bad sizes");
+    MLLM_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "gemm_qkv_cache: page size %d is no power of two", page_size);
+    MLLM_REQUIRE(dtype == MLLM_F32 || dtype == MLLM_BF16, "gemm_qkv_cache: unknown dtype %d", dtype);
+    MLLM_REQUIRE(K % (dtype == MLLM_F32 ? 4 : 8) == 0, "gemm_qkv_cache: K=%d is not a multiple of a 16-byte piece", K);
+    if (M == 0) return 0;
+    CacheScatter scatter{k_pages, v_pages, slots, q_width, kv_width, n_kv_heads, head_size, 0, 1};
+    while ((1 << scatter.page_shift) < page_size) scatter.page_shift++;
+    int N = q_width + 2 * kv_width;
+#define MLLM_QKV_CASE(T)                                                                                              \
+    if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
+    else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
+    else launch_skinny<T, T, 4>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
+    if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
+#undef MLLM_QKV_CASE
+    return mllm_check_launch("gemm_qkv_cache");
 }

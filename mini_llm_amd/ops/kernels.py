@@ -153,9 +153,35 @@ def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
     check(library().mllm_cache_write(_ptr(k_src), _ptr(v_src), k_src.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(slots), n, n_kv_heads, head_size, page_size, _code(k_pages.dtype), _stream()))
 
 
+FUSED_QKV_MAX_ROWS = 64
+
+
+def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_heads, head_size):
+    """The fused q/k/v projection of up to 64 rows: returns q [rows, n_heads*head_size] and writes
+    the key and value columns straight into the cache pages at slots[row] (negative: skip)."""
+    _device_tensor(x, "x", dim=2)
+    _device_tensor(weight, "weight", x.dtype, 2)
+    num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    _require(k_pages.dtype == x.dtype, "pages and x differ in element type")
+    m, k = x.shape
+    q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
+    _require(m <= FUSED_QKV_MAX_ROWS, f"{m} rows; the fused projection takes up to {FUSED_QKV_MAX_ROWS}")
+    _require(tuple(weight.shape) == (q_width + 2 * kv_width, k), "weight does not match the heads or x")
+    _require(k % (16 // x.element_size()) == 0, "the input width is not a multiple of a 16-byte piece")
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == weight.shape[0], "bias does not match weight")
+    _device_tensor(slots, "slots", torch.int32, 1)
+    _require(slots.shape[0] >= m, "fewer slots than rows")
+    q = torch.empty((m, q_width), dtype=x.dtype, device=x.device)
+    check(library().mllm_gemm_qkv_cache(_ptr(x), _ptr(weight), _ptr(bias), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(slots), m, k, q_width, kv_width, n_kv_heads, head_size, page_size, _code(x.dtype), _stream()))
+    return q
+
+
 DECODE_MAX_Q_LEN = 8        # portions up to this many tokens take the split-key kernel
-DECODE_TARGET_WAVES = 2048  # enough waves to fill 256 compute units several times over
-DECODE_MIN_SPLIT = 64       # keys
+DECODE_TARGET_WAVES = 1024  # waves that fill the chip
+DECODE_MIN_SPLIT = 64       # keys a wave should at least have
+DECODE_MAX_SPLITS = 16      # waves per block
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None):
@@ -164,7 +190,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
     row of block_tables that holds the request's pages (negative: padding row, output zero).
     ``max_q_len`` (the longest portion in the batch) picks the kernel; ``max_len`` (the longest
-    sequence after this step) only balances the split of the keys over waves. ``q_starts``
+    sequence after this step) only sets how many waves share a token's keys. ``q_starts``
     ([requests + 1], first row of each request's portion; its rows are contiguous) and
     ``context_lens`` ([requests], keys stored before this step) let long portions take the
     matrix-core kernel, which walks tiles of one request's queries."""
@@ -188,15 +214,13 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     rows_aligned = q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0  # 16-byte loads of q
     if (max_q_len is not None and max_q_len <= DECODE_MAX_Q_LEN and rows_aligned
             and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))):
-        # decoding and short portions: the keys of each (token, head) are split over waves
+        # decoding and short portions: a block per (token, head) whose waves share the keys; more
+        # waves per block when there are few blocks, never more than one per 64 keys of reach
         reach = block_tables.shape[1] * page_size if max_len is None else max(1, min(max_len, block_tables.shape[1] * page_size))
-        n_splits = max(1, min(DECODE_TARGET_WAVES // (n * n_heads), -(-reach // DECODE_MIN_SPLIT)))
-        keys_per_split = -(-reach // n_splits)
-        keys_per_split = -(-keys_per_split // DECODE_MIN_SPLIT) * DECODE_MIN_SPLIT
-        n_splits = -(-reach // keys_per_split)
-        floats = lib.mllm_attention_decode_scratch(n, n_heads, head_size, n_splits)
-        scratch = torch.empty((floats,), dtype=torch.float32, device=q.device)
-        check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(scratch), floats, _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), keys_per_split, n_splits, _code(q.dtype), _stream()))
+        n_splits = 1
+        while n_splits < DECODE_MAX_SPLITS and n * n_heads * n_splits < DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < reach:
+            n_splits *= 2
+        check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), _stream()))
         return out
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):

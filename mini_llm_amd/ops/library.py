@@ -19,9 +19,10 @@ _SIGNATURES = {
     "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_qkv_cache": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
-    "mllm_attention_decode": [P, c_int, P, P, P, c_longlong, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
@@ -52,8 +53,6 @@ def library() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = c_int
-        lib.mllm_attention_decode_scratch.argtypes = [c_int, c_int, c_int, c_int]
-        lib.mllm_attention_decode_scratch.restype = c_longlong
         lib.mllm_last_error.restype = ctypes.c_char_p
         lib.mllm_last_error.argtypes = []
         lib.path = path

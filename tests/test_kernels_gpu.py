@@ -304,3 +304,30 @@ def test_operands_are_checked_on_the_host(K):
         K.layernorm(x, torch.ones(7, device=DEV), torch.ones(8, device=DEV), 1e-5)
     with pytest.raises(OperandError):
         K.linear(x.t(), torch.zeros((3, 4), device=DEV))  # not contiguous
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16)])
+def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size):
+    rng = np.random.default_rng(rows)
+    width = 72
+    qw, kvw = n_heads * head_size, n_kv_heads * head_size
+    x, w, b = rng.standard_normal((rows, width)), rng.standard_normal((qw + 2 * kvw, width)) / 8, rng.standard_normal(qw + 2 * kvw)
+    num_pages = 8
+    kp = torch.full((num_pages, n_kv_heads, page_size, head_size), 7.0, device=DEV).to(dtype)
+    vp = torch.full_like(kp, 7.0)
+    slots = rng.permutation(num_pages * page_size)[:rows].astype(np.int32)
+    if rows > 2:
+        slots[1] = -1  # a padding row writes nothing
+    q = K.linear_qkv_cache(dev(x, dtype), dev(w, dtype), dev(b), kp, vp, dev(slots, torch.int32), n_heads, n_kv_heads, head_size)
+    xr, wr = (x.astype(np.float32).astype(np.float64), w.astype(np.float32).astype(np.float64)) if dtype == torch.float32 else (bf16_round(x), bf16_round(w))
+    ref = xr @ wr.T + b.astype(np.float32)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(q), ref[:, :qw], rtol=tol, atol=tol)
+    k_ref, v_ref = np.full((num_pages, n_kv_heads, page_size, head_size), 7.0), np.full((num_pages, n_kv_heads, page_size, head_size), 7.0)
+    for r, slot in enumerate(slots):
+        if slot >= 0:
+            k_ref[slot // page_size, :, slot % page_size, :] = ref[r, qw : qw + kvw].reshape(n_kv_heads, head_size)
+            v_ref[slot // page_size, :, slot % page_size, :] = ref[r, qw + kvw :].reshape(n_kv_heads, head_size)
+    np.testing.assert_allclose(host(kp), k_ref, rtol=tol, atol=tol)
+    np.testing.assert_allclose(host(vp), v_ref, rtol=tol, atol=tol)
