@@ -217,7 +217,9 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     CacheScatter scatter) {
     constexpr int VEC = Tile<T>::VEC;
     constexpr int KSTEP = 4 * VEC;  // k covered by one load of the wave: 4 lane groups x 16 bytes
-    constexpr int UNROLL = 4;
+    // Loads in flight per wave before any is used. At decode sizes a wave's whole share of K fits
+    // in one round (768 / 4 waves = 6 steps), and the kernel waits for memory once.
+    constexpr int UNROLL = MT == 1 ? 8 : 4;
     __shared__ float sums[KSPLIT][MT * 4][WAVE];
 
     const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
@@ -319,9 +321,11 @@ void launch_skinny(const T* a, const T* w, const float* bias, const float* resid
     constexpr int KSTEP = 4 * Tile<T>::VEC;
     int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
     int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
-    while (split < 8 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
+    while (split < 16 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
     dim3 grid(tiles);
-    if (split == 1)
+    if (split == 16)
+        gemm_skinny_kernel<T, OutT, MT, 16><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    else if (split == 1)
         gemm_skinny_kernel<T, OutT, MT, 1><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
     else if (split == 2)
         gemm_skinny_kernel<T, OutT, MT, 2><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
