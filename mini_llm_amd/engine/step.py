@@ -15,7 +15,7 @@ buffer per bucket that is overwritten before each replay."""
 from __future__ import annotations
 
 from ..cache import CacheManager, OutOfPages
-from .batch import BatchStaging, StepBatch, StepEntry, build_step_batch, padded_size
+from .batch import BatchStaging, DecodeBatchBuilder, StepBatch, StepEntry, build_step_batch
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 
@@ -31,7 +31,9 @@ class _DecodeGraph:
         import torch
 
         self.runner, self.capacity = runner, capacity
-        self.buffer = torch.zeros(padded_size(runner.cache, capacity), dtype=torch.int32, device=runner.device)
+        self.builder = DecodeBatchBuilder(runner.cache, capacity)
+        self.buffer = torch.zeros(len(self.builder.flat), dtype=torch.int32, device=runner.device)
+        self.static_batch = self.builder.batch(self.buffer, [])
         self.graph = None
         self.logits = None
 
@@ -39,8 +41,9 @@ class _DecodeGraph:
         import torch
 
         runner = self.runner
-        batch = build_step_batch(entries, runner.cache, runner.staging, vocab_size=runner.model.vocab_size,
-                                 capacity=self.capacity, device_buffer=self.buffer)
+        runner.staging.upload(self.builder.fill(entries), into=self.buffer)
+        batch = self.static_batch
+        batch.request_ids = [e.request_id for e in entries]
         if self.graph is None:
             # once eagerly (on a side stream, as capture needs), then the capture itself
             side = torch.cuda.Stream(device=runner.device)
