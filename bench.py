@@ -147,6 +147,7 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
+    parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})")
@@ -160,6 +161,9 @@ def main() -> int:
     largest = max(args.batch, 1 if args.no_points else 64)
     engine = Engine.from_random(config, SEED, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
 
+    if args.prefill_only:
+        print(json.dumps({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}))
+        return 0
     seconds, step_bytes = DecodeBench(engine, args.batch).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
     achieved = step_bytes / (seconds / args.steps) / 1e9

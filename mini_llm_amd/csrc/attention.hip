@@ -493,6 +493,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     constexpr int UNITS = (SPAN / ROWS_PER_UNIT) * PIECES_PER_ROW;
     constexpr int UNITS_PER_THREAD = (UNITS + THREADS - 1) / THREADS;
     Vec16 k_regs[UNITS_PER_THREAD][ROWS_PER_UNIT], v_regs[UNITS_PER_THREAD][ROWS_PER_UNIT];
+    bool kv_valid[UNITS_PER_THREAD][ROWS_PER_UNIT];
     auto fetch = [&](int k_base) {
 #pragma unroll
         for (int i = 0; i < UNITS_PER_THREAD; i++) {
@@ -509,10 +510,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
                 size_t at = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask)) * head_size + min(c * VEC, head_size - VEC);
                 k_regs[i][e] = *reinterpret_cast<const Vec16*>(k_pages + at);
                 v_regs[i][e] = *reinterpret_cast<const Vec16*>(v_pages + at);
-                if (!valid) {
-                    k_regs[i][e] = Vec16{{0u, 0u, 0u, 0u}};
-                    v_regs[i][e] = Vec16{{0u, 0u, 0u, 0u}};
-                }
+                kv_valid[i][e] = valid;  // applied when the tile is staged: nothing here waits for a load
             }
         }
     };
@@ -526,8 +524,15 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
             T* k_tile = k_tiles + tile * L::K_ELEMS;
             T* v_tile = v_tiles + tile * L::V_ELEMS;
 #pragma unroll
-            for (int e = 0; e < ROWS_PER_UNIT; e++)
+            for (int e = 0; e < ROWS_PER_UNIT; e++) {
+                uint32_t mask = kv_valid[i][e] ? 0xffffffffu : 0u;
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    k_regs[i][e].w[w] &= mask;
+                    v_regs[i][e].w[w] &= mask;
+                }
                 *reinterpret_cast<Vec16*>(&k_tile[(in_tile + e) * L::K_STRIDE + c * VEC]) = k_regs[i][e];
+            }
             if constexpr (HALF) {
                 const uint16_t* v0 = reinterpret_cast<const uint16_t*>(&v_regs[i][0]);
                 const uint16_t* v1 = reinterpret_cast<const uint16_t*>(&v_regs[i][ROWS_PER_UNIT - 1]);
@@ -551,7 +556,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
         __syncthreads();  // the previous tiles have been consumed
         stage();
         __syncthreads();
-        if (k_base + SPAN <= block_last_position) fetch(k_base + SPAN);
+        fetch(k_base + SPAN);  // unconditional: beyond the last key it reads a clamped address and is masked away
         const int k0 = k_base + key_split * PF_KEYS;
         // a wave whose queries all lie before its tile, or whose windows have all passed it, has nothing to add
         if (!wave_active || k0 > wave_last_position) continue;

@@ -35,21 +35,21 @@ struct Tile<bf16_t> {
     static constexpr int PAD = 8;
 };
 
-// One 16-byte piece of a row, zero where the matrix ends. With ALIGNED (K a multiple of VEC, so
-// every row starts on a 16-byte boundary and a piece is whole or absent) the load is
-// unconditional from a clamped address and the result is selected afterwards: no branch stands
-// between the loads of a tile, so they are all in flight together. Otherwise the piece is
-// gathered element by element.
+// One 16-byte piece of a row. With ALIGNED (K a multiple of VEC, so every row starts on a
+// 16-byte boundary and a piece is whole or absent) the load is unconditional from a clamped
+// address; whether the piece lies inside the matrix is returned in `valid` and applied later,
+// when the piece goes to LDS (mask_piece). Nothing then depends on a load until the tile is
+// staged, so all loads of two tiles stay in flight. Otherwise (unaligned K) the piece is gathered
+// element by element, zero where the matrix ends.
 template <typename T, bool ALIGNED>
-__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k, int K) {
+__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k, int K, bool& valid) {
     constexpr int VEC = Tile<T>::VEC;
     if constexpr (ALIGNED) {
-        bool valid = row < n_rows && k < K;
+        valid = row < n_rows && k < K;
         int safe_row = min(row, n_rows - 1), safe_k = min(k, K - VEC);
-        Vec16 v = *reinterpret_cast<const Vec16*>(base + (size_t)safe_row * K + safe_k);
-        if (!valid) v = Vec16{{0u, 0u, 0u, 0u}};
-        return v;
+        return *reinterpret_cast<const Vec16*>(base + (size_t)safe_row * K + safe_k);
     } else {
+        valid = true;
         Vec16 v = {{0u, 0u, 0u, 0u}};
         if (row >= n_rows || k >= K) return v;
         const T* p = base + (size_t)row * K + k;
@@ -59,6 +59,11 @@ __device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row,
             if (k + i < K) e[i] = p[i];
         return v;
     }
+}
+
+__device__ __forceinline__ Vec16 mask_piece(Vec16 v, bool valid) {
+    uint32_t mask = valid ? 0xffffffffu : 0u;
+    return Vec16{{v.w[0] & mask, v.w[1] & mask, v.w[2] & mask, v.w[3] & mask}};
 }
 
 // Block tile BM x BN, 4 waves laid out WAVES_M x WAVES_N, each wave TM x TN tiles of 32x32.
@@ -96,28 +101,29 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     Vec16 a_regs[2][A_PIECES], w_regs[2][W_PIECES];
+    bool a_valid[2][A_PIECES], w_valid[2][W_PIECES];
     auto fetch = [&](int set, int k0) {
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (piece < BM * VPR) a_regs[set][i] = load_piece<T, ALIGNED>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K);
+            if (BM * VPR % THREADS == 0 || piece < BM * VPR) a_regs[set][i] = load_piece<T, ALIGNED>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K, a_valid[set][i]);
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (piece < BN * VPR) w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K);
+            if (BN * VPR % THREADS == 0 || piece < BN * VPR) w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, w_valid[set][i]);
         }
     };
     auto stage = [&](int set) {
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (piece < BM * VPR) *reinterpret_cast<Vec16*>(&a_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = a_regs[set][i];
+            if (piece < BM * VPR) *reinterpret_cast<Vec16*>(&a_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = mask_piece(a_regs[set][i], a_valid[set][i]);
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = w_regs[set][i];
+            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = mask_piece(w_regs[set][i], w_valid[set][i]);
         }
     };
     auto products = [&]() {
@@ -164,19 +170,21 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
         }
     };
 
+    // Every fetch is unconditional (beyond K it reads a clamped address and is masked away): with
+    // no branch around the loads, the wait before a tile is staged counts exactly the loads of the
+    // other set that may still be in flight.
     fetch(0, 0);
-    if (BK < K) fetch(1, BK);
+    fetch(1, BK);
     for (int k0 = 0; k0 < K; k0 += 2 * BK) {
         __syncthreads();  // the previous tile has been consumed
         stage(0);
         __syncthreads();
-        if (k0 + 2 * BK < K) fetch(0, k0 + 2 * BK);
+        fetch(0, k0 + 2 * BK);
         products();
-        if (k0 + BK >= K) break;
         __syncthreads();
-        stage(1);
+        stage(1);  // all zeros if K ended with the tile above
         __syncthreads();
-        if (k0 + 3 * BK < K) fetch(1, k0 + 3 * BK);
+        fetch(1, k0 + 3 * BK);
         products();
     }
 
@@ -248,16 +256,19 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         Vec16 w_piece[UNROLL], x_piece[UNROLL][MT];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
-            int k = (step0 + u) * KSTEP + quad * VEC;
-            bool k_valid = k < K;  // K is a multiple of VEC: a piece is whole or absent
+            int k = (step0 + u) * KSTEP + quad * VEC;  // K is a multiple of VEC: a piece is whole or absent
             int safe_k = min(k, K - VEC);  // loads are unconditional, from a clamped address: no branch between them
             w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + safe_k);
-            if (!(k_valid && n_valid)) w_piece[u] = Vec16{{0u, 0u, 0u, 0u}};
 #pragma unroll
-            for (int i = 0; i < MT; i++) {
-                x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + safe_k);
-                if (!(k_valid && x_valid[i])) x_piece[u][i] = Vec16{{0u, 0u, 0u, 0u}};
-            }
+            for (int i = 0; i < MT; i++) x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + safe_k);
+        }
+        // what lies outside the matrices is zeroed only now, so that nothing above waits for a load
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            bool k_valid = (step0 + u) * KSTEP + quad * VEC < K;
+            w_piece[u] = mask_piece(w_piece[u], k_valid && n_valid);
+#pragma unroll
+            for (int i = 0; i < MT; i++) x_piece[u][i] = mask_piece(x_piece[u][i], k_valid && x_valid[i]);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
