@@ -99,8 +99,13 @@ class DecodeBench:
             n = min(steps - done, CONTEXT - self.length)
             torch.cuda.synchronize()
             begin = time.perf_counter()
-            for _ in range(n):
-                self.last = self.engine.decode_batch(self.handles, self.last)
+            # Queued decoding, one step ahead: step k+1 takes its tokens from the device, where
+            # step k's sampler left them, and is launched before the host reads step k's tokens.
+            self.engine.decode_batch_enqueue(self.handles)
+            for _ in range(n - 1):
+                self.engine.decode_batch_enqueue(self.handles)
+                self.last = self.engine.take()
+            self.last = self.engine.take()
             torch.cuda.synchronize()
             seconds += time.perf_counter() - begin
             for k in range(n):

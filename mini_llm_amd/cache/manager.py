@@ -50,8 +50,14 @@ class CacheManager:
         self.state_needs = dict(state_needs)
         self.device, self.dtype = device, dtype
         self.k_pages, self.v_pages, self.state = {}, {}, {}
+        # Per request, whatever the model: the token the sampler chose last, kept on the device so
+        # that the next step can start before the host has seen it (the reference keeps such a
+        # token queue inside each cache object: engine/include/gpt2_gpu_internal.h:38-48).
+        self.last_token = None
         if device is not None:
             import torch
+
+            self.last_token = torch.zeros((max_requests,), dtype=torch.int32, device=device)
 
             for gi, g in enumerate(self.groups):
                 shape = (len(g.layers), 2, self.pools[gi].num_pages, g.n_kv_heads, page_size, g.head_size)

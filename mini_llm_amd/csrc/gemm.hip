@@ -84,8 +84,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
     constexpr int A_PIECES = (BM * VPR + THREADS - 1) / THREADS, W_PIECES = (BN * VPR + THREADS - 1) / THREADS;
     static_assert(TM >= 1 && TN >= 1, "tile layout");
 
-    __shared__ __attribute__((aligned(16))) T a_tile[BM * LDK];
-    __shared__ __attribute__((aligned(16))) T w_tile[BN * LDK];
+    __shared__ __attribute__((aligned(16))) T a_tiles[2][BM * LDK];  // two buffers: one is read while
+    __shared__ __attribute__((aligned(16))) T w_tiles[2][BN * LDK];  // the next tile is written to the other
 
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
@@ -114,7 +114,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
             if (BN * VPR % THREADS == 0 || piece < BN * VPR) w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, w_valid[set][i]);
         }
     };
-    auto stage = [&](int set) {
+    auto stage = [&](int set) {  // register set `set` -> LDS buffer `set`
+        T* a_tile = a_tiles[set];
+        T* w_tile = w_tiles[set];
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
             int piece = tid + i * THREADS;
@@ -126,7 +128,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
             if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = mask_piece(w_regs[set][i], w_valid[set][i]);
         }
     };
-    auto products = [&]() {
+    auto products = [&](int buffer) {
+        const T* a_tile = a_tiles[buffer];
+        const T* w_tile = w_tiles[buffer];
         if constexpr (sizeof(T) == 2) {
 #pragma unroll
             for (int kk = 0; kk < BK / 16; kk++) {
@@ -172,20 +176,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 
     // Every fetch is unconditional (beyond K it reads a clamped address and is masked away): with
     // no branch around the loads, the wait before a tile is staged counts exactly the loads of the
-    // other set that may still be in flight.
+    // other set that may still be in flight. One barrier a tile: while buffer b is multiplied, the
+    // next tile goes into buffer 1-b, which every wave left before the barrier above.
     fetch(0, 0);
     fetch(1, BK);
+    stage(0);
+    fetch(0, 2 * BK);
+    __syncthreads();
     for (int k0 = 0; k0 < K; k0 += 2 * BK) {
-        __syncthreads();  // the previous tile has been consumed
-        stage(0);
-        __syncthreads();
-        fetch(0, k0 + 2 * BK);
-        products();
-        __syncthreads();
-        stage(1);  // all zeros if K ended with the tile above
-        __syncthreads();
+        stage(1);  // tile k0 + BK (zeros beyond K)
         fetch(1, k0 + 3 * BK);
-        products();
+        products(0);
+        __syncthreads();
+        stage(0);  // tile k0 + 2 BK
+        fetch(0, k0 + 4 * BK);
+        products(1);
+        __syncthreads();
     }
 
     // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
@@ -382,11 +388,17 @@ void launch_gemm(const void* A, const void* W, const float* bias, const float* r
     const T* a = (const T*)A;
     const T* w = (const T*)W;
     OutT* o = (OutT*)out;
-    if (M <= 64 && K % Tile<T>::VEC == 0) {
+    const bool aligned = K % Tile<T>::VEC == 0;
+    // Few rows: the skinny kernel, except for a very wide matrix (the head over the vocabulary),
+    // where a block of the skinny kernel would read the rows again for every 16 columns and the
+    // tiled kernel with a short tile streams faster. The borders are measured on MI355X.
+    const bool wide = N >= 8192;
+    const int skinny_rows = !wide ? 64 : (sizeof(T) == 2 ? 0 : 12);
+    if (g_forced_tile == 0 && aligned && M <= skinny_rows) {
         if (M <= 16) launch_skinny<T, OutT, 1>(a, w, bias, residual, o, M, N, K, epilogue, stream);
         else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream);
         else launch_skinny<T, OutT, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream);
-    } else if (K % Tile<T>::VEC == 0) {
+    } else if (aligned) {
         launch_tiled<T, OutT, true>(a, w, bias, residual, o, M, N, K, epilogue, stream);
     } else {
         launch_tiled<T, OutT, false>(a, w, bias, residual, o, M, N, K, epilogue, stream);

@@ -63,14 +63,17 @@ __device__ __forceinline__ float uniform_open(uint64_t seed, uint32_t step, uint
     return ((float)(z >> 40) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
 }
 
-// One block per row. temperature 0: argmax. Otherwise a draw from softmax(logits / temperature)
+// One block per row. With token_slots the chosen token is also left in token_slots[slot_of_row[row]]
+// (the request's last-token slot), from where the next step can take it without the host having
+// seen it. temperature 0: argmax. Otherwise a draw from softmax(logits / temperature)
 // cut to the nucleus top_p (token i stays if the mass of all strictly more likely tokens is
 // below top_p), taken as argmax(logit/temperature + Gumbel noise): it reuses the argmax
 // reduction and does not depend on a summation order.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int vocab, const float* __restrict__ temperatures,
     const float* __restrict__ top_ps, const uint64_t* __restrict__ seeds,
-    const int* __restrict__ steps, int* __restrict__ out_tokens) {
+    const int* __restrict__ steps, int* __restrict__ out_tokens, int* __restrict__ token_slots,
+    const int* __restrict__ slot_of_row) {
     __shared__ float shared_values[SAMPLE_THREADS / WAVE];
     __shared__ int shared_indices[SAMPLE_THREADS / WAVE];
     const int row = blockIdx.x, tid = threadIdx.x;
@@ -86,7 +89,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
     block_best(best, best_index, shared_values, shared_indices);
     if (!(temperature > 0.0f) || best != best) {  // greedy, or a NaN in the row
-        if (tid == 0) out_tokens[row] = best_index;
+        if (tid == 0) {
+            out_tokens[row] = best_index;
+            if (token_slots && slot_of_row[row] >= 0) token_slots[slot_of_row[row]] = best_index;
+        }
         return;
     }
 
@@ -130,17 +136,20 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
     }
     block_best(chosen, chosen_index, shared_values, shared_indices);
-    if (tid == 0) out_tokens[row] = chosen_index;
+    if (tid == 0) {
+        out_tokens[row] = chosen_index;
+        if (token_slots && slot_of_row[row] >= 0) token_slots[slot_of_row[row]] = chosen_index;
+    }
 }
 
 }  // namespace
 
 MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float* temperatures,
                          const float* top_ps, const unsigned long long* seeds, const int* steps,
-                         int* out_tokens, hipStream_t stream) {
+                         int* out_tokens, int* token_slots, const int* slot_of_row, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", n_rows, vocab);
     if (n_rows == 0) return 0;
     sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, vocab, temperatures, top_ps,
-                                                         (const uint64_t*)seeds, steps, out_tokens);
+                                                         (const uint64_t*)seeds, steps, out_tokens, token_slots, slot_of_row);
     return mllm_check_launch("sample");
 }

@@ -20,6 +20,9 @@ class StepEntry:
     request_id: object
     tokens: list
     want: list = field(default_factory=list)
+    # The (single) token is the one the sampler left in the request's last-token slot on the
+    # device in an earlier step; ``tokens`` then holds a placeholder the host never looks at.
+    from_slot: bool = False
 
 
 @dataclass
@@ -42,6 +45,7 @@ class StepBatch:
     context_lens: object    # int32 [n_requests]: tokens stored before this step
     state_slots: object     # int32 [n_requests]
     logit_rows: object      # int32 [n_logit_rows]: rows whose logits are computed
+    token_sources: object   # int32 [n_tokens]: last-token slot a row's token is taken from, -1 = as given
     groups: list            # GroupStepData per cache group
     request_ids: list = field(default_factory=list)
     host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
@@ -127,6 +131,10 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     q_starts[1 : n_requests + 1] = np.cumsum(q_lens)
     logit_rows = np.asarray([q_starts[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
     state_slots = np.asarray([cache.requests[e.request_id].state_slot for e in entries], dtype=np.int32)
+    token_sources = np.full(cap_tokens, -1, dtype=np.int32)
+    for i, e in enumerate(entries):
+        if e.from_slot:
+            token_sources[q_starts[i]] = state_slots[i]
     tables, slots = [], []
     for gi in range(n_groups):
         table = np.full((cap_requests, table_width), -1, dtype=np.int32)
@@ -143,7 +151,8 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         logit_rows = _pad(logit_rows, cap_tokens, 0)
 
     sections = [_pad(tokens, cap_tokens, -1), _pad(positions, cap_tokens, 0), _pad(token_request, cap_tokens, -1), q_starts,
-                _pad(np.asarray(contexts, dtype=np.int32), cap_requests, 0), _pad(state_slots, cap_requests, 0), logit_rows]
+                _pad(np.asarray(contexts, dtype=np.int32), cap_requests, 0), _pad(state_slots, cap_requests, 0), logit_rows,
+                token_sources]
     for table, slot in zip(tables, slots):
         sections += [table.reshape(-1), slot]
     offsets, total = [], 0
@@ -152,7 +161,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         total += _aligned(len(section))
     host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts[: n_requests + 1],
             "context_lens": sections[4][:n_requests], "state_slots": state_slots, "logit_rows": logit_rows[:n_logit_rows],
-            "block_tables": tables, "slots": slots}
+            "token_sources": token_sources[:n_tokens], "block_tables": tables, "slots": slots}
     if staging is None:
         views = sections
     else:
@@ -162,14 +171,15 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         device = staging.upload(flat, into=device_buffer)
         views = [device[o : o + len(s)] for o, s in zip(offsets, sections)]
     groups = [
-        GroupStepData(block_tables=views[7 + 2 * gi].reshape(cap_requests, table_width), slots=views[8 + 2 * gi])
+        GroupStepData(block_tables=views[8 + 2 * gi].reshape(cap_requests, table_width), slots=views[9 + 2 * gi])
         for gi in range(n_groups)
     ]
     return StepBatch(
         n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
         max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
-        state_slots=views[5], logit_rows=views[6], groups=groups, request_ids=[e.request_id for e in entries], host=host,
+        state_slots=views[5], logit_rows=views[6], token_sources=views[7], groups=groups,
+        request_ids=[e.request_id for e in entries], host=host,
     )
 
 
@@ -183,7 +193,7 @@ class DecodeBatchBuilder:
         self.cache, self.capacity = cache, capacity
         self.table_width = cache.max_blocks()
         n_groups = len(cache.groups)
-        lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 3
+        lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
         for _ in range(n_groups):
             lengths += [capacity * self.table_width, capacity]
         self.offsets, total = [], 0
@@ -194,9 +204,9 @@ class DecodeBatchBuilder:
         self.flat = np.zeros(max(total, 4), dtype=np.int32)
         view = lambda i: self.flat[self.offsets[i] : self.offsets[i] + lengths[i]]
         self.tokens, self.positions, self.token_request, self.q_starts = view(0), view(1), view(2), view(3)
-        self.context_lens, self.state_slots, self.logit_rows = view(4), view(5), view(6)
-        self.tables = [view(7 + 2 * g).reshape(capacity, self.table_width) for g in range(n_groups)]
-        self.slots = [view(8 + 2 * g) for g in range(n_groups)]
+        self.context_lens, self.state_slots, self.logit_rows, self.token_sources = view(4), view(5), view(6), view(7)
+        self.tables = [view(8 + 2 * g).reshape(capacity, self.table_width) for g in range(n_groups)]
+        self.slots = [view(9 + 2 * g) for g in range(n_groups)]
         self.filled = capacity  # rows that held a request in the previous step (all, so the first fill pads all)
 
     def fill(self, entries) -> np.ndarray:
@@ -209,6 +219,7 @@ class DecodeBatchBuilder:
         self.context_lens[:stale] = 0
         self.state_slots[:stale] = 0
         self.logit_rows[:] = 0
+        self.token_sources[:stale] = -1
         for table, slots in zip(self.tables, self.slots):
             table[:stale] = -1
             slots[:stale] = -1
@@ -222,6 +233,8 @@ class DecodeBatchBuilder:
             self.context_lens[i] = length
             self.state_slots[i] = request.state_slot
             self.logit_rows[i] = i
+            if entry.from_slot:
+                self.token_sources[i] = request.state_slot
             for g, pages in enumerate(request.tables):
                 self.tables[g][i, : len(pages)] = pages
                 self.slots[g][i] = pages[length // page] * page + length % page
@@ -231,20 +244,20 @@ class DecodeBatchBuilder:
     def batch(self, device_flat, entries) -> StepBatch:
         views = [device_flat[o : o + n] for o, n in zip(self.offsets, self.lengths)]
         n_groups = len(self.tables)
-        groups = [GroupStepData(block_tables=views[7 + 2 * g].reshape(self.capacity, self.table_width), slots=views[8 + 2 * g])
+        groups = [GroupStepData(block_tables=views[8 + 2 * g].reshape(self.capacity, self.table_width), slots=views[9 + 2 * g])
                   for g in range(n_groups)]
         return StepBatch(
             n_tokens=self.capacity, n_requests=self.capacity, n_logit_rows=self.capacity, max_q_len=1,
             max_total_len=self.cache.max_length, tokens=views[0], positions=views[1], token_request=views[2],
-            q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], groups=groups,
-            request_ids=[e.request_id for e in entries], host={},
+            q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], token_sources=views[7],
+            groups=groups, request_ids=[e.request_id for e in entries], host={},
         )
 
 
 def padded_size(cache, capacity: int) -> int:
     """int32 elements of a batch laid out for ``capacity`` tokens and requests."""
     table_width = cache.max_blocks()
-    lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 3
+    lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
     for _ in cache.groups:
         lengths += [capacity * table_width, capacity]
     return sum(_aligned(n) for n in lengths)

@@ -8,6 +8,7 @@ this framework's own scheduler with ``submit`` / ``step`` / ``generate``."""
 
 from __future__ import annotations
 
+import collections
 from dataclasses import dataclass
 
 import numpy as np
@@ -68,7 +69,7 @@ class _Executor:
         return self._engine.cache.can_reserve([(("scheduled", r), n) for r, n in wanted])
 
     def run(self, entries, sampling, steps):
-        entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want) for e in entries]
+        entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want, e.from_slot) for e in entries]
         logits = self._engine.runner.step(entries)
         if logits is None:
             return []
@@ -129,6 +130,8 @@ class Engine:
         self.sampler = Sampler(self.runner.staging)
         self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step)
         self._next_handle = 0
+        self._queued = collections.deque()   # (pinned tokens, count, event) of steps whose tokens were not taken yet
+        self._token_buffers, self._queue_turn = [], 0
 
     @classmethod
     def from_random(cls, config, seed: int, options: EngineOptions = EngineOptions()):
@@ -174,18 +177,56 @@ class Engine:
     def release_cache(self, handle) -> None:
         self.cache.close(handle)
 
+    def _greedy(self, logits, n: int):
+        """argmax per row on the device; each token is also left in its request's last-token slot."""
+        return self.sampler.sample(logits, [SamplingParams()] * n, [0] * n, token_slots=self.cache.last_token,
+                                   slot_of_row=self.runner.last_batch.state_slots)
+
     def prefill_greedy(self, handle, token_ids) -> int:
         tokens = [int(t) for t in token_ids]
         if not tokens:
             raise RuntimeError("the prompt has no tokens")
         logits = self.runner.step([StepEntry(handle, tokens, [len(tokens) - 1])])
-        return int(self.sampler.sample(logits, [SamplingParams()], [0]).cpu()[0])
+        return int(self._greedy(logits, 1).cpu()[0])
 
     def decode_batch(self, handles, tokens) -> list[int]:
         if len(handles) != len(tokens) or not handles:
             raise RuntimeError("a batch has one token per sequence and at least one sequence")
         logits = self.runner.step([StepEntry(h, [int(t)], [0]) for h, t in zip(handles, tokens)])
-        return self.sampler.sample(logits, [SamplingParams()] * len(handles), [0] * len(handles)).cpu().tolist()
+        return self._greedy(logits, len(handles)).cpu().tolist()
+
+    # --- queued decoding: step n+1 is launched before the host has read token n ------------------------
+    # (the reference's enqueue / take: engine/src/gpt2_gpu_greedy.cu:80-123, native.py:123-155)
+    MAX_QUEUED = 4
+
+    def decode_batch_enqueue(self, handles) -> None:
+        """Queues one greedy decode step for these sequences. Each sequence's input is the token
+        its previous step (``prefill_greedy``, ``decode_batch`` or an earlier enqueue) chose, taken
+        from its last-token slot on the device; the host need not have read it yet."""
+        import torch
+
+        if not handles:
+            raise RuntimeError("a batch has at least one sequence")
+        if len(self._queued) >= self.MAX_QUEUED:
+            raise RuntimeError(f"{self.MAX_QUEUED} steps are queued already: take one first")
+        logits = self.runner.step([StepEntry(h, [0], [0], from_slot=True) for h in handles])
+        tokens = self._greedy(logits, len(handles))
+        if len(self._token_buffers) < self.MAX_QUEUED:
+            self._token_buffers.append(torch.empty(self.options.max_sessions, dtype=torch.int32, pin_memory=True))
+        host = self._token_buffers[self._queue_turn % self.MAX_QUEUED]
+        self._queue_turn += 1
+        host[: len(handles)].copy_(tokens, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        self._queued.append((host, len(handles), event))
+
+    def take(self) -> list[int]:
+        """The tokens of the oldest queued step (waits for it)."""
+        if not self._queued:
+            raise RuntimeError("no step is queued")
+        host, n, event = self._queued.popleft()
+        event.synchronize()
+        return host[:n].tolist()
 
     # --- continuous batching ------------------------------------------------------------------------------
     def submit(self, request: Request) -> None:

@@ -15,6 +15,7 @@ buffer per bucket that is overwritten before each replay."""
 from __future__ import annotations
 
 from ..cache import CacheManager, OutOfPages
+from ..ops import kernels
 from .batch import BatchStaging, DecodeBatchBuilder, StepBatch, StepEntry, build_step_batch
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -49,12 +50,12 @@ class _DecodeGraph:
             side = torch.cuda.Stream(device=runner.device)
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                runner.model.forward(batch, runner.cache)
+                runner.forward(batch)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize(runner.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                self.logits = runner.model.forward(batch, runner.cache)
+                self.logits = runner.forward(batch)
             self.graph = graph
         self.graph.replay()
         return batch, self.logits[: len(entries)]
@@ -84,7 +85,9 @@ class ModelRunner:
             n = len(entry.tokens)
             if n < 1:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
-            for token in entry.tokens:
+            if entry.from_slot and n != 1:
+                raise StepError(f"request {entry.request_id!r}: only a single token can come from the last-token slot")
+            for token in ([] if entry.from_slot else entry.tokens):
                 if not isinstance(token, (int,)) and not hasattr(token, "__index__"):
                     raise StepError(f"request {entry.request_id!r}: token {token!r} is not an integer")
                 if not 0 <= int(token) < vocab:
@@ -95,6 +98,12 @@ class ModelRunner:
             for w in entry.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
+
+    def forward(self, batch, resolve: bool = True):
+        """Tokens that come from last-token slots are fetched on the device, then the model runs."""
+        if resolve:
+            kernels.resolve_tokens(batch.tokens, batch.token_sources, self.cache.last_token)
+        return self.model.forward(batch, self.cache)
 
     def _graph_for(self, entries):
         if not self.use_graphs or len(entries) > GRAPH_BUCKETS[-1]:
@@ -128,7 +137,7 @@ class ModelRunner:
                 self.graph_steps += 1
             else:
                 batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size)
-                logits = self.model.forward(batch, self.cache)
+                logits = self.forward(batch, resolve=any(e.from_slot for e in entries))
         except Exception:
             for request_id in reserved:
                 self.cache.rollback(request_id)

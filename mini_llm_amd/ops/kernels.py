@@ -179,7 +179,7 @@ def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_hea
 
 
 DECODE_MAX_Q_LEN = 8        # portions up to this many tokens take the split-key kernel
-DECODE_TARGET_WAVES = 1024  # waves that fill the chip
+DECODE_TARGET_WAVES = 4096  # waves that fill the chip (256 compute units, 16 each) and hide the latency of their loads
 DECODE_MIN_SPLIT = 64       # keys a wave should at least have
 DECODE_MAX_SPLITS = 16      # waves per block
 
@@ -235,10 +235,12 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     return out
 
 
-def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=None):
+def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=None, token_slots=None, slot_of_row=None):
     """One token per row of float32 logits. Without temperatures (or where one is 0): argmax by
     numpy's rules. Else a draw from softmax(logits/temperature) within the top_p nucleus; the
-    random numbers are a function of (seeds[row], steps[row], token index) alone."""
+    random numbers are a function of (seeds[row], steps[row], token index) alone. With
+    ``token_slots`` and ``slot_of_row`` the token of row r is also stored in
+    token_slots[slot_of_row[r]] (negative: not stored)."""
     _device_tensor(logits, "logits", torch.float32, 2)
     n, vocab = logits.shape
     for t, name, dtype in ((temperatures, "temperatures", torch.float32), (top_ps, "top_ps", torch.float32), (seeds, "seeds", torch.int64), (steps, "steps", torch.int32)):
@@ -249,5 +251,18 @@ def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=N
         out = torch.empty((n,), dtype=torch.int32, device=logits.device)
     _device_tensor(out, "out", torch.int32, 1)
     _require(out.shape[0] >= n, "out is too short")
-    check(library().mllm_sample(_ptr(logits), n, vocab, _ptr(temperatures), _ptr(top_ps), _ptr(seeds), _ptr(steps), _ptr(out), _stream()))
+    if token_slots is not None:
+        _device_tensor(token_slots, "token_slots", torch.int32, 1)
+        _device_tensor(slot_of_row, "slot_of_row", torch.int32, 1)
+        _require(slot_of_row.shape[0] >= n, "slot_of_row has fewer entries than rows")
+    check(library().mllm_sample(_ptr(logits), n, vocab, _ptr(temperatures), _ptr(top_ps), _ptr(seeds), _ptr(steps), _ptr(out), _ptr(token_slots), _ptr(slot_of_row if token_slots is not None else None), _stream()))
     return out
+
+
+def resolve_tokens(tokens, sources, token_slots):
+    """tokens[row] = token_slots[sources[row]] where sources[row] >= 0 (in place)."""
+    _device_tensor(tokens, "tokens", torch.int32, 1)
+    _device_tensor(sources, "sources", torch.int32, 1)
+    _device_tensor(token_slots, "token_slots", torch.int32, 1)
+    _require(sources.shape[0] >= tokens.shape[0], "fewer sources than tokens")
+    check(library().mllm_resolve_tokens(_ptr(tokens), _ptr(sources), _ptr(token_slots), tokens.shape[0], _stream()))

@@ -26,7 +26,8 @@ _SIGNATURES = {
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
-    "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P],
+    "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
+    "mllm_resolve_tokens": [P, P, P, c_int, P],
 }
 
 

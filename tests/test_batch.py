@@ -19,17 +19,18 @@ def test_decode_builder_matches_the_general_one():
         cache.reserve(name, lengths[name]); cache.commit(name, lengths[name])
     builder = DecodeBatchBuilder(cache, 8)
     for live in (["a", "b", "c", "d", "e"], ["e", "b"], ["c"], ["a", "b", "c", "d", "e"]):  # shrinking, then growing again
-        entries = [StepEntry(name, [int(rng.integers(0, 100))], [0]) for name in live]
+        entries = [StepEntry(name, [int(rng.integers(0, 100))], [0], from_slot=(k % 2 == 0)) for k, name in enumerate(live)]
         for e in entries:
             cache.reserve(e.request_id, 1)
         general = build_step_batch(entries, cache, None, vocab_size=100, capacity=8)
         flat = builder.fill(entries)
         fast = builder.batch(flat, entries)
-        for field in ("tokens", "positions", "token_request", "q_starts", "context_lens", "state_slots", "logit_rows"):
+        for field in ("tokens", "positions", "token_request", "q_starts", "context_lens", "state_slots", "logit_rows", "token_sources"):
             np.testing.assert_array_equal(getattr(fast, field), getattr(general, field), err_msg=field)
         for g in range(2):
             np.testing.assert_array_equal(fast.groups[g].block_tables, general.groups[g].block_tables)
             np.testing.assert_array_equal(fast.groups[g].slots, general.groups[g].slots)
+        assert (fast.token_sources[: len(live)] >= 0).tolist() == [k % 2 == 0 for k in range(len(live))]
         assert (fast.n_tokens, fast.n_requests, fast.n_logit_rows, fast.max_q_len) == (8, 8, 8, 1)
         for e in entries:
             cache.commit(e.request_id, 1)

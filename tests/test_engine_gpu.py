@@ -150,7 +150,9 @@ def test_the_reference_schedulers_four_calls(model_dirs, engines):
     for h in handles:
         engine.release_cache(h)
     assert got == [plain_gpt2.greedy(config, weights, p, 8) for p in prompts]
-    assert engine.try_take_cache() is not None
+    handle = engine.try_take_cache()
+    assert handle is not None
+    engine.release_cache(handle)
 
 
 def test_step_checks_everything_before_it_changes_anything(model_dirs, engines):
@@ -289,3 +291,50 @@ def test_graph_replays_match_eager_steps(model_dirs, dtype):
                 np.testing.assert_allclose(row, ref[name][position], err_msg=f"{name} {position} graphs={use_graphs}", **tol)
     for name in seqs:
         assert results[True][name].keys() == results[False][name].keys()
+
+
+def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
+    # step n+1 is launched before the host has read token n; the tokens must be those of the
+    # step-by-step calls and of the plain implementation (the reference's queued mode:
+    # engine/tests/test_gpt2_gpu_greedy.c:59-322)
+    _, config, weights = model_dirs["A"]
+    engine = engines("A", "float32", max_sessions=5)
+    prompts = [random_tokens(70 + i, n, config["vocab_size"]) for i, n in enumerate((4, 19, 60))]
+    handles = [engine.try_take_cache() for _ in prompts]
+    got = [[engine.prefill_greedy(h, p)] for h, p in zip(handles, prompts)]
+    engine.decode_batch_enqueue(handles)
+    engine.decode_batch_enqueue(handles)          # two steps in flight
+    for _ in range(10):
+        engine.decode_batch_enqueue(handles)
+        for g, t in zip(got, engine.take()):
+            g.append(t)
+    for _ in range(2):
+        for g, t in zip(got, engine.take()):
+            g.append(t)
+    with pytest.raises(RuntimeError, match="no step is queued"):
+        engine.take()
+    # a sequence leaves, the others go on; then a step-by-step call continues from the same state
+    engine.release_cache(handles[0])
+    engine.decode_batch_enqueue(handles[1:])
+    for g, t in zip(got[1:], engine.take()):
+        g.append(t)
+    last = engine.decode_batch(handles[1:], [g[-1] for g in got[1:]])
+    for g, t in zip(got[1:], last):
+        g.append(t)
+    for h in handles[1:]:
+        engine.release_cache(h)
+    assert got[0] == plain_gpt2.greedy(config, weights, prompts[0], 13)
+    assert got[1] == plain_gpt2.greedy(config, weights, prompts[1], 15)
+    assert got[2] == plain_gpt2.greedy(config, weights, prompts[2], 15)
+    for _ in range(engine.MAX_QUEUED):
+        h = engine.try_take_cache()
+        engine.prefill_greedy(h, prompts[0])
+        engine.decode_batch_enqueue([h])
+        engine.release_cache(h)
+    h = engine.try_take_cache()
+    engine.prefill_greedy(h, prompts[0])
+    with pytest.raises(RuntimeError, match="queued already"):
+        engine.decode_batch_enqueue([h])
+    engine.release_cache(h)
+    while engine._queued:
+        engine.take()
