@@ -82,11 +82,22 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
     float best = -INFINITY;
     int best_index = 0x7fffffff;
-    for (int i = tid; i < vocab; i += SAMPLE_THREADS)
-        if (beats(x[i], i, best, best_index)) {
-            best = x[i];
-            best_index = i;
+    // eight loads in flight per thread before any is compared: the row is read in a few rounds
+    // of memory latency instead of one per element
+    constexpr int BATCH = 8;
+    for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * BATCH) {
+        float values[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) values[u] = x[min(i0 + u * SAMPLE_THREADS, vocab - 1)];
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) {
+            int i = i0 + u * SAMPLE_THREADS;
+            if (i < vocab && beats(values[u], i, best, best_index)) {
+                best = values[u];
+                best_index = i;
+            }
         }
+    }
     block_best(best, best_index, shared_values, shared_indices);
     if (!(temperature > 0.0f) || best != best) {  // greedy, or a NaN in the row
         if (tid == 0) {
