@@ -62,12 +62,24 @@ TINY_C = {
 TINY = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 8)}
 
 
+def sharpen_attention(weights: dict, config: dict, factor: float = 8.0) -> None:
+    """With the benchmark's init the scores are a few hundredths and every softmax is nearly
+    uniform: keys could be swapped or a page mixed up and the logits would hardly move. The query
+    and key columns of c_attn are scaled up so that attention weights differ by orders of
+    magnitude and a wrong key shows."""
+    d = config["n_embd"]
+    for i in range(config["n_layer"]):
+        weights[f"h.{i}.attn.c_attn.weight"][:, : 2 * d] *= factor
+        weights[f"h.{i}.attn.c_attn.bias"][: 2 * d] *= factor
+
+
 def make_plain_model_dir(path: Path, config: dict, seed: int, bf16: bool = False, prefix: str = "transformer."):
     """A model folder written by the plain implementation's own writer."""
     import plain_gpt2
 
     path.mkdir(parents=True, exist_ok=True)
     weights = plain_gpt2.random_weights(config, seed)
+    sharpen_attention(weights, config)
     (path / "config.json").write_text(json.dumps(config))
     plain_gpt2.write_safetensors(
         path / "model.safetensors", {prefix + k: v for k, v in weights.items()}, bf16=bf16

@@ -331,3 +331,50 @@ def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_hea
             v_ref[slot // page_size, :, slot % page_size, :] = ref[r, qw + kvw :].reshape(n_kv_heads, head_size)
     np.testing.assert_allclose(host(kp), k_ref, rtol=tol, atol=tol)
     np.testing.assert_allclose(host(vp), v_ref, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("path", ["general", "split_keys", "matrix_cores"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("page_size,window", [(16, 0), (64, 0), (32, 100)])
+def test_attention_picks_out_single_keys(K, path, dtype, page_size, window):
+    # Random keys hide a wrong page or a missed tile among hundreds of near-equal weights. Here one
+    # key at a time gets a score far above the rest (at page edges, tile edges, the window's two
+    # sides, the first and the last key), and the output must be that key's value row, or, for
+    # the key just outside the window, must not be.
+    rng = np.random.default_rng(page_size)
+    H, hs, total, new = 2, 32, 333, 40
+    first_allowed = max(0, (total - 1) - window + 1) if window else 0
+    special = sorted({first_allowed, first_allowed + 1, page_size - 1, page_size, 2 * page_size - 1, 2 * page_size, 63, 64, 127, 128,
+                      255, 256, total - 2, total - 1} | ({first_allowed - 1} if window else set()))
+    special = [p for p in special if 0 <= p < total]
+    n_req = len(special)
+    blocks = (total + page_size - 1) // page_size
+    pages = rng.permutation(n_req * blocks).reshape(n_req, blocks).astype(np.int32)
+    kp = torch.zeros((n_req * blocks, H, page_size, hs), device=DEV).to(dtype)
+    vp = torch.zeros_like(kp)
+    q_all, refs, treq, tpos = [], [], [], []
+    for r, hot in enumerate(special):
+        k = bf16_round(rng.standard_normal((total, H * hs)) * 0.1)
+        v = bf16_round(rng.standard_normal((total, H * hs)))
+        q = bf16_round(rng.standard_normal((new, H * hs)) * 0.1)
+        direction = np.tile(np.r_[1.0, np.zeros(hs - 1)], H)
+        q[-1] = direction * 16.0            # the last query looks along one direction ...
+        k[hot] = direction * 16.0           # ... and one key lies along it: its score is 256/sqrt(32) above the rest
+        slots = np.array([pages[r, p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+        K.cache_write(dev(k, dtype), dev(v, dtype), kp, vp, dev(slots, torch.int32), H, hs)
+        q_all.append(q)
+        treq += [r] * new
+        tpos += list(range(total - new, total))
+        refs.append((hot, v))
+    extra = {}
+    if path == "matrix_cores":
+        extra = dict(q_starts=dev(np.arange(n_req + 1) * new, torch.int32), context_lens=dev([total - new] * n_req, torch.int32))
+    out = host(K.paged_attention(
+        dev(np.concatenate(q_all), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(pages, torch.int32),
+        H, H, hs, 1.0 / math.sqrt(hs), window=window, max_q_len={"general": None, "matrix_cores": new}.get(path, 1), **extra))
+    for r, (hot, v) in enumerate(refs):
+        last = out[(r + 1) * new - 1]
+        if hot >= first_allowed:
+            np.testing.assert_allclose(last, v[hot], atol=2e-2, err_msg=f"key {hot} should carry the whole weight")
+        else:
+            assert np.abs(last - v[hot]).max() > 0.2, f"key {hot} lies outside the window and must not count"
