@@ -99,18 +99,26 @@ def multi_head_attention(q, k, v, n_head, n_kv_head=None, window=None):
     return out
 
 
-def block(x, w, n_head, eps, activation):
+def _keep(x):
+    return x
+
+
+def block(x, w, n_head, eps, activation, stored=_keep):
     """Pre-norm block in the reference's order (engine/src/transformer_block.c:49-71):
     ln_1 -> q,k,v (columns of the fused c_attn, engine/src/gpt2.c:79-90) -> attention -> c_proj ->
-    residual add -> ln_2 -> c_fc -> activation -> mlp.c_proj -> residual add."""
+    residual add -> ln_2 -> c_fc -> activation -> mlp.c_proj -> residual add.
+
+    ``stored`` is applied to every tensor a reduced-precision run keeps between kernels (norm
+    outputs, q/k/v, the attention output, the activated MLP row); the residual stream is not one
+    of them. The reference keeps everything in 32-bit, which is the default here."""
     d = x.shape[-1]
-    ln1 = layernorm(x, w["ln_1.weight"], w["ln_1.bias"], eps)
-    qkv = linear(ln1, w["attn.c_attn.weight"], w["attn.c_attn.bias"])
+    ln1 = stored(layernorm(x, w["ln_1.weight"], w["ln_1.bias"], eps))
+    qkv = stored(linear(ln1, w["attn.c_attn.weight"], w["attn.c_attn.bias"]))
     q, k, v = qkv[:, :d], qkv[:, d : 2 * d], qkv[:, 2 * d :]
-    a = multi_head_attention(q, k, v, n_head)
+    a = stored(multi_head_attention(q, k, v, n_head))
     r = x + linear(a, w["attn.c_proj.weight"], w["attn.c_proj.bias"])
-    ln2 = layernorm(r, w["ln_2.weight"], w["ln_2.bias"], eps)
-    u = ACTIVATIONS[activation](linear(ln2, w["mlp.c_fc.weight"], w["mlp.c_fc.bias"]))
+    ln2 = stored(layernorm(r, w["ln_2.weight"], w["ln_2.bias"], eps))
+    u = stored(ACTIVATIONS[activation](linear(ln2, w["mlp.c_fc.weight"], w["mlp.c_fc.bias"])))
     return r + linear(u, w["mlp.c_proj.weight"], w["mlp.c_proj.bias"])
 
 
@@ -122,9 +130,9 @@ def lm_head(x, wte):
 # --------------------------------------------------------------------------------------------
 # whole model
 # --------------------------------------------------------------------------------------------
-def forward(config: dict, weights: dict, tokens, dtype=np.float64):
+def forward(config: dict, weights: dict, tokens, dtype=np.float64, stored=_keep):
     """Logits [len(tokens), vocab] of one whole sequence (engine/src/gpt2.c:198-262): embed,
-    n_layer blocks, ln_f on every row, tied head."""
+    n_layer blocks, ln_f on every row, tied head. ``stored``: see ``block``."""
     w = {name: np.asarray(t, dtype=dtype) for name, t in weights.items()}
     n_layer = config["n_layer"]
     eps = config.get("layer_norm_epsilon", 1e-5)
@@ -135,8 +143,8 @@ def forward(config: dict, weights: dict, tokens, dtype=np.float64):
     for i in range(n_layer):
         prefix = f"h.{i}."
         layer = {k[len(prefix) :]: t for k, t in w.items() if k.startswith(prefix)}
-        h = block(h, layer, config["n_head"], eps, activation)
-    h = layernorm(h, w["ln_f.weight"], w["ln_f.bias"], eps)
+        h = block(h, layer, config["n_head"], eps, activation, stored)
+    h = stored(layernorm(h, w["ln_f.weight"], w["ln_f.bias"], eps))
     return lm_head(h, w["wte.weight"])
 
 
@@ -191,6 +199,16 @@ def f32_to_bf16_rne(x: np.ndarray) -> np.ndarray:
 def round_to_bf16(x: np.ndarray) -> np.ndarray:
     """The float32 value nearest-even rounded to bfloat16 precision."""
     return (f32_to_bf16_rne(x).astype(np.uint32) << 16).view(np.float32).reshape(np.shape(x))
+
+
+def stored_as_bf16(x: np.ndarray) -> np.ndarray:
+    """``stored`` for a bfloat16 run: values rounded to bfloat16, arithmetic type kept."""
+    return round_to_bf16(np.asarray(x, dtype=np.float32)).astype(x.dtype)
+
+
+def bf16_weights(weights: dict) -> dict:
+    """The tensors as a bfloat16 run keeps them: matrices and tables rounded, vectors untouched."""
+    return {k: round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
 
 
 def read_safetensors(path) -> dict:

@@ -12,6 +12,18 @@ import plain_gpt2
 
 ROOT = Path(__file__).resolve().parent.parent
 
+# float32: the engine's own rounding (sums in another order than numpy's) is a few 1e-7 at 128
+# positions and 7e-6 at 600 with sharp attention; the bound leaves a factor of three.
+F32_TOL = dict(atol=2e-5, rtol=2e-5)
+# bfloat16, against the plain implementation storing the same tensors in bfloat16: what is left is
+# single roundings that fall the other way (sums in another order) and what the softmax makes of
+# them; measured 2e-3 to 1.6e-2 on logits up to 2.4.
+BF16_TOL = dict(atol=2.5e-2, rtol=2e-2)
+
+
+def tolerance(dtype: str) -> dict:
+    return F32_TOL if dtype == "float32" else BF16_TOL
+
 
 def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, timeout=600):
     """Runs bin/trace_run over the steps; returns {step: array [wanted, vocab]}."""
@@ -145,8 +157,13 @@ def peak_tokens(collector, page=64):
     return peak
 
 
-def plain_logits(config, weights, requests, dtype=np.float64):
-    return {name: plain_gpt2.forward(config, weights, tokens, dtype) for name, tokens in requests.items()}
+def plain_logits(config, weights, requests, dtype=np.float64, bf16=False):
+    """The plain implementation's logits; ``bf16``: as a bfloat16 run stores tensors (matrices,
+    tables and the activations between kernels rounded to bfloat16, arithmetic in float64)."""
+    if bf16:
+        weights = plain_gpt2.bf16_weights(weights)
+    stored = plain_gpt2.stored_as_bf16 if bf16 else plain_gpt2._keep
+    return {name: plain_gpt2.forward(config, weights, tokens, dtype, stored) for name, tokens in requests.items()}
 
 
 def compare(got, ref, atol, rtol):

@@ -28,11 +28,11 @@ def engines(model_dirs):
     return get
 
 
-def plain_check_greedy(config, weights, prompt, generated, margin):
+def plain_check_greedy(config, weights, prompt, generated, margin, stored=plain_gpt2._keep):
     """Every generated token must be (within margin) the plain implementation's argmax."""
     tokens = list(prompt)
     for token in generated:
-        logits = plain_gpt2.forward(config, weights, tokens)[-1]
+        logits = plain_gpt2.forward(config, weights, tokens, stored=stored)[-1]
         assert logits[token] >= logits.max() - margin, f"token {token} at length {len(tokens)}: {logits[token]} < {logits.max()}"
         tokens.append(token)
 
@@ -49,12 +49,12 @@ def test_greedy_generation_matches_plain_f32(model_dirs, engines):
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_greedy_generation_bf16(model_dirs, engines, name):
     _, config, weights = model_dirs[name]
-    rounded = {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
+    rounded = plain_gpt2.bf16_weights(weights)
     prompts = [random_tokens(1 + i, n, config["vocab_size"]) for i, n in enumerate((5, 17, 33))]
     out = engines(name, "bfloat16").generate(prompts, max_new_tokens=16)
     for prompt, generated in zip(prompts, out):
         assert len(generated) == 16
-        plain_check_greedy(config, rounded, prompt, generated, margin=0.05)
+        plain_check_greedy(config, rounded, prompt, generated, margin=0.03, stored=plain_gpt2.stored_as_bf16)
 
 
 def host_uniform(seed, step, index):
@@ -121,14 +121,17 @@ def test_sessions_and_forward_last(model_dirs, engines):
     _, config, weights = model_dirs["A"]
     engine = engines("A")
     tokens = random_tokens(7, 30, config["vocab_size"])
+    import replay
+
     ref = plain_gpt2.forward(config, weights, tokens)
-    np.testing.assert_allclose(engine.forward_last(tokens), ref[-1], atol=2e-5, rtol=1e-4)
+    tol = replay.F32_TOL
+    np.testing.assert_allclose(engine.forward_last(tokens), ref[-1], **tol)
     with engine.open_session() as session:
-        np.testing.assert_allclose(session.prefill(tokens[:1]), ref[0], atol=2e-5, rtol=1e-4)   # the very first token
-        np.testing.assert_allclose(session.decode(tokens[1]), ref[1], atol=2e-5, rtol=1e-4)
-        np.testing.assert_allclose(session.prefill(tokens[2:20]), ref[19], atol=2e-5, rtol=1e-4)
+        np.testing.assert_allclose(session.prefill(tokens[:1]), ref[0], **tol)   # the very first token
+        np.testing.assert_allclose(session.decode(tokens[1]), ref[1], **tol)
+        np.testing.assert_allclose(session.prefill(tokens[2:20]), ref[19], **tol)
         for i in range(20, 30):
-            np.testing.assert_allclose(session.decode(tokens[i]), ref[i], atol=2e-5, rtol=1e-4)
+            np.testing.assert_allclose(session.decode(tokens[i]), ref[i], **tol)
         assert session.length() == 30
     with pytest.raises(RuntimeError, match="closed"):
         session.decode(1)
@@ -205,10 +208,9 @@ def test_long_decoding_and_page_edges(model_dirs, tmp_path):
     folder, config, weights = model_dirs["C"]
     requests = {"long": random_tokens(40, 580, config["vocab_size"])}
     collector = replay.prefill_then_decode(requests, tail=540)
-    for dtype, tol in (("float32", dict(atol=2e-5, rtol=1e-4)), ("bfloat16", dict(atol=4e-2, rtol=4e-2))):
+    for dtype in ("float32", "bfloat16"):
         got = collector.gather(replay.run_trace(folder, dtype, collector.steps, tmp_path / dtype, 640))
-        w = weights if dtype == "float32" else {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
-        replay.compare(got, replay.plain_logits(config, w, requests), **tol)
+        replay.compare(got, replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16")), **replay.tolerance(dtype))
 
 
 @pytest.mark.parametrize("page_size", [16, 32, 128])
@@ -220,7 +222,7 @@ def test_other_page_sizes(model_dirs, tmp_path, page_size):
     collector = replay.mixed(requests, seed=page_size)
     max_tokens = replay.peak_tokens(collector, page=max(64, page_size))
     got = collector.gather(replay.run_trace(folder, "float32", collector.steps, tmp_path / "o", max_tokens, page_size=page_size))
-    replay.compare(got, replay.plain_logits(config, weights, requests), atol=2e-5, rtol=1e-4)
+    replay.compare(got, replay.plain_logits(config, weights, requests), **replay.F32_TOL)
 
 
 def test_trace_run_refuses_bad_folders(tmp_path, model_dirs):
@@ -253,10 +255,10 @@ def test_graph_replays_match_eager_steps(model_dirs, dtype):
     folder, config, weights = model_dirs["C"]
     vocab = config["vocab_size"]
     seqs = {name: random_tokens(60 + i, n, vocab) for i, (name, n) in enumerate((("a", 150), ("b", 90), ("c", 131), ("d", 70)))}
-    if dtype == "bfloat16":
-        weights = {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
-    ref = {name: plain_gpt2.forward(config, weights, t) for name, t in seqs.items()}
-    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=4e-2, rtol=4e-2)
+    import replay
+
+    ref = replay.plain_logits(config, weights, seqs, bf16=(dtype == "bfloat16"))
+    tol = replay.tolerance(dtype)
     results = {}
     for use_graphs in (True, False):
         engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=8, max_tokens=1024, use_graphs=use_graphs))

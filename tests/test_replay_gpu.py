@@ -11,11 +11,6 @@ from conftest import random_tokens
 
 pytestmark = pytest.mark.gpu
 
-# float32: the engine's own rounding (sums in another order than numpy's) stays below this.
-F32_TOL = dict(atol=2e-5, rtol=1e-4)
-# bfloat16 activations between kernels: 8 bits of fraction on values of order one.
-BF16_TOL = dict(atol=4e-2, rtol=4e-2)
-
 
 def requests_for(name, config):
     vocab, limit = config["vocab_size"], config["n_positions"]
@@ -41,7 +36,5 @@ def test_replay_matches_plain(model_dirs, tmp_path, name, mode, dtype):
     max_tokens = replay.peak_tokens(collector)  # exactly what is needed: pages are used again
     outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", max_tokens)
     got = collector.gather(outputs)
-    if dtype == "bfloat16":
-        weights = {k: plain_gpt2.round_to_bf16(v) if v.ndim == 2 else v for k, v in weights.items()}
-    ref = replay.plain_logits(config, weights, requests)
-    replay.compare(got, ref, **(F32_TOL if dtype == "float32" else BF16_TOL))
+    ref = replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16"))
+    replay.compare(got, ref, **replay.tolerance(dtype))
