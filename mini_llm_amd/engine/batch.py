@@ -252,12 +252,3 @@ class DecodeBatchBuilder:
             q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], token_sources=views[7],
             groups=groups, request_ids=[e.request_id for e in entries], host={},
         )
-
-
-def padded_size(cache, capacity: int) -> int:
-    """int32 elements of a batch laid out for ``capacity`` tokens and requests."""
-    table_width = cache.max_blocks()
-    lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
-    for _ in cache.groups:
-        lengths += [capacity * table_width, capacity]
-    return sum(_aligned(n) for n in lengths)

@@ -13,12 +13,11 @@ from dataclasses import dataclass
 
 import numpy as np
 
-from ..cache import OutOfPages
 from ..sampling import SamplingParams
 from .batch import StepEntry
 from .loading import DEFAULT_PAGE_SIZE, load_model, make_cache, random_model
 from .scheduler import Request, Scheduler
-from .step import ModelRunner, StepError
+from .step import ModelRunner
 
 
 @dataclass(frozen=True)

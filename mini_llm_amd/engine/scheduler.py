@@ -29,7 +29,6 @@ import threading
 from dataclasses import dataclass, field
 from typing import Callable, Literal, Protocol
 
-from ..cache import OutOfPages
 from ..sampling import SamplingParams
 from .batch import StepEntry
 

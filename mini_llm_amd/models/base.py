@@ -8,7 +8,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-from ..parts.base import Block, LayerContext, Norm, Part, PositionEncoding
+from ..parts.base import Norm, Part, PositionEncoding
 from ..parts.embedding import TokenEmbedding
 
 
