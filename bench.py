@@ -143,6 +143,42 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
 
 
+def measure_peaks():
+    """What this machine reaches with nothing in the way: a pure read of 1 GiB, and the matrix
+    cores with operands in registers (the library's two probes)."""
+    import ctypes
+
+    import torch
+
+    from mini_llm_amd.ops.library import check, library
+
+    lib = library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    n_bytes = 1 << 30
+    buffer = torch.zeros(n_bytes // 4, dtype=torch.float32, device="cuda:0")
+    blocks, iterations = 2048, 20000
+    out = torch.zeros(blocks * 256, dtype=torch.float32, device="cuda:0")
+
+    def timed(fn, reps=3):
+        fn()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = float("inf")
+        for _ in range(reps):
+            start.record()
+            fn()
+            stop.record()
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(stop) / 1e3)
+        return best
+
+    read_s = timed(lambda: check(lib.mllm_probe_read(ctypes.c_void_p(buffer.data_ptr()), n_bytes, ctypes.c_void_p(out.data_ptr()), 4096, stream)))
+    result = {"hbm_read_GBs": round(n_bytes / read_s / 1e9, 1)}
+    for name, code, flops in (("bf16", 1, 32768.0), ("fp32", 0, 4096.0)):
+        s = timed(lambda: check(lib.mllm_probe_mfma(ctypes.c_void_p(out.data_ptr()), blocks, iterations, code, stream)))
+        result[f"mfma_{name}_TFLOPs"] = round(blocks * 4 * iterations * 4 * flops / s / 1e12, 1)
+    return result
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -153,10 +189,15 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
+    parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})")
         return 2
+
+    if args.peaks:
+        print(json.dumps({"measured_peaks": measure_peaks(), "published": {"hbm_GBs": HBM_GBS, "mfma_bf16_TFLOPs": 2500.0, "mfma_fp32_TFLOPs": 157.3}}))
+        return 0
 
     from mini_llm_amd.config import config_from_dict
     from mini_llm_amd.engine.engine import Engine, EngineOptions

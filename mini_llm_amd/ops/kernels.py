@@ -128,6 +128,19 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
     return out
 
 
+def convert(src, dtype, transpose=False):
+    """A 1-D or 2-D float32/bfloat16 tensor in another element type, a 2-D one transposed on request
+    (contiguous result). Load-time work on weights."""
+    _device_tensor(src, "src")
+    _require(src.dim() in (1, 2), "convert takes vectors and matrices")
+    rows, cols = (1, src.shape[0]) if src.dim() == 1 else src.shape
+    _require(not transpose or src.dim() == 2, "only a matrix can be transposed")
+    shape = src.shape if not transpose else (cols, rows)
+    out = torch.empty(tuple(shape), dtype=dtype, device=src.device)
+    check(library().mllm_convert(_ptr(src), _ptr(out), rows, cols, _code(src.dtype), _code(dtype), int(bool(transpose)), _stream()))
+    return out
+
+
 def _check_pages(k_pages, v_pages, n_kv_heads, head_size):
     _device_tensor(k_pages, "k_pages", dim=4)
     _device_tensor(v_pages, "v_pages", k_pages.dtype, 4)

@@ -20,6 +20,9 @@ _SIGNATURES = {
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_gemm_qkv_cache": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_convert": [P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_probe_read": [P, c_longlong, P, c_int, P],
+    "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],

@@ -68,13 +68,18 @@ def place(tensor: torch.Tensor, spec: TensorSpec, precision, device) -> torch.Te
     32-bit is only narrowed if it is a matrix or a table of a bfloat16 run."""
     tensor = tensor.to(device)
     if spec.role == INT_TABLE:
-        tensor = tensor.to(torch.int32)
-    elif spec.role == VECTOR:
-        tensor = tensor.to(precision.vector)
+        return tensor.to(torch.int32).contiguous()
+    if spec.role == VECTOR:
+        target = precision.vector
     elif spec.role in (MATRIX, TABLE):
-        tensor = tensor.to(precision.compute)
+        target = precision.compute
     else:
         raise ValueError(f"unknown tensor role {spec.role!r}")
+    if tensor.is_cuda and tensor.dtype in (torch.float32, torch.bfloat16) and tensor.dim() in (1, 2):
+        from ..ops import kernels  # on the GPU the conversion and the transpose are this framework's kernel
+
+        return kernels.convert(tensor.contiguous(), target, transpose=spec.keep_transposed)
+    tensor = tensor.to(target)  # other stored types (F16, F64) and host-only checks of the loader
     if spec.keep_transposed:
         tensor = tensor.t()
     return tensor.contiguous()

@@ -378,3 +378,17 @@ def test_attention_picks_out_single_keys(K, path, dtype, page_size, window):
             np.testing.assert_allclose(last, v[hot], atol=2e-2, err_msg=f"key {hot} should carry the whole weight")
         else:
             assert np.abs(last - v[hot]).max() > 0.2, f"key {hot} lies outside the window and must not count"
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (33, 65), (96, 288), (1000, 96), (31, 32)])
+@pytest.mark.parametrize("src,dst", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float32, torch.float32)])
+def test_convert_and_transpose(K, rows, cols, src, dst):
+    rng = np.random.default_rng(rows + cols)
+    a = rng.standard_normal((rows, cols)).astype(np.float32)
+    t = dev(a, src)
+    ref = host(t) if dst == torch.float32 else bf16_round(host(t))
+    np.testing.assert_array_equal(host(K.convert(t, dst)), ref)
+    out = K.convert(t, dst, transpose=True)
+    assert tuple(out.shape) == (cols, rows) and out.is_contiguous()
+    np.testing.assert_array_equal(host(out), ref.T)
+    np.testing.assert_array_equal(host(K.convert(t[0].contiguous(), dst)), ref[0])
