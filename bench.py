@@ -143,6 +143,51 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
 
 
+MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
+
+
+def measure_serving(dtype: str, temperature: float):
+    """Continuous batching through the scheduler: 64 concurrent requests on the GPT-2 medium shape,
+    prompts of 32 to 768 uniform-random ids, 256 new tokens each, prompts cut into portions under a
+    budget of 512 tokens a step and run beside the decodes."""
+    import numpy as np
+    import torch
+
+    from mini_llm_amd.config import config_from_dict
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.scheduler import Request
+    from mini_llm_amd.sampling import SamplingParams
+
+    config = config_from_dict(MEDIUM)
+    engine = Engine.from_random(config, 6, EngineOptions(dtype=dtype, max_sessions=64, max_tokens=64 * CONTEXT, max_tokens_per_step=512))
+    rng = np.random.default_rng(6)
+    prompts = [rng.integers(0, config.vocab_size, int(n)).tolist() for n in rng.integers(32, 769, 64)]
+    counts = [0] * len(prompts)
+
+    def run_once():
+        for i, prompt in enumerate(prompts):
+            def emit(token, finish, i=i):
+                counts[i] += 1
+            engine.submit(Request(prompt, 256, None, emit, lambda message: None, SamplingParams(temperature=temperature, seed=i)))
+        torch.cuda.synchronize()
+        begin = time.perf_counter()
+        engine.scheduler.run_until_idle()
+        torch.cuda.synchronize()
+        return time.perf_counter() - begin
+
+    run_once()  # warm-up: captures the decode graphs
+    for i in range(len(counts)):
+        counts[i] = 0
+    before = engine.stats()
+    seconds = run_once()
+    after = engine.stats()
+    generated, prompt_tokens = sum(counts), sum(len(p) for p in prompts)
+    return {"model": "gpt2-medium shape", "dtype": dtype, "requests": len(prompts), "prompt_tokens": prompt_tokens,
+            "generated_tokens": generated, "seconds": round(seconds, 3), "generated_tokens_per_s": round(generated / seconds, 1),
+            "all_tokens_per_s": round((generated + prompt_tokens) / seconds, 1), "steps": after["steps"] - before["steps"],
+            "temperature": temperature, "preemptions": after["preemptions"] - before["preemptions"]}
+
+
 def measure_peaks():
     """What this machine reaches with nothing in the way: a pure read of 1 GiB, and the matrix
     cores with operands in registers (the library's two probes)."""
@@ -189,6 +234,8 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
+    parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
+    parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -197,6 +244,10 @@ def main() -> int:
 
     if args.peaks:
         print(json.dumps({"measured_peaks": measure_peaks(), "published": {"hbm_GBs": HBM_GBS, "mfma_bf16_TFLOPs": 2500.0, "mfma_fp32_TFLOPs": 157.3}}))
+        return 0
+
+    if args.serving:
+        print(json.dumps({"serving": measure_serving(args.dtype, args.temperature)}))
         return 0
 
     from mini_llm_amd.config import config_from_dict

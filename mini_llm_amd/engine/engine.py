@@ -64,8 +64,11 @@ class _Executor:
     def length(self, request_id):
         return self._engine.cache.length(("scheduled", request_id))
 
-    def fits(self, wanted):
-        return self._engine.cache.can_reserve([(("scheduled", r), n) for r, n in wanted])
+    def pages_needed(self, request_id, n_new):
+        return self._engine.cache.pages_needed(("scheduled", request_id), n_new)
+
+    def free_pages(self):
+        return self._engine.cache.free_pages()
 
     def run(self, entries, sampling, steps):
         entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want, e.from_slot) for e in entries]

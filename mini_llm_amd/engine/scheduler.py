@@ -48,11 +48,12 @@ class StepExecutor(Protocol):
     def open(self, request_id) -> None: ...
     def close(self, request_id) -> None: ...
     def length(self, request_id) -> int: ...
-    def fits(self, wanted: list) -> bool: ...                        # [(request_id, n_new)] all at once
+    def pages_needed(self, request_id, n_new: int) -> list[int]: ...  # per layer group, for its next n_new tokens
+    def free_pages(self) -> list[int]: ...                            # per layer group
     def run(self, entries: list, sampling: list, steps: list) -> list[int]: ...
 
 
-@dataclass
+@dataclass(eq=False)
 class Request:
     """The reference's Request (scheduler.py:41-53) plus how to sample."""
 
@@ -69,7 +70,7 @@ class Request:
         self.cancelled = True
 
 
-@dataclass
+@dataclass(eq=False)  # compared by identity: membership tests must not walk every field
 class _Running:
     request: Request
     request_id: int
@@ -79,6 +80,20 @@ class _Running:
     prompt_len: int = 0        # of the original prompt (a preempted request's recompute does not count)
     order: int = 0             # admission order; the largest is preempted first
     finished: bool = False
+
+
+class _PagePlan:
+    """Pages the step being planned has claimed so far, against what is free, per layer group."""
+
+    def __init__(self, free):
+        self.free = list(free)
+        self.taken = [0] * len(self.free)
+
+    def fits(self, need) -> bool:
+        return all(t + n <= f for t, n, f in zip(self.taken, need, self.free))
+
+    def take(self, need) -> None:
+        self.taken = [t + n for t, n in zip(self.taken, need)]
 
 
 class Scheduler:
@@ -172,15 +187,19 @@ class Scheduler:
             self._executor.close(running.request_id)
             self._running.remove(running)
 
-    def _portion_that_fits(self, running: _Running, wanted_so_far: list, most: int) -> int:
-        """The largest portion <= most whose pages can be had beside what is planned already."""
+    def _portion_that_fits(self, running: _Running, plan: "_PagePlan", most: int):
+        """(n, pages): the largest portion n <= most whose pages can be had beside what is planned
+        already, and those pages per group; n = 0 if not even one token fits."""
         n = most
-        while n >= 1 and not self._executor.fits(wanted_so_far + [(running.request_id, n)]):
+        while n >= 1:
+            need = self._executor.pages_needed(running.request_id, n)
+            if plan.fits(need):
+                return n, need
             # shrink to the end of the page before the last one the portion touches
             length = self._executor.length(running.request_id)
             page = self._executor.page_size
             n = min(n - 1, ((length + n - 1) // page) * page - length)
-        return max(n, 0)
+        return 0, None
 
     def _preempt(self, victim: _Running) -> None:
         """The victim gives everything back and waits at the front of the queue; what it has been
@@ -194,7 +213,8 @@ class Scheduler:
             self._waiting.appendleft(victim)
 
     def _plan(self):
-        entries, owners, wanted = [], [], []
+        entries, owners = [], []
+        plan = _PagePlan(self._executor.free_pages())
         budget = self._budget
         preempted = False
         # Running requests first, in admission order: decodes bring one token, prompts a portion.
@@ -206,7 +226,7 @@ class Scheduler:
             if budget < 1:
                 break
             most = min(len(running.pending), budget)
-            n = self._portion_that_fits(running, wanted, most)
+            n, need = self._portion_that_fits(running, plan, most)
             while n == 0:
                 victim = max(self._running, key=lambda r: r.order)
                 preempted = True
@@ -220,10 +240,11 @@ class Scheduler:
                         self._preempt(running)
                     break
                 self._preempt(victim)
-                n = self._portion_that_fits(running, wanted, most)
+                plan.free = self._executor.free_pages()
+                n, need = self._portion_that_fits(running, plan, most)
             if n == 0:
                 continue
-            self._add_entry(entries, owners, wanted, running, n)
+            self._add_entry(entries, owners, plan, running, n, need)
             budget -= n
         # Then admissions, in arrival order; the head of the queue is never overtaken. None in a
         # step that had to preempt: the preempted request would come straight back.
@@ -234,25 +255,25 @@ class Scheduler:
             item = self._pop_waiting()
             if item is None:
                 break
-            running = self._admit(item, wanted, budget)
+            running = self._admit(item, plan, bool(entries))
             if running is None:
                 continue          # cancelled or failed: the next one gets its turn
             if running is False:
                 self._push_front(item)
                 break             # no room yet: wait for a running request to end
-            n = self._portion_that_fits(running, wanted, min(len(running.pending), budget))
-            self._add_entry(entries, owners, wanted, running, n)
+            n, need = self._portion_that_fits(running, plan, min(len(running.pending), budget))
+            self._add_entry(entries, owners, plan, running, n, need)
             budget -= n
             admitted += 1
         return entries, owners
 
-    def _add_entry(self, entries, owners, wanted, running, n) -> None:
+    def _add_entry(self, entries, owners, plan, running, n, need) -> None:
         completes = n == len(running.pending)
         entries.append(StepEntry(running.request_id, list(running.pending[:n]), [n - 1] if completes else []))
         owners.append(running)
-        wanted.append((running.request_id, n))
+        plan.take(need)
 
-    def _admit(self, item, wanted, budget):
+    def _admit(self, item, plan, others_planned: bool):
         """None: the request is gone (cancelled / failed). False: no room now. Else the _Running."""
         request = item.request if isinstance(item, _Running) else item
         if request.cancelled:
@@ -275,9 +296,9 @@ class Scheduler:
         self._executor.open(request_id)
         # Admitted only if its whole prompt has room beside what is planned: a request that could
         # take a first portion and then stall would only be preempted again.
-        if not self._executor.fits(wanted + [(request_id, len(running.pending))]):
+        if not plan.fits(self._executor.pages_needed(request_id, len(running.pending))):
             self._executor.close(request_id)
-            if not self._running and not wanted:
+            if not self._running and not others_planned:
                 request.fail("the request needs more cache pages than the pool has")
                 return None
             return False

@@ -43,11 +43,17 @@ def _device_tensor(t: torch.Tensor, name: str, dtype=None, dim=None) -> None:
 
 
 def _ptr(t: torch.Tensor | None):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    return None if t is None else t.data_ptr()  # ctypes turns the integer into the pointer argument
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    """The raw handle of torch's current stream (also the capturing one inside a graph capture)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
 def embed(tokens, positions, wte, wpe, out=None):

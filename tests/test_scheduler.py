@@ -47,8 +47,11 @@ class FakeExecutor:
     def length(self, request_id):
         return self.cache.length(request_id)
 
-    def fits(self, wanted):
-        return self.cache.can_reserve(wanted)
+    def pages_needed(self, request_id, n_new):
+        return self.cache.pages_needed(request_id, n_new)
+
+    def free_pages(self):
+        return self.cache.free_pages()
 
     def run(self, entries, sampling, steps):
         if self.fail_next_run:
