@@ -6,6 +6,7 @@
 // all), which after cache_write include the tokens of its own step: decoding and prompt
 // portions are the same kernel.
 #include "common.h"
+#include "key_sweep.h"
 
 namespace {
 
@@ -175,21 +176,6 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-template <typename T>
-struct Chunk;  // 16 bytes of a row
-template <>
-struct Chunk<float> {
-    static constexpr int VEC = 4;
-    typedef f32x4 Raw;
-    static __device__ __forceinline__ float get(const Raw& r, int i) { return r[i]; }
-};
-template <>
-struct Chunk<bf16_t> {
-    static constexpr int VEC = 8;
-    typedef bf16x8 Raw;
-    static __device__ __forceinline__ float get(const Raw& r, int i) { return static_cast<float>(r[i]); }
-};
-
 constexpr int DECODE_MAX_SPLITS = 16;
 
 // A block per (token, head); its waves (blockDim.x / 64 of them, a power of two up to 16) split
@@ -201,12 +187,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
     int page_shift, int window, float scale) {
-    constexpr int VEC = Chunk<T>::VEC;
-    constexpr int LPR = HD / VEC;          // lanes that share a row
-    constexpr int RPI = WAVE / LPR;        // rows one load instruction covers
-    constexpr int UNROLL = 8;
-    constexpr int KPI = RPI * UNROLL;      // keys per iteration
-    static_assert(HD % VEC == 0 && (LPR & (LPR - 1)) == 0 && LPR <= WAVE, "head size must be a power of two");
+    constexpr int VEC = KeySweep<T, HD>::VEC, LPR = KeySweep<T, HD>::LPR, RPI = KeySweep<T, HD>::RPI;
     __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
 
     const int lane = threadIdx.x % WAVE, split = threadIdx.x / WAVE, n_splits = blockDim.x / WAVE;
@@ -223,74 +204,24 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const int chunk = (((n_keys + n_splits - 1) / n_splits + RPI - 1) / RPI) * RPI;  // keys per wave
     const int begin = first_key + split * chunk;
     const int end = min(position + 1, begin + chunk);  // exclusive
-    const int sub = lane % LPR, group = lane / LPR;
+    const int sub = lane % LPR;
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
-    const int page_mask = (1 << page_shift) - 1;
 
-    typedef typename Chunk<T>::Raw Raw;
-    float o[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; i++) o[i] = 0.0f;
-    float running_max = -INFINITY, running_sum = 0.0f;  // the sum is this lane's share
-
+    KeySweep<T, HD> sweep;
+    sweep.init();
     if (begin < end) {
         float qf[VEC];
         {
-            Raw raw = *reinterpret_cast<const Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
+            typename Chunk<T>::Raw raw = *reinterpret_cast<const typename Chunk<T>::Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
 #pragma unroll
             for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
         }
-        for (int base = begin; base < end; base += KPI) {
-            Raw kf[UNROLL], vf[UNROLL];  // kept as loaded: converted where they are used
-            bool valid[UNROLL];
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                int key = base + u * RPI + group;
-                valid[u] = key < end;
-                // unconditional loads from a clamped key: no branch between them, all in flight together
-                int safe_key = min(key, end - 1);
-                int page = table[safe_key >> page_shift];
-                size_t row = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask));
-                kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
-                vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
-            }
-            float score[UNROLL];
-            float tile_max = -INFINITY;
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                float dot = 0.0f;
-#pragma unroll
-                for (int i = 0; i < VEC; i++) dot += qf[i] * Chunk<T>::get(kf[u], i);
-#pragma unroll
-                for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
-                score[u] = valid[u] ? dot : -INFINITY;
-                tile_max = fmaxf(tile_max, score[u]);
-            }
-#pragma unroll
-            for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
-            float new_max = fmaxf(running_max, tile_max);  // finite: the first key of the tile is valid
-            float rescale = expf(running_max - new_max);
-            running_sum *= rescale;
-#pragma unroll
-            for (int i = 0; i < VEC; i++) o[i] *= rescale;
-#pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                float p = valid[u] ? expf(score[u] - new_max) : 0.0f;
-                running_sum += p;
-#pragma unroll
-                for (int i = 0; i < VEC; i++) o[i] += p * Chunk<T>::get(vf[u], i);
-            }
-            running_max = new_max;
-        }
-        // every lane of a row group counted the same keys: merge across the groups only
-#pragma unroll
-        for (int offset = LPR; offset < WAVE; offset <<= 1) {
-            running_sum += __shfl_xor(running_sum, offset, WAVE);
-#pragma unroll
-            for (int i = 0; i < VEC; i++) o[i] += __shfl_xor(o[i], offset, WAVE);
-        }
+        sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin, end, lane);
     }
+    sweep.merge_groups();
+    const float* o = sweep.o;
+    const float running_max = sweep.running_max, running_sum = sweep.running_sum;
     if (lane < LPR) {
 #pragma unroll
         for (int i = 0; i < VEC; i++) partial[split][sub * VEC + i] = o[i];

@@ -1,0 +1,148 @@
+// One wave's pass over a run of cached keys of one request and head, shared by the kernels that
+// decode: scores, online softmax in 32-bit and the unnormalised value sum.
+//
+// The rows of one head inside a page lie together, so a wave reads them as one contiguous
+// stream: each lane loads 16 bytes, LPR = head bytes / 16 lanes share a row, and one load
+// instruction covers RPI = 64 / LPR consecutive keys. A lane therefore holds VEC head dimensions
+// (those from sub * VEC on, sub = lane % LPR) of several keys; dot products are finished with
+// shuffles inside the LPR lanes, and the value sums stay per lane until merge_groups().
+#pragma once
+
+#include "common.h"
+
+template <typename T>
+struct Chunk;  // 16 bytes of a row
+template <>
+struct Chunk<float> {
+    static constexpr int VEC = 4;
+    typedef f32x4 Raw;
+    static __device__ __forceinline__ float get(const Raw& r, int i) { return r[i]; }
+};
+template <>
+struct Chunk<bf16_t> {
+    static constexpr int VEC = 8;
+    typedef bf16x8 Raw;
+    static __device__ __forceinline__ float get(const Raw& r, int i) { return static_cast<float>(r[i]); }
+};
+
+template <typename T, int HD>
+struct KeySweep {
+    static constexpr int VEC = Chunk<T>::VEC;
+    static constexpr int LPR = HD / VEC;      // lanes that share a row
+    static constexpr int RPI = WAVE / LPR;    // rows one load instruction covers
+    static constexpr int UNROLL = 8;
+    static constexpr int KPI = RPI * UNROLL;  // keys per iteration
+    static_assert(HD % VEC == 0 && (LPR & (LPR - 1)) == 0 && LPR <= WAVE, "head size must be a power of two");
+    typedef typename Chunk<T>::Raw Raw;
+
+    float o[VEC];         // this lane's share of sum p * v, dimensions sub * VEC ..
+    float running_max;    // the same in every lane
+    float running_sum;    // this lane's share until merge_groups()
+
+    __device__ __forceinline__ void init() {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] = 0.0f;
+        running_max = -INFINITY;
+        running_sum = 0.0f;
+    }
+
+    // KPI keys as loaded: converted where they are used.
+    struct Fetched {
+        Raw kf[UNROLL], vf[UNROLL];
+    };
+
+    // Asks for the keys base .. base+KPI-1 of the request whose block table is given, those from
+    // `end` on replaced by `spare_key` (any key whose page the table holds). No branch between the
+    // loads: all are in flight together, and nothing here waits for them. KEYS / VALUES: which of
+    // the two to ask for (a caller short of registers asks for the values later).
+    template <bool KEYS = true, bool VALUES = true>
+    __device__ __forceinline__ void fetch(Fetched& f, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                                          const int* __restrict__ table, int kv_head, int n_kv_heads, int page_shift,
+                                          int base, int end, int spare_key, int lane) const {
+        const int sub = lane % LPR, group = lane / LPR;
+        const int page_mask = (1 << page_shift) - 1;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            int key = base + u * RPI + group;
+            int safe_key = key < end ? key : spare_key;
+            int page = table[safe_key >> page_shift];
+            size_t row = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask));
+            if constexpr (KEYS) f.kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
+            if constexpr (VALUES) f.vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
+        }
+    }
+
+    // Takes the fetched keys base .. min(base+KPI, end)-1 (at least one) into the running softmax.
+    // qf: the lane's VEC dimensions of the query, already scaled.
+    __device__ __forceinline__ void consume(const Fetched& f, const float (&qf)[VEC], int base, int end, int lane) {
+        const int group = lane / LPR;
+        float score[UNROLL];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < VEC; i++) dot += qf[i] * Chunk<T>::get(f.kf[u], i);
+#pragma unroll
+            for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
+            score[u] = base + u * RPI + group < end ? dot : -INFINITY;
+            tile_max = fmaxf(tile_max, score[u]);
+        }
+#pragma unroll
+        for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
+        float new_max = fmaxf(running_max, tile_max);  // finite: the first key of the tile is valid
+        float rescale = expf(running_max - new_max);
+        running_sum *= rescale;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] *= rescale;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            float p = base + u * RPI + group < end ? expf(score[u] - new_max) : 0.0f;
+            running_sum += p;
+#pragma unroll
+            for (int i = 0; i < VEC; i++) o[i] += p * Chunk<T>::get(f.vf[u], i);
+        }
+        running_max = new_max;
+    }
+
+    // Keys begin .. end-1 (begin < end).
+    __device__ __forceinline__ void keys(const float (&qf)[VEC], const T* __restrict__ k_pages,
+                                         const T* __restrict__ v_pages, const int* __restrict__ table,
+                                         int kv_head, int n_kv_heads, int page_shift, int begin, int end, int lane) {
+        for (int base = begin; base < end; base += KPI) {
+            Fetched f;
+            fetch(f, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, base, end, end - 1, lane);
+            consume(f, qf, base, end, lane);
+        }
+    }
+
+    // One more key that is not in the cache: key_row and value_row hold its HD dimensions in
+    // 32-bit (LDS or memory). Counted once, by the lanes of row group 0.
+    __device__ __forceinline__ void one_key(const float (&qf)[VEC], const float* key_row, const float* value_row, int lane) {
+        const int sub = lane % LPR, group = lane / LPR;
+        float dot = 0.0f;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) dot += qf[i] * key_row[sub * VEC + i];
+#pragma unroll
+        for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
+        float new_max = fmaxf(running_max, dot);
+        float rescale = expf(running_max - new_max);
+        running_sum *= rescale;
+        float p = group == 0 ? expf(dot - new_max) : 0.0f;
+        running_sum += p;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) o[i] = o[i] * rescale + p * value_row[sub * VEC + i];
+        running_max = new_max;
+    }
+
+    // Every lane of a row group counted the same keys: the groups' shares are added up, after
+    // which every lane holds the wave's sum and lanes 0..LPR-1 its output.
+    __device__ __forceinline__ void merge_groups() {
+#pragma unroll
+        for (int offset = LPR; offset < WAVE; offset <<= 1) {
+            running_sum += __shfl_xor(running_sum, offset, WAVE);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) o[i] += __shfl_xor(o[i], offset, WAVE);
+        }
+    }
+};

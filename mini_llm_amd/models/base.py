@@ -8,6 +8,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
+from ..ops import kernels
 from ..parts.base import Norm, Part, PositionEncoding
 from ..parts.embedding import TokenEmbedding
 
@@ -105,9 +106,13 @@ class Model(Part):
         returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only."""
         hidden = self.embedding.forward(batch.tokens, batch.positions, self.position_encoding)
         for call in self.schedule:
-            hidden = self.blocks[call.block].forward(hidden, cache.layer_context(batch, call))
+            block = self.blocks[call.block]
+            if not block.takes_pending:
+                hidden = kernels.settle(hidden)
+            hidden = block.forward(hidden, cache.layer_context(batch, call))
         if batch.n_logit_rows == 0:
             return None
+        hidden = kernels.settle(hidden)
         # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
         normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
         return self.head.forward(normed)

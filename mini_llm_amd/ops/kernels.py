@@ -7,7 +7,7 @@ anything here. Kernels run on torch's current stream."""
 
 from __future__ import annotations
 
-import ctypes
+from dataclasses import dataclass
 
 import torch
 
@@ -285,3 +285,124 @@ def resolve_tokens(tokens, sources, token_slots):
     _device_tensor(token_slots, "token_slots", torch.int32, 1)
     _require(sources.shape[0] >= tokens.shape[0], "fewer sources than tokens")
     check(library().mllm_resolve_tokens(_ptr(tokens), _ptr(sources), _ptr(token_slots), tokens.shape[0], _stream()))
+
+
+# -- a whole layer for rows that bring one token each -------------------------------------------------
+@dataclass
+class PendingRows:
+    """Rows of the residual stream whose last sums are not taken yet:
+    base + bias + partials[0] + partials[1] + ... The layer kernels for decoding leave their
+    output products cut into such partial rows and take them up again in the next kernel."""
+
+    base: torch.Tensor             # [rows, width] float32
+    partials: torch.Tensor | None  # [n, rows, width] float32
+    bias: torch.Tensor | None      # [width] float32
+
+    @property
+    def shape(self):
+        return self.base.shape
+
+
+MLP_SLICE_UNITS = 64         # hidden units a block of the feed-forward kernel takes
+LAYER_KERNEL_MAX_ROWS = 0    # rows up to this many take the layer kernels (0: off until they beat the separate kernels)
+
+
+def _pending(hidden):
+    if isinstance(hidden, PendingRows):
+        base, partials, bias = hidden.base, hidden.partials, hidden.bias
+    else:
+        base, partials, bias = hidden, None, None
+    _device_tensor(base, "the stream's rows", torch.float32, 2)
+    rows, width = base.shape
+    if partials is not None:
+        _device_tensor(partials, "the partial rows", torch.float32, 3)
+        _require(tuple(partials.shape[1:]) == (rows, width), "the partial rows do not match the stream")
+    if bias is not None:
+        _device_tensor(bias, "the pending bias", torch.float32, 1)
+        _require(bias.shape[0] == width, "the pending bias does not match the stream")
+    return base, partials, bias, 0 if partials is None else partials.shape[0]
+
+
+def settle(hidden):
+    """The stream as plain float32 rows: a tensor as it is, pending rows with their sums taken."""
+    if not isinstance(hidden, PendingRows):
+        return hidden
+    base, partials, bias, n_partials = _pending(hidden)
+    if n_partials == 0 and bias is None:
+        return base
+    out = torch.empty_like(base)
+    check(library().mllm_pending_sum(_ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(out), base.shape[0], base.shape[1], _stream()))
+    return out
+
+
+def decode_layer_supported(width, head_size=0, page_size=0, inner=0) -> bool:
+    """Whether the layer kernels for decoding take these sizes (0: that size is not asked about)."""
+    return bool(library().mllm_decode_layer_supported(int(width), int(head_size), int(page_size), int(inner)))
+
+
+def _norm_vectors(gamma, beta, width):
+    _device_tensor(gamma, "gamma", torch.float32, 1)
+    _device_tensor(beta, "beta", torch.float32, 1)
+    _require(gamma.shape[0] == width and beta.shape[0] == width, "the norm's vectors do not match the width")
+
+
+def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, k_pages, v_pages, slots, token_request,
+                          positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, write_cache=True):
+    """norm, q/k/v, cache write, attention and output product of a pre-norm layer's first half, for
+    rows that are each the newest token of their request, in one kernel (bfloat16 only).
+
+    ``hidden``: float32 rows or PendingRows. Returns PendingRows: the stream before this half
+    with its sums taken, one partial row per head, and the output product's bias."""
+    base, partials, bias, n_partials = _pending(hidden)
+    rows, width = base.shape
+    _norm_vectors(gamma, beta, width)
+    num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
+    _require(k_pages.dtype == torch.bfloat16, "the layer kernels for decoding are bfloat16 only")
+    _require(decode_layer_supported(width, head_size, page_size), f"no layer kernel for width {width}, head size {head_size}, pages of {page_size}")
+    q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
+    _device_tensor(w_qkv, "w_qkv", torch.bfloat16, 2)
+    _device_tensor(w_out, "w_out", torch.bfloat16, 2)
+    _require(tuple(w_qkv.shape) == (q_width + 2 * kv_width, width), "w_qkv does not match the heads or the width")
+    _require(tuple(w_out.shape) == (width, q_width), "w_out does not match the heads or the width")
+    for t, name, n in ((b_qkv, "b_qkv", q_width + 2 * kv_width), (b_out, "b_out", width)):
+        if t is not None:
+            _device_tensor(t, name, torch.float32, 1)
+            _require(t.shape[0] == n, f"{name} does not match its matrix")
+    for t, name in ((slots, "slots"), (token_request, "token_request"), (positions, "positions")):
+        _device_tensor(t, name, torch.int32, 1)
+        _require(t.shape[0] >= rows, f"{name} has fewer entries than rows")
+    _device_tensor(block_tables, "block_tables", torch.int32, 2)
+    summed = torch.empty_like(base)
+    out = torch.empty((n_heads, rows, width), dtype=torch.float32, device=base.device)
+    check(library().mllm_decode_attention_half(
+        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_qkv),
+        _ptr(b_qkv), _ptr(w_out), _ptr(k_pages), _ptr(v_pages), _ptr(slots), _ptr(token_request), _ptr(positions),
+        _ptr(block_tables), block_tables.shape[1], _ptr(out), rows, width, n_heads, n_kv_heads, head_size, page_size,
+        int(window), float(scale), int(bool(write_cache)), _stream()))
+    return PendingRows(summed, out, b_out)
+
+
+def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activation=None, slice_units=MLP_SLICE_UNITS):
+    """norm, up product, activation and down product of a pre-norm layer's second half in one
+    kernel (bfloat16 matrices). Returns PendingRows: the stream before this half with its sums
+    taken, one partial row per slice of ``slice_units`` hidden units, and the down product's bias."""
+    base, partials, bias, n_partials = _pending(hidden)
+    rows, width = base.shape
+    _norm_vectors(gamma, beta, width)
+    _require(activation in EPILOGUES, f"unknown activation {activation!r}")
+    _device_tensor(w_up, "w_up", torch.bfloat16, 2)
+    _device_tensor(w_down, "w_down", torch.bfloat16, 2)
+    inner = w_up.shape[0]
+    _require(decode_layer_supported(width, inner=inner), f"no layer kernel for width {width} with {inner} hidden units")
+    _require(tuple(w_up.shape) == (inner, width) and tuple(w_down.shape) == (width, inner), "the two matrices do not match the width")
+    for t, name, n in ((b_up, "b_up", inner), (b_down, "b_down", width)):
+        if t is not None:
+            _device_tensor(t, name, torch.float32, 1)
+            _require(t.shape[0] == n, f"{name} does not match its matrix")
+    _require(slice_units in (64, 128), "slices of 64 or 128 hidden units")
+    summed = torch.empty_like(base)
+    out = torch.empty(((inner + slice_units - 1) // slice_units, rows, width), dtype=torch.float32, device=base.device)
+    check(library().mllm_decode_mlp_half(
+        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_up),
+        _ptr(b_up), _ptr(w_down), _ptr(out), rows, width, inner, slice_units, EPILOGUES[activation], _stream()))
+    return PendingRows(summed, out, b_down)

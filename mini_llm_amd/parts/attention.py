@@ -9,9 +9,12 @@ from __future__ import annotations
 
 import math
 
+import torch
+
 from ..ops import kernels
 from .base import KVNeed, LayerContext, Mixer, register_part
 from .linear import Linear
+from .norms import LayerNorm
 
 
 class CausalSelfAttention(Mixer):
@@ -61,6 +64,17 @@ class CausalSelfAttention(Mixer):
             q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens,
         )
         return self.out.forward(mixed, residual=residual)
+
+    def forward_normed(self, hidden, norm, compute_dtype, ctx: LayerContext):
+        # rows that are each the newest token of their request: the whole chain in one kernel
+        if (ctx.batch.max_q_len == 1 and hidden.shape[0] <= kernels.LAYER_KERNEL_MAX_ROWS and isinstance(norm, LayerNorm)
+                and self.qkv.weight.dtype == torch.bfloat16 and ctx.k_pages.dtype == torch.bfloat16
+                and kernels.decode_layer_supported(self.width, self.head_size, ctx.k_pages.shape[2])):
+            return kernels.decode_attention_half(
+                hidden, norm.weight, norm.bias, norm.eps, self.qkv.weight, self.qkv.bias, self.out.weight, self.out.bias,
+                ctx.k_pages, ctx.v_pages, ctx.group.slots, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
+                self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0, write_cache=ctx.write_cache)
+        return super().forward_normed(hidden, norm, compute_dtype, ctx)
 
 
 register_part("mixer", "causal_attention", CausalSelfAttention)

@@ -105,11 +105,27 @@ class Mixer(Part):
         token; what came before is in the cache / the state slot."""
         raise NotImplementedError
 
+    def forward_normed(self, hidden, norm: Norm, compute_dtype, ctx: LayerContext):
+        """norm, then ``forward``, then the residual sum, as one call: a mixer that has a kernel
+        for the whole chain overrides this. ``hidden`` and the result are float32 rows or rows
+        whose last sums are pending (ops.kernels.PendingRows)."""
+        from ..ops import kernels
+
+        hidden = kernels.settle(hidden)
+        return self.forward(norm.forward(hidden, compute_dtype), hidden, ctx)
+
 
 class FeedForward(Part):
     def forward(self, x, residual):
         """x: [rows, width] in the compute dtype; returns residual + f(x) in float32."""
         raise NotImplementedError
+
+    def forward_normed(self, hidden, norm: Norm, compute_dtype, ctx: LayerContext):
+        """norm, then ``forward``, then the residual sum, as one call (see Mixer.forward_normed)."""
+        from ..ops import kernels
+
+        hidden = kernels.settle(hidden)
+        return self.forward(norm.forward(hidden, compute_dtype), hidden)
 
 
 class PositionEncoding(Part):
@@ -120,6 +136,10 @@ class PositionEncoding(Part):
 
 
 class Block(Part):
+    # True if ``forward`` takes and may return rows whose last sums are pending
+    # (ops.kernels.PendingRows); a block that says False always gets plain float32 rows.
+    takes_pending = False
+
     def forward(self, hidden, ctx: LayerContext):
         """hidden: [rows, width] float32 residual stream -> the same after this layer."""
         raise NotImplementedError

@@ -20,9 +20,11 @@ class PreNormBlock(Block):
     def mixer_part(self):
         return self.mixer
 
+    takes_pending = True
+
     def forward(self, hidden, ctx: LayerContext):
-        hidden = self.mixer.forward(self.norm_1.forward(hidden, self.compute_dtype), hidden, ctx)
-        return self.feed_forward.forward(self.norm_2.forward(hidden, self.compute_dtype), hidden)
+        hidden = self.mixer.forward_normed(hidden, self.norm_1, self.compute_dtype, ctx)
+        return self.feed_forward.forward_normed(hidden, self.norm_2, self.compute_dtype, ctx)
 
 
 register_part("block", "pre_norm", PreNormBlock)

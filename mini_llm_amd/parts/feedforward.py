@@ -4,8 +4,12 @@ residual sum into the down product."""
 
 from __future__ import annotations
 
+import torch
+
+from ..ops import kernels
 from .base import FeedForward, register_part
 from .linear import Linear
+from .norms import LayerNorm
 
 ACTIVATIONS = ("gelu_new", "gelu")
 
@@ -25,6 +29,14 @@ class DenseMLP(FeedForward):
 
     def forward(self, x, residual):
         return self.down.forward(self.up.forward(x, activation=self.activation), residual=residual)
+
+    def forward_normed(self, hidden, norm, compute_dtype, ctx):
+        # few rows: the whole chain in one kernel, cut along the hidden units
+        if (hidden.shape[0] <= kernels.LAYER_KERNEL_MAX_ROWS and ctx.batch.max_q_len == 1 and isinstance(norm, LayerNorm)
+                and self.up.weight.dtype == torch.bfloat16 and kernels.decode_layer_supported(self.width, inner=self.inner)):
+            return kernels.decode_mlp_half(hidden, norm.weight, norm.bias, norm.eps, self.up.weight, self.up.bias,
+                                           self.down.weight, self.down.bias, activation=self.activation)
+        return super().forward_normed(hidden, norm, compute_dtype, ctx)
 
 
 register_part("feed_forward", "dense_mlp", DenseMLP)

@@ -392,3 +392,136 @@ def test_convert_and_transpose(K, rows, cols, src, dst):
     assert tuple(out.shape) == (cols, rows) and out.is_contiguous()
     np.testing.assert_array_equal(host(out), ref.T)
     np.testing.assert_array_equal(host(K.convert(t[0].contiguous(), dst)), ref[0])
+
+
+# -- a whole layer for rows that bring one token each ---------------------------------------------------
+def _pending_rows(K, rng, rows, width, n_partials, with_bias):
+    """A stream in pending form and its sum in float64."""
+    base = rng.standard_normal((rows, width)).astype(np.float32)
+    partials = (rng.standard_normal((n_partials, rows, width)) * 0.3).astype(np.float32) if n_partials else None
+    bias = (rng.standard_normal(width) * 0.1).astype(np.float32) if with_bias else None
+    total = base.astype(np.float64)
+    if bias is not None:
+        total = total + bias
+    if partials is not None:
+        total = total + partials.astype(np.float64).sum(axis=0)
+    if partials is None and bias is None:
+        return dev(base), total
+    return K.PendingRows(dev(base), None if partials is None else dev(partials), None if bias is None else dev(bias)), total
+
+
+@pytest.mark.parametrize(
+    "width,n_heads,n_kv_heads,head_size,page_size,window,n_partials,with_bias",
+    [(96, 3, 3, 32, 16, 0, 0, False), (80, 6, 2, 16, 32, 37, 5, True), (768, 12, 12, 64, 64, 0, 48, True),
+     (264, 2, 1, 128, 64, 100, 3, False), (256, 1, 1, 256, 16, 0, 17, True), (2048, 4, 4, 64, 128, 0, 2, True)],
+)
+def test_decode_attention_half(K, width, n_heads, n_kv_heads, head_size, page_size, window, n_partials, with_bias):
+    # norm, q/k/v, cache write, attention over the cache and output product in one kernel, for
+    # rows that are each the newest token of a request, against the same steps one by one in
+    # float64 with bfloat16 kept where the kernel keeps it (normed rows, q, k, v, mixed rows)
+    rng = np.random.default_rng(width + head_size)
+    q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
+    eps = 3e-5
+    contexts = [0, 1, page_size - 1, page_size, 150, 700, -1, 333]  # -1: a padding row
+    rows = len(contexts)
+    hidden, total = _pending_rows(K, rng, rows, width, n_partials, with_bias)
+    gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
+    w_qkv = bf16_round(rng.standard_normal((q_width + 2 * kv_width, width)) * (2.0 / math.sqrt(width)))
+    b_qkv = 0.1 * rng.standard_normal(q_width + 2 * kv_width)
+    w_out = bf16_round(rng.standard_normal((width, q_width)) / math.sqrt(q_width))
+    b_out = 0.1 * rng.standard_normal(width)
+
+    num_pages = sum((c + 1 + page_size - 1) // page_size for c in contexts if c >= 0) + 3
+    order = rng.permutation(num_pages).tolist()
+    kp = torch.full((num_pages, n_kv_heads, page_size, head_size), float("nan"), device=DEV).bfloat16()
+    vp = torch.full_like(kp, float("nan"))
+    max_blocks = max((c + 1 + page_size - 1) // page_size for c in contexts)
+    tables = np.zeros((rows, max_blocks), dtype=np.int32)
+    new_slots, treq, tpos, expected = [], [], [], np.zeros((rows, width))
+    expect_k, expect_v = {}, {}
+    for r, ctx in enumerate(contexts):
+        if ctx < 0:
+            new_slots.append(-1), treq.append(-1), tpos.append(0)
+            continue
+        n_blocks = (ctx + 1 + page_size - 1) // page_size
+        pages = [order.pop() for _ in range(n_blocks)]
+        tables[r, :n_blocks] = pages
+        slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(ctx + 1)], dtype=np.int32)
+        k_all, v_all = bf16_round(rng.standard_normal((ctx + 1, kv_width))), bf16_round(rng.standard_normal((ctx + 1, kv_width)))
+        if ctx:
+            K.cache_write(dev(k_all[:ctx], torch.bfloat16), dev(v_all[:ctx], torch.bfloat16), kp, vp, dev(slots[:ctx], torch.int32), n_kv_heads, head_size)
+        new_slots.append(int(slots[ctx])), treq.append(r), tpos.append(ctx)
+        normed = bf16_round(P.layernorm(total[r : r + 1], gamma, beta, eps))
+        qkv = bf16_round(normed @ w_qkv.T + b_qkv)[0]
+        k_all[ctx], v_all[ctx] = qkv[q_width : q_width + kv_width], qkv[q_width + kv_width :]
+        expect_k[int(slots[ctx])], expect_v[int(slots[ctx])] = k_all[ctx], v_all[ctx]
+        mixed = bf16_round(plain_paged_attention(qkv[None, :q_width], k_all, v_all, n_heads, n_kv_heads, window or None))
+        expected[r] = total[r] + mixed[0] @ w_out.T + b_out
+    k_before, v_before = kp.clone(), vp.clone()
+    out = K.decode_attention_half(
+        hidden, dev(gamma), dev(beta), eps, dev(w_qkv, torch.bfloat16), dev(b_qkv), dev(w_out, torch.bfloat16), dev(b_out), kp, vp,
+        dev(new_slots, torch.int32), dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+        n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window)
+    assert out.partials.shape == (n_heads, rows, width)
+    live = [r for r, c in enumerate(contexts) if c >= 0]
+    np.testing.assert_allclose(host(out.base)[live], total[live], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(K.settle(out))[live], expected[live], rtol=5e-3, atol=5e-3)
+    assert torch.isfinite(K.settle(out)).all()  # the padding row too
+    # the new keys and values are in their slots, rounded to bfloat16; nothing else was written
+    for pages, before, expect in ((kp, k_before, expect_k), (vp, v_before, expect_v)):
+        flat, flat_before = pages.permute(0, 2, 1, 3).reshape(-1, kv_width), before.permute(0, 2, 1, 3).reshape(-1, kv_width)
+        for slot, row in expect.items():
+            np.testing.assert_allclose(host(flat[slot]), row, rtol=1e-2, atol=1e-2)
+            flat_before[slot] = flat[slot]
+        assert torch.equal(flat.view(torch.int16), flat_before.view(torch.int16))
+
+
+def test_decode_attention_half_reads_a_cache_it_does_not_write(K):
+    # write_cache=False: the token's own key and value still count, the pages stay as they were
+    rng = np.random.default_rng(5)
+    width, n_heads, head_size, page_size = 64, 2, 32, 16
+    hidden, total = _pending_rows(K, rng, 1, width, 0, False)
+    kp = torch.zeros((2, n_heads, page_size, head_size), device=DEV).bfloat16()
+    vp = torch.zeros_like(kp)
+    args = (dev(np.ones(width)), dev(np.zeros(width)), 1e-5, dev(rng.standard_normal((3 * width, width)) * 0.2, torch.bfloat16), None,
+            dev(rng.standard_normal((width, width)) * 0.2, torch.bfloat16), None, kp, vp, dev([3], torch.int32), dev([0], torch.int32),
+            dev([3], torch.int32), dev([[0]], torch.int32), n_heads, n_heads, head_size, 0.25)
+    reading = K.settle(K.decode_attention_half(hidden, *args, write_cache=False))
+    assert not kp.any() and not vp.any()
+    writing = K.settle(K.decode_attention_half(hidden, *args, write_cache=True))
+    assert kp.any() and vp.any()
+    assert torch.equal(reading, writing)
+
+
+@pytest.mark.parametrize(
+    "width,inner,rows,activation,slice_units,n_partials,with_bias",
+    [(96, 320, 5, "gelu", 64, 3, True), (768, 3072, 8, "gelu_new", 64, 12, True), (240, 200, 19, "gelu_new", 128, 0, False),
+     (2048, 512, 33, "gelu", 128, 2, False), (1032, 136, 16, None, 64, 5, True), (8, 8, 1, "gelu", 64, 1, False)],
+)
+def test_decode_mlp_half(K, width, inner, rows, activation, slice_units, n_partials, with_bias):
+    rng = np.random.default_rng(width + inner)
+    eps = 1e-6
+    hidden, total = _pending_rows(K, rng, rows, width, n_partials, with_bias)
+    gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
+    w_up, b_up = bf16_round(rng.standard_normal((inner, width)) * (2.0 / math.sqrt(width))), 0.1 * rng.standard_normal(inner)
+    w_down, b_down = bf16_round(rng.standard_normal((width, inner)) / math.sqrt(inner)), 0.1 * rng.standard_normal(width)
+    act = {"gelu": P.gelu_erf, "gelu_new": P.gelu_new, None: lambda x: x}[activation]
+    normed = bf16_round(P.layernorm(total, gamma, beta, eps))
+    expected = total + bf16_round(act(normed @ w_up.T + b_up)) @ w_down.T + b_down
+    out = K.decode_mlp_half(hidden, dev(gamma), dev(beta), eps, dev(w_up, torch.bfloat16), dev(b_up), dev(w_down, torch.bfloat16),
+                            dev(b_down), activation=activation, slice_units=slice_units)
+    assert out.partials.shape == ((inner + slice_units - 1) // slice_units, rows, width)
+    np.testing.assert_allclose(host(out.base), total, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(host(K.settle(out)), expected, rtol=5e-3, atol=5e-3)
+
+
+def test_layer_kernels_refuse_what_they_do_not_take(K):
+    assert K.decode_layer_supported(768, 64, 64, 3072)
+    assert not K.decode_layer_supported(4096)          # wider than a block's threads cover
+    assert not K.decode_layer_supported(100)           # rows that are no multiple of 16 bytes
+    assert not K.decode_layer_supported(96, 48, 16)    # a head size that is no power of two
+    assert not K.decode_layer_supported(96, 32, 24)    # pages that are no power of two
+    x = torch.zeros((1, 96), device=DEV)
+    ones = torch.ones(96, device=DEV)
+    with pytest.raises(K.OperandError):
+        K.decode_mlp_half(x, ones, ones, 1e-5, torch.zeros((100, 96), device=DEV).bfloat16(), None, torch.zeros((96, 100), device=DEV).bfloat16(), None)
