@@ -32,6 +32,21 @@ struct alignas(16) Vec16 {
     uint32_t w[4];
 };
 
+// The packed layout of a weight matrix W [rows, cols]: chunks of 16 rows x 64 bytes (32 bfloat16 or
+// 16 float columns), row tiles outermost, zeros beyond the matrix. Inside a chunk piece p (16
+// bytes) holds row p % 16, columns (p / 16) * VEC .. of the chunk: exactly what lane p of a wave
+// feeds a 16x16 MFMA as its 16-row operand. A wave therefore loads a chunk as 1 KiB of contiguous
+// memory, straight into operand registers; from row-major memory the same load would touch 16
+// cache lines per quarter wave, which the vector cache serves several times slower.
+template <typename T>
+__host__ __device__ __forceinline__ size_t packed_offset(int row_tile, int k_step, int k_steps, int lane) {
+    return (((size_t)row_tile * k_steps + k_step) * 64 + lane) * (16 / sizeof(T));
+}
+template <typename T>
+__host__ __device__ __forceinline__ int packed_k_steps(int cols) {
+    return (cols * (int)sizeof(T) + 63) / 64;
+}
+
 void mllm_set_error(const char* format, ...);
 int mllm_check_launch(const char* what);
 
@@ -63,6 +78,25 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// The sum over a wave without a trip through the LDS crossbar: four steps between neighbours
+// inside rows of 16 lanes (data-parallel primitives: a few cycles each), then the four row sums are
+// read out and added. Every lane gets the result; the order of the additions is fixed.
+template <int CONTROL>
+__device__ __forceinline__ float dpp_moved(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CONTROL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wave_total(float v) {
+    v += dpp_moved<0xB1>(v);   // lanes 1,0,3,2 of each four
+    v += dpp_moved<0x4E>(v);   // lanes 2,3,0,1 of each four
+    v += dpp_moved<0x141>(v);  // the other four of each eight (mirrored)
+    v += dpp_moved<0x140>(v);  // the other eight of each sixteen (mirrored)
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int offset = WAVE / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, WAVE));
@@ -89,4 +123,4 @@ __device__ __forceinline__ float apply_activation(float x) {
     return x;
 }
 
-static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

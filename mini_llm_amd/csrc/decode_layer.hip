@@ -16,8 +16,8 @@
 // depend on the order in which blocks finish.
 //
 // Matrix products run on the matrix cores with W as the 16-row operand, streamed from memory
-// straight into registers (a lane loads 16 bytes of one of 16 rows), and the activations, which
-// are tiny, as the other operand from LDS.
+// straight into registers (the matrices are in the packed layout: a wave's operand is 1 KiB of
+// contiguous memory), and the activations, which are tiny, as the other operand from LDS.
 #include "common.h"
 #include "key_sweep.h"
 
@@ -52,6 +52,13 @@ struct PendingSum {
 
 __device__ __forceinline__ f32x4 load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
 
+// 16 bytes at base + byte_offset, where base is the same in every lane (it then lives in scalar
+// registers) and only the 32-bit offset differs: the address costs a lane one register, not two.
+template <typename V>
+__device__ __forceinline__ V load16(const void* uniform_base, unsigned byte_offset) {
+    return *reinterpret_cast<const V*>(reinterpret_cast<const char*>(uniform_base) + byte_offset);
+}
+
 __device__ __forceinline__ Vec16 mask16(Vec16 v, bool keep) {
     Vec16 out;
 #pragma unroll
@@ -66,20 +73,26 @@ __device__ __forceinline__ void store_bf16x4(bf16_t* at, f32x4 v) {
     *reinterpret_cast<bf16x4*>(at) = packed;
 }
 
-// The block's waves meet once this wave's LDS traffic is done. Unlike __syncthreads() it does not
-// wait for this wave's loads from memory: what was asked for early stays in flight across it. Only
-// LDS carries data between the waves of a block here, so nothing more is needed.
+// The compiler moves loads up as far as it can, across loads the code asks for earlier on purpose,
+// and then runs out of registers: this keeps what is above it above and what is below it below.
+__device__ __forceinline__ void keep_order() { __builtin_amdgcn_sched_barrier(0); }
+
+// The block's waves meet once this wave's LDS traffic is done: what __syncthreads() comes to on
+// this target, spelled out because the kernels below count on it. It does not wait for this wave's
+// loads from memory, so what was asked for early stays in flight across it; and only LDS carries
+// data between the waves of a block here, so nothing more is needed.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // ------------------------------------------------------------------------------------------------
 // norm -> q/k/v -> cache write -> attention over the cache -> this head's share of the output
 // product. grid (n_heads, tokens), 1024 threads in two roles:
 //   waves 0..7  "project": norm, q/k/v product, output product;
-//   waves 8..15 "attend":  ask for their shares of the cached keys and values at once, wait for
-//                          the query, then run the softmax over them.
-// A wave's loads from memory complete in the order they were issued, so a wave that asks for the
-// keys early cannot use anything it asks for later before the keys have come: hence the roles.
-// All 16 waves share the pending sums first (short loads from the cache of the chip).
+//   waves 8..15 "attend":  the pending sums, then their shares of the cached keys and values, asked
+//                          for long before the query exists, then the softmax over them.
+// A wave's loads from memory complete in the order they were issued, and every trip to memory
+// costs microseconds: so each role asks early, in the order of use, for all it will need, and the
+// roles are split so that no wave has to wait for the keys before it can use something else.
+// What the waves exchange goes through LDS, between meetings that both roles pass in step.
 // ------------------------------------------------------------------------------------------------
 constexpr int DL_PROJECT_WAVES = 8, DL_ATTEND_WAVES = DL_WAVES - DL_PROJECT_WAVES;
 constexpr int DL_PROJECT_THREADS = DL_PROJECT_WAVES * WAVE;
@@ -88,8 +101,8 @@ template <int HD>
 __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     PendingSum in, float* __restrict__ summed,  // [tokens, width]: the stream with its sums taken, written by head 0
     const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-    const bf16_t* __restrict__ w_qkv, const float* __restrict__ b_qkv,  // [q_width + 2 kv_width, width]
-    const bf16_t* __restrict__ w_out,                                    // [width, q_width]
+    const bf16_t* __restrict__ w_qkv, const float* __restrict__ b_qkv,  // [q_width + 2 kv_width, width], packed
+    const bf16_t* __restrict__ w_out,                                    // [width, q_width], packed
     bf16_t* __restrict__ k_pages, bf16_t* __restrict__ v_pages, const int* __restrict__ slots,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks,
@@ -99,110 +112,134 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     constexpr int VEC = Sweep::VEC, LPR = Sweep::LPR, RPI = Sweep::RPI, KPI = Sweep::KPI;
     constexpr int ROW_TILES = 3 * HD / 16;
     constexpr int UNITS = (ROW_TILES * DL_KSPLIT + DL_PROJECT_WAVES - 1) / DL_PROJECT_WAVES;  // (tile, k share) pairs a wave owns
-    constexpr int AT_ONCE = UNITS < 3 ? UNITS : 3;  // of which it works on so many at a time,
-    constexpr int ROUND = 18 / AT_ONCE;             // with so many k steps of each in flight
+    constexpr int AT_ONCE = UNITS < 2 ? UNITS : 2;  // of which it works on so many at a time,
+    constexpr int ROUND = 12 / AT_ONCE;             // with so many k steps of each in flight
     constexpr int HD_PAD = (HD + 31) / 32 * 32;
     constexpr int OUT_STEPS = HD_PAD / 32, OUT_GROUP = OUT_STEPS <= 2 ? 12 / OUT_STEPS : (OUT_STEPS <= 4 ? 2 : 1);
     constexpr int ROWS_PER_THREAD = (3 * HD + DL_PROJECT_THREADS - 1) / DL_PROJECT_THREADS;
-    constexpr int MAX_PIECES = DL_MAX_WIDTH / 4;
+    constexpr int MAX_PIECES = DL_MAX_WIDTH / 4, PIECES_PER_LANE = MAX_PIECES / WAVE;
+    constexpr int NEAR_KEYS = DL_ATTEND_WAVES * KPI;  // keys the waves that attend can ask for in one go
 
-    __shared__ f32x4 stage[4][MAX_PIECES];
+    __shared__ f32x4 stage[DL_ATTEND_WAVES][MAX_PIECES];
     __shared__ f32x4 row_lds[MAX_PIECES];
     __shared__ __attribute__((aligned(16))) bf16_t x_hat[DL_MAX_WIDTH];
     __shared__ float qkv_part[DL_KSPLIT][3 * HD];
     __shared__ float qkv_row[3][HD];  // q, k, v of this token and head, rounded as the cache holds them
-    __shared__ float merged[DL_ATTEND_WAVES][HD + 2];
+    __shared__ float merged[DL_WAVES][HD + 2];
     __shared__ __attribute__((aligned(16))) bf16_t mixed[HD_PAD];
 
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);  // the same in every lane: kept in a scalar register
     const bool attends = wave >= DL_PROJECT_WAVES;
+    const int role_wave = attends ? wave - DL_PROJECT_WAVES : wave;
     const int head = blockIdx.x, token = blockIdx.y;
     const int n_pieces = width / 4;
     DL_STAMP(0);
     float* out_row = partial_out + ((size_t)head * n_tokens + token) * width;
     const int request = token_request[token];
-    if (request < 0) {  // a padding row: zeros, so that what follows stays finite
+    const int position = positions[token];
+    const int slot = slots[token];
+    // A padding row (request < 0) leaves zeros, so that what follows stays finite. Each role finds
+    // that out only after it has asked for what does not depend on the request: the wait for the
+    // request then costs nothing. No wave has met another by then, and all of them leave.
+    auto leave_zeros = [&]() {
         for (int c = tid; c < width; c += DL_THREADS) {
             out_row[c] = 0.0f;
             if (head == 0) summed[(size_t)token * width + c] = 0.0f;
         }
-        return;
-    }
-    const int position = positions[token];
-    const int slot = slots[token];
+    };
     const int kv_head = head / (n_heads / n_kv_heads);
     const int q_width = n_heads * HD, kv_width = n_kv_heads * HD;
     const int row16 = lane % 16, quad = lane / 16;
+    const int sub = lane % LPR;
 
-    // ---- the pending sums of this token's row, by all waves: four groups of 256 threads take
-    // every fourth partial row each; the four sums meet in LDS and are added in a fixed order
-    {
-        const int group = tid / 256, piece0 = tid % 256;
-#pragma unroll
-        for (int j = 0; j < MAX_PIECES / 256; j++) {
-            if (256 * j >= n_pieces) break;  // the same for every thread
-            int piece = piece0 + 256 * j;
-            int safe_piece = min(piece, n_pieces - 1);
-            f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (int s0 = group; s0 < in.n_partials; s0 += 4 * 12) {
-                f32x4 part[12];
-#pragma unroll
-                for (int u = 0; u < 12; u++) {
-                    int s = min(s0 + 4 * u, in.n_partials - 1);
-                    part[u] = load4(in.partials + ((size_t)s * in.rows + token) * width + 4 * safe_piece);
-                }
-#pragma unroll
-                for (int u = 0; u < 12; u++)
-                    if (s0 + 4 * u < in.n_partials) sum += part[u];
-            }
-            stage[group][piece] = sum;
-        }
-    }
-
-    // From here on the two roles run apart: each passes the same seven meetings of the waves, so
-    // that a role's registers hold that role's data only.
-    if (attends) {
-        // ---- the waves that attend ask for their shares of the cached keys and values now, and
-        // for nothing else until they have used them
+    // The cached keys first_key .. position-1: the first NEAR_KEYS of them are shared by the waves
+    // that attend, KPI or fewer each, asked for in one go; what a long context has beyond them is
+    // shared by the waves that project, which ask when the q/k/v product has given their registers
+    // back. A wave without keys asks for the token's own slot instead: a page the table holds,
+    // memory that may not be written yet, never counted. (Worked out by each role after its first
+    // loads are under way: it is the first use of the position and would wait for it.)
+    int n_far, begin, end, spare_key;
+    const int* table;
+    auto share_of_keys = [&]() {
         const int first_key = window > 0 ? max(0, position - window + 1) : 0;
         const int n_cached = position - first_key;
-        const int chunk = (((n_cached + DL_ATTEND_WAVES - 1) / DL_ATTEND_WAVES + RPI - 1) / RPI) * RPI;
-        const int begin = first_key + (wave - DL_PROJECT_WAVES) * chunk;
-        const int end = min(position, begin + chunk);
-        const int* table = block_tables + (size_t)request * max_blocks;
-        Sweep sweep;
-        typename Sweep::Fetched fetched;
-        // a wave without keys asks for the token's own slot instead: a page the table holds, never used
-        sweep.fetch(fetched, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin, end, begin < end ? end - 1 : position, lane);
-        DL_STAMP(20);
-        lds_barrier();  // 1
+        const int n_near = min(n_cached, NEAR_KEYS);
+        n_far = n_cached - n_near;
+        const int chunk = attends ? (((n_near + DL_ATTEND_WAVES - 1) / DL_ATTEND_WAVES + RPI - 1) / RPI) * RPI
+                                  : (((n_far + DL_PROJECT_WAVES - 1) / DL_PROJECT_WAVES + RPI - 1) / RPI) * RPI;
+        const int share_first = attends ? first_key : first_key + n_near, share_end = attends ? first_key + n_near : position;
+        begin = share_first + role_wave * chunk;
+        end = min(share_end, begin + chunk);
+        spare_key = begin < end ? end - 1 : position;
+        table = block_tables + (size_t)request * max_blocks;
+    };
+    Sweep sweep;
+
+    if (attends) {
+        // ---- the pending sums of this token's row: wave a takes the partial rows a, a + 8, ..., a
+        // lane the pieces lane, lane + 64, ...; the eight sums meet in LDS
+        {
+            const int pieces_here = (n_pieces + WAVE - 1) / WAVE;  // pieces a lane has: 3 for a width of 768
+            for (int j0 = 0; j0 < pieces_here; j0 += 3) {          // three at a time, six partial rows of each in flight
+                f32x4 sum[3];
+#pragma unroll
+                for (int j = 0; j < 3; j++) sum[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                for (int s0 = role_wave; s0 < in.n_partials; s0 += DL_ATTEND_WAVES * 6) {
+                    f32x4 part[6][3];
+#pragma unroll
+                    for (int u = 0; u < 6; u++) {
+                        const int s = __builtin_amdgcn_readfirstlane(min(s0 + DL_ATTEND_WAVES * u, in.n_partials - 1));
+                        const float* partial_row = in.partials + ((size_t)s * in.rows + token) * width;
+#pragma unroll
+                        for (int j = 0; j < 3; j++) part[u][j] = load16<f32x4>(partial_row, 16 * min(lane + WAVE * (j0 + j), n_pieces - 1));
+                    }
+#pragma unroll
+                    for (int u = 0; u < 6; u++) {
+                        const float counts = s0 + DL_ATTEND_WAVES * u < in.n_partials ? 1.0f : 0.0f;  // times zero, not a branch
+#pragma unroll
+                        for (int j = 0; j < 3; j++) sum[j] += part[u][j] * counts;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 3; j++)
+                    if (lane + WAVE * (j0 + j) < n_pieces) stage[role_wave][lane + WAVE * (j0 + j)] = sum[j];
+            }
+        }
+        if (request < 0) {
+            leave_zeros();
+            return;
+        }
+        share_of_keys();
+        int key_page[Sweep::UNROLL];
+        sweep.look_up(key_page, table, page_shift, begin, end, spare_key, lane);  // the table's answer is under way early
+        lds_barrier();  // 1: the eight sums are in LDS
         lds_barrier();  // 2
         lds_barrier();  // 3
+        // ---- their shares of the cached keys and values, asked for now (the pages are known by
+        // now); they ask for nothing else until they have used them
+        typename Sweep::Fetched fetched;
+        sweep.fetch_rows(fetched, key_page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
+        DL_STAMP(20);
         lds_barrier();  // 4
         lds_barrier();  // 5: q, k, v of this token are in LDS
-        // the waves that attend share the cached keys before this token; the token's own key and
-        // value come from LDS (the first of them)
         DL_STAMP(21);
-        const int sub = lane % LPR;
         float qf[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) qf[i] = qkv_row[0][sub * VEC + i] * scale;
         sweep.init();
-        if (begin < end) {
-            sweep.consume(fetched, qf, begin, end, lane);
-            if (begin + KPI < end)  // a context longer than the first round of every wave covers
-                sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin + KPI, end, lane);
-        }
-        if (wave == DL_PROJECT_WAVES) sweep.one_key(qf, qkv_row[1], qkv_row[2], lane);
+        // not under a condition (a wave without keys counts none): the compiler would move the loads
+        // above down into a conditional block, behind the meetings of the waves
+        sweep.template consume<true>(fetched, qf, begin, end, lane);
+        if (wave == DL_PROJECT_WAVES) sweep.one_key(qf, qkv_row[1], qkv_row[2], lane);  // the token's own key and value, from LDS
         sweep.merge_groups();
         if (lane < LPR) {
 #pragma unroll
-            for (int i = 0; i < VEC; i++) merged[wave - DL_PROJECT_WAVES][sub * VEC + i] = sweep.o[i];
+            for (int i = 0; i < VEC; i++) merged[wave][sub * VEC + i] = sweep.o[i];
         }
         if (lane == 0) {
-            merged[wave - DL_PROJECT_WAVES][HD] = sweep.running_max;
-            merged[wave - DL_PROJECT_WAVES][HD + 1] = sweep.running_sum;
+            merged[wave][HD] = sweep.running_max;
+            merged[wave][HD + 1] = sweep.running_sum;
         }
         DL_STAMP(22);
         lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
@@ -210,147 +247,199 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         return;
     }
 
-    // ---- the waves that project: first what they need of the vectors
+    // ---- the waves that project: what they need of the vectors, and the first round of the
+    // q/k/v matrix, in one trip to memory
     const bool owns = tid < n_pieces;  // threads 0 .. width/4-1 own four columns of the row each
     const int own_piece = min(tid, n_pieces - 1);
     f32x4 row = load4(in.base + (size_t)token * width + 4 * own_piece);
-    if (in.bias) row += load4(in.bias + 4 * own_piece);
+    const f32x4 pending_bias = load4((in.bias ? in.bias : gamma) + 4 * own_piece);  // a vector that is there stands in for one that is not
     const f32x4 gain = load4(gamma + 4 * own_piece), offset = load4(beta + 4 * own_piece);
     float qkv_bias[ROWS_PER_THREAD];
 #pragma unroll
     for (int i = 0; i < ROWS_PER_THREAD; i++) {
         int r = min(tid + DL_PROJECT_THREADS * i, 3 * HD - 1), which = r / HD, within = r % HD;
         int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
-        qkv_bias[i] = b_qkv ? b_qkv[w_row] : 0.0f;
+        qkv_bias[i] = (b_qkv ? b_qkv : gamma)[b_qkv ? w_row : 0];
     }
+    // q, k, v of this head: 3*HD rows of the matrix in tiles of 16, each tile's k range shared by
+    // DL_KSPLIT waves; a wave owns UNITS (tile, share) pairs and works on AT_ONCE of them at a time
+    const int n_steps = (width + 31) / 32;
+    const int steps_per_unit = (n_steps + DL_KSPLIT - 1) / DL_KSPLIT;
+    int w_at[AT_ONCE], part_of[AT_ONCE], tile_of[AT_ONCE];
+    Vec16 w_piece[AT_ONCE][ROUND];
+    auto choose_units = [&](int u0) {
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) {
+            int unit = min(wave + DL_PROJECT_WAVES * (u0 + u), ROW_TILES * DL_KSPLIT - 1);  // beyond the last: computed again, not kept
+            tile_of[u] = unit % ROW_TILES, part_of[u] = unit / ROW_TILES;
+            int local = tile_of[u] * 16, which = local / HD, within = local % HD;  // HD is a multiple of 16: a tile lies in one of q, k, v
+            int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
+            w_at[u] = w_row / 16;
+        }
+    };
+    auto ask_for_round = [&](int i0) {
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++)
+#pragma unroll
+            for (int j = 0; j < ROUND; j++) {
+                int step = min(part_of[u] + DL_KSPLIT * (i0 + j), n_steps - 1);
+                w_piece[u][j] = load16<Vec16>(w_qkv + packed_offset<bf16_t>(w_at[u], step, n_steps, 0), lane * 16);
+            }
+    };
+    choose_units(0);
+    ask_for_round(0);
+    if (request < 0) {
+        leave_zeros();
+        return;
+    }
+    share_of_keys();
     DL_STAMP(1);
-    lds_barrier();  // 1: the four groups' sums are in LDS
+    lds_barrier();  // 1: the eight sums of the partial rows are in LDS
+    DL_STAMP(8);
     // width / 4 <= 512: the threads of these waves cover the row
+    row += pending_bias * (in.bias ? 1.0f : 0.0f);
     if (owns) {
-        row += ((stage[0][tid] + stage[1][tid]) + stage[2][tid]) + stage[3][tid];
+        row += ((stage[0][tid] + stage[1][tid]) + (stage[2][tid] + stage[3][tid])) + ((stage[4][tid] + stage[5][tid]) + (stage[6][tid] + stage[7][tid]));
         if (head == 0) *reinterpret_cast<f32x4*>(summed + (size_t)token * width + 4 * tid) = row;
     } else {
         row = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     row_lds[tid] = row;
+    DL_STAMP(9);
     lds_barrier();  // 2: the row with its sums taken is in LDS
+    DL_STAMP(16);
 
     // the norm, centred, in 32-bit: every wave takes the statistics of the whole row for itself (no
     // further meeting of the waves), then norms the four columns it owns
     {
         const float n = (float)width;
-        f32x4 others[MAX_PIECES / WAVE];
+        // the row is read from LDS twice rather than kept: the registers are full of the matrix
+        const int pieces_here = (n_pieces + WAVE - 1) / WAVE;
         float sum = 0.0f;
-#pragma unroll
-        for (int j = 0; j < MAX_PIECES / WAVE; j++) {
-            others[j] = row_lds[lane + WAVE * j];  // zeros beyond the width
-            sum += (others[j][0] + others[j][1]) + (others[j][2] + others[j][3]);
+#pragma unroll 2
+        for (int j = 0; j < pieces_here; j++) {
+            f32x4 piece = row_lds[lane + WAVE * j];  // zeros beyond the width
+            sum += (piece[0] + piece[1]) + (piece[2] + piece[3]);
         }
-        const float mean = wave_sum(sum) / n;
+        const float mean = wave_total(sum) / n;
         float squares = 0.0f;
-#pragma unroll
-        for (int j = 0; j < MAX_PIECES / WAVE; j++) {
-            f32x4 d = lane + WAVE * j < n_pieces ? others[j] - mean : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 2
+        for (int j = 0; j < pieces_here; j++) {
+            f32x4 d = lane + WAVE * j < n_pieces ? row_lds[lane + WAVE * j] - mean : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
             squares += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
         }
-        const float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) / n + eps);
+        const float inverse_stddev = 1.0f / sqrtf(wave_total(squares) / n + eps);
         f32x4 y = (row - mean) * inverse_stddev * gain + offset;
         if (!owns) y = f32x4{0.0f, 0.0f, 0.0f, 0.0f};  // beyond the width: zeros, the products read whole 32-column steps
         store_bf16x4(x_hat + 4 * tid, y);
     }
+    DL_STAMP(17);
     lds_barrier();  // 3: the normed row is in LDS
     DL_STAMP(2);
+    int far_page[Sweep::UNROLL];  // the pages of this wave's share of the far keys (of the spare key, if there are none)
+    sweep.look_up(far_page, table, page_shift, begin, end, spare_key, lane);
 
-    // q, k, v of this head: 3*HD rows of the matrix in tiles of 16, each tile's k range shared by
-    // DL_KSPLIT waves; a wave owns UNITS (tile, share) pairs
-    {
-        const int n_steps = (width + 31) / 32;
-        const int steps_per_unit = (n_steps + DL_KSPLIT - 1) / DL_KSPLIT;
 #pragma unroll 1
-        for (int u0 = 0; u0 < UNITS; u0 += AT_ONCE) {
-            int w_at[AT_ONCE];  // offsets into w_qkv: the matrix has fewer than 2^31 elements
-            int part[AT_ONCE], tile[AT_ONCE];
-            f32x4 acc[AT_ONCE];
+    for (int u0 = 0; u0 < UNITS; u0 += AT_ONCE) {
+        f32x4 acc[AT_ONCE];
 #pragma unroll
-            for (int u = 0; u < AT_ONCE; u++) {
-                int unit = min(wave + DL_PROJECT_WAVES * (u0 + u), ROW_TILES * DL_KSPLIT - 1);  // beyond the last: computed again, not kept
-                tile[u] = unit % ROW_TILES, part[u] = unit / ROW_TILES;
-                int local = tile[u] * 16 + row16, which = local / HD, within = local % HD;
-                int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
-                w_at[u] = w_row * width;
-                acc[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
+        for (int u = 0; u < AT_ONCE; u++) acc[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (u0 > 0) choose_units(u0);
 #pragma unroll 1
-            for (int i0 = 0; i0 < steps_per_unit; i0 += ROUND) {
-                Vec16 w_piece[AT_ONCE][ROUND];
-#pragma unroll
-                for (int u = 0; u < AT_ONCE; u++)
-#pragma unroll
-                    for (int j = 0; j < ROUND; j++) {
-                        int k = (part[u] + DL_KSPLIT * (i0 + j)) * 32 + quad * 8;
-                        w_piece[u][j] = *reinterpret_cast<const Vec16*>(w_qkv + (w_at[u] + min(k, width - 8)));
-                    }
-#pragma unroll
-                for (int u = 0; u < AT_ONCE; u++)
-#pragma unroll
-                    for (int j = 0; j < ROUND; j++) {
-                        int step = part[u] + DL_KSPLIT * (i0 + j);
-                        Vec16 w = mask16(w_piece[u][j], step * 32 + quad * 8 < width);
-                        bf16x8 x = *reinterpret_cast<const bf16x8*>(x_hat + min(step, n_steps - 1) * 32 + quad * 8);
-                        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc[u], 0, 0, 0);
-                    }
-            }
-            // every column of the product is this one token; column 0 is kept
+        for (int i0 = 0; i0 < steps_per_unit; i0 += ROUND) {
+            if (u0 > 0 || i0 > 0) ask_for_round(i0);  // the first round has been under way since the start
 #pragma unroll
             for (int u = 0; u < AT_ONCE; u++)
-                if (row16 == 0 && wave + DL_PROJECT_WAVES * (u0 + u) < ROW_TILES * DL_KSPLIT) {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) qkv_part[part[u]][tile[u] * 16 + 4 * quad + r] = acc[u][r];
+                for (int j = 0; j < ROUND; j++) {
+                    int step = part_of[u] + DL_KSPLIT * (i0 + j);
+                    Vec16 w = mask16(w_piece[u][j], step < n_steps);
+                    bf16x8 x = *reinterpret_cast<const bf16x8*>(x_hat + min(step, n_steps - 1) * 32 + quad * 8);
+                    acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc[u], 0, 0, 0);
                 }
         }
+        // every column of the product is this one token; column 0 is kept
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++)
+            if (row16 == 0 && wave + DL_PROJECT_WAVES * (u0 + u) < ROW_TILES * DL_KSPLIT) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) qkv_part[part_of[u]][tile_of[u] * 16 + 4 * quad + r] = acc[u][r];
+            }
     }
-    // the output product's rows are asked for now, not earlier (the compiler would move these loads
-    // up among the ones above and run out of registers): they are needed last
-    asm volatile("" ::: "memory");
+    auto finish_qkv_rows = [&]() {  // sums of the k shares, bias, rounding; k and v go into their cache slot
+#pragma unroll
+        for (int i = 0; i < ROWS_PER_THREAD; i++) {
+            const int r = tid + DL_PROJECT_THREADS * i;
+            if (r < 3 * HD) {
+                const int which = r / HD, within = r % HD;
+                float value = ((qkv_part[0][r] + qkv_part[1][r]) + qkv_part[2][r]) + qkv_part[3][r] + (b_qkv ? qkv_bias[i] : 0.0f);
+                bf16_t kept = static_cast<bf16_t>(value);
+                qkv_row[which][within] = static_cast<float>(kept);
+                if (which > 0 && write_cache && slot >= 0 && head % (n_heads / n_kv_heads) == 0) {
+                    int page = slot >> page_shift, at = slot & ((1 << page_shift) - 1);
+                    bf16_t* pages = which == 1 ? k_pages : v_pages;
+                    pages[((((size_t)page * n_kv_heads + kv_head) << page_shift) + at) * HD + within] = kept;
+                }
+            }
+        }
+    };
+    DL_STAMP(3);
+    if (n_far > 0) {  // a long context (the same for the whole block): these waves attend to their shares of the far keys
+        typename Sweep::Fetched fetched;
+        sweep.fetch_rows(fetched, far_page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
+        lds_barrier();  // 4: the shares of the q/k/v product are in LDS
+        finish_qkv_rows();
+        lds_barrier();  // 5: q, k, v of this token are in LDS
+        float qf[VEC];
+#pragma unroll
+        for (int i = 0; i < VEC; i++) qf[i] = qkv_row[0][sub * VEC + i] * scale;
+        sweep.init();
+        sweep.template consume<true>(fetched, qf, begin, end, lane);  // not under a further condition, as above
+        if (begin + KPI < end)  // a context longer than one round of every wave of the block covers
+            sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin + KPI, end, lane);
+        sweep.merge_groups();
+    } else {
+        lds_barrier();  // 4
+        finish_qkv_rows();
+        lds_barrier();  // 5
+        sweep.init();
+    }
+    DL_STAMP(4);
+    if (lane < LPR) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) merged[wave][sub * VEC + i] = sweep.o[i];
+    }
+    if (lane == 0) {
+        merged[wave][HD] = sweep.running_max;
+        merged[wave][HD + 1] = sweep.running_sum;
+    }
+    // the output product's rows are asked for now: they are needed last
+    keep_order();
+    // w_out [width, q_width]: this head's columns start in chunk out_step0, at column out_shift of
+    // it (not 0 only for heads of 16, two of which share a chunk of 32 columns)
+    const int out_tiles = (width + 15) / 16, out_k_steps = packed_k_steps<bf16_t>(q_width);
+    const int out_step0 = head * HD / 32, out_shift = head * HD % 32;
     Vec16 out_piece[OUT_GROUP][OUT_STEPS];
 #pragma unroll
     for (int g = 0; g < OUT_GROUP; g++) {
-        int out_col = min((wave + DL_PROJECT_WAVES * g) * 16 + row16, width - 1);
+        int out_tile = min(wave + DL_PROJECT_WAVES * g, out_tiles - 1);
 #pragma unroll
         for (int s = 0; s < OUT_STEPS; s++)
-            out_piece[g][s] = *reinterpret_cast<const Vec16*>(w_out + (size_t)out_col * q_width + head * HD + min(s * 32 + quad * 8, HD - 8));
+            out_piece[g][s] = load16<Vec16>(w_out + packed_offset<bf16_t>(out_tile, out_step0 + s, out_k_steps, 0), lane * 16);
     }
-    DL_STAMP(3);
-    lds_barrier();  // 4: the shares of the q/k/v product are in LDS
-#pragma unroll
-    for (int i = 0; i < ROWS_PER_THREAD; i++) {
-        const int r = tid + DL_PROJECT_THREADS * i;
-        if (r < 3 * HD) {
-            const int which = r / HD, within = r % HD;
-            float value = ((qkv_part[0][r] + qkv_part[1][r]) + qkv_part[2][r]) + qkv_part[3][r] + qkv_bias[i];
-            bf16_t kept = static_cast<bf16_t>(value);
-            qkv_row[which][within] = static_cast<float>(kept);
-            if (which > 0 && write_cache && slot >= 0 && head % (n_heads / n_kv_heads) == 0) {
-                int page = slot >> page_shift, at = slot & ((1 << page_shift) - 1);
-                bf16_t* pages = which == 1 ? k_pages : v_pages;
-                pages[((((size_t)page * n_kv_heads + kv_head) << page_shift) + at) * HD + within] = kept;
-            }
-        }
-    }
-    lds_barrier();  // 5: q, k, v of this token are in LDS
-    DL_STAMP(4);
-    lds_barrier();  // 6: the waves that attend are done
+    lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
     DL_STAMP(5);
-    if (tid < HD_PAD) {  // HD_PAD <= 256 threads
+    if (tid < HD_PAD) {  // HD_PAD <= 256 threads; the mixed row lies where its columns lie in the chunks of w_out, zeros around it
         float value = 0.0f;
-        if (tid < HD) {
+        const int d = tid - out_shift;
+        if (d >= 0 && d < HD) {
             float total_max = -INFINITY;
-            for (int s = 0; s < DL_ATTEND_WAVES; s++) total_max = fmaxf(total_max, merged[s][HD]);
+            for (int s = 0; s < DL_WAVES; s++) total_max = fmaxf(total_max, merged[s][HD]);
             float total = 0.0f;
-            for (int s = 0; s < DL_ATTEND_WAVES; s++) {
+            for (int s = 0; s < DL_WAVES; s++) {
                 float weight = expf(merged[s][HD] - total_max);
                 total += merged[s][HD + 1] * weight;
-                value += merged[s][tid] * weight;
+                value += merged[s][d] * weight;
             }
             value /= total;
         }
@@ -360,31 +449,27 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     DL_STAMP(6);
 
     // this head's share of the output product: rows of w_out in tiles of 16, columns head*HD ..
-    {
-        const int n_tiles = (width + 15) / 16;
-        for (int tile0 = wave; tile0 < n_tiles; tile0 += DL_PROJECT_WAVES * OUT_GROUP) {
-            if (tile0 != wave) {  // wider than the rows asked for above cover
-#pragma unroll
-                for (int g = 0; g < OUT_GROUP; g++) {
-                    int out_col = min((tile0 + DL_PROJECT_WAVES * g) * 16 + row16, width - 1);
-#pragma unroll
-                    for (int s = 0; s < OUT_STEPS; s++)
-                        out_piece[g][s] = *reinterpret_cast<const Vec16*>(w_out + (size_t)out_col * q_width + head * HD + min(s * 32 + quad * 8, HD - 8));
-                }
-            }
+    for (int tile0 = wave; tile0 < out_tiles; tile0 += DL_PROJECT_WAVES * OUT_GROUP) {
+        if (tile0 != wave) {  // wider than the rows asked for above cover
 #pragma unroll
             for (int g = 0; g < OUT_GROUP; g++) {
-                int tile = tile0 + DL_PROJECT_WAVES * g;
-                f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+                int out_tile = min(tile0 + DL_PROJECT_WAVES * g, out_tiles - 1);
 #pragma unroll
-                for (int s = 0; s < OUT_STEPS; s++) {
-                    Vec16 w = mask16(out_piece[g][s], s * 32 + quad * 8 < HD && tile * 16 + row16 < width);
-                    bf16x8 x = *reinterpret_cast<const bf16x8*>(mixed + s * 32 + quad * 8);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc, 0, 0, 0);
-                }
-                int out_col = tile * 16 + 4 * quad;  // 4 columns; the width is a multiple of 4
-                if (row16 == 0 && out_col < width) *reinterpret_cast<f32x4*>(out_row + out_col) = acc;
+                for (int s = 0; s < OUT_STEPS; s++)
+                    out_piece[g][s] = load16<Vec16>(w_out + packed_offset<bf16_t>(out_tile, out_step0 + s, out_k_steps, 0), lane * 16);
             }
+        }
+#pragma unroll
+        for (int g = 0; g < OUT_GROUP; g++) {
+            int tile = tile0 + DL_PROJECT_WAVES * g;
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int s = 0; s < OUT_STEPS; s++) {
+                bf16x8 x = *reinterpret_cast<const bf16x8*>(mixed + s * 32 + quad * 8);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&out_piece[g][s]), x, acc, 0, 0, 0);
+            }
+            int out_col = tile * 16 + 4 * quad;  // 4 columns; the width is a multiple of 4
+            if (row16 == 0 && out_col < width) *reinterpret_cast<f32x4*>(out_row + out_col) = acc;
         }
     }
     DL_STAMP(7);
@@ -392,7 +477,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
 
 // ------------------------------------------------------------------------------------------------
 // norm -> up product -> activation -> this slice's share of the down product.
-// grid (slices of U hidden units, groups of 16 tokens), 1024 threads. The first pieces of both
+// grid (slices of U hidden units, groups of 4, 8 or 16 tokens), 1024 threads. The first pieces of both
 // matrices are asked for at once; while they come, the waves take the pending sums (16 / tokens
 // waves a token, every so-manieth partial row each) and the norm; then all waves run the two
 // products.
@@ -400,15 +485,16 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
 template <int NV, int U>
 __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
     PendingSum in, float* __restrict__ summed, const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
-    const bf16_t* __restrict__ w_up, const float* __restrict__ b_up,  // [inner, width]
-    const bf16_t* __restrict__ w_down,                                 // [width, inner]
+    const bf16_t* __restrict__ w_up, const float* __restrict__ b_up,  // [inner, width], packed
+    const bf16_t* __restrict__ w_down,                                 // [width, inner], packed
     float* __restrict__ partial_out,                                   // [slices, tokens, width]
-    int n_tokens, int width, int inner, int epilogue, int stage_pieces) {
+    int n_tokens, int width, int inner, int epilogue, int stage_pieces, int tokens_per_block) {
     constexpr int TILES = U / 16, K_STEPS_DOWN = U / 32, H_STRIDE = U + 8;
     constexpr int UP_UNITS = (TILES * DL_KSPLIT + DL_WAVES - 1) / DL_WAVES;  // (tile, k share) pairs a wave owns
     constexpr int UP_ROUND = 6 / UP_UNITS;                                   // k steps of each in flight together
     constexpr int DOWN_GROUP = 6 / K_STEPS_DOWN;                             // output tiles a wave works on at a time
-    constexpr int ROWS_AT_ONCE = NV <= 3 ? 4 : (NV <= 4 ? 2 : 1);            // partial rows asked for before any is added
+    constexpr int ROWS_AT_ONCE = NV <= 3 ? 3 : (NV <= 4 ? 2 : 1);                            // partial rows asked for before any is added
+    constexpr int BIAS_PER_THREAD = (TILES * 256 + DL_THREADS - 1) / DL_THREADS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int x_stride = (width + 31) / 32 * 32 + 8;  // 16 bytes of padding: the 16 rows fall on different banks
     bf16_t* x_hat = reinterpret_cast<bf16_t*>(lds);                                          // [16][x_stride]
@@ -418,7 +504,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
 
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
-    const int slice = blockIdx.x, token0 = blockIdx.y * DL_TOKENS;
+    const int slice = blockIdx.x, token0 = blockIdx.y * tokens_per_block;
     const int n_pieces = width / 4;
     const int row16 = lane % 16, quad = lane / 16;
     const int n_steps = (width + 31) / 32;
@@ -430,70 +516,103 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
     // A wave's loads complete in the order they were issued: the first partial rows are asked for
     // first, then the first pieces of both matrices, which stay in flight through all that follows
     // until the products need them.
-    const int tokens_here = min(DL_TOKENS, n_tokens - token0);
+    const int tokens_here = min(tokens_per_block, n_tokens - token0);
     int t2 = 1;
     while (t2 < tokens_here) t2 *= 2;
     if (stage_pieces < n_pieces) t2 = DL_TOKENS;  // no room to share a token's sums among waves
-    const int waves_per_token = DL_WAVES / t2;
-    const int local = wave % t2, sub = wave / t2;
+    const int waves_per_token = __builtin_amdgcn_readfirstlane(DL_WAVES >> (31 - __builtin_clz(t2)));
+    // t2 is a power of two; the scalar unit has no division, and a quotient computed by the vector
+    // unit would drag every address below into vector registers
+    const int local = wave & (t2 - 1), sub = __builtin_amdgcn_readfirstlane(wave >> (31 - __builtin_clz(t2)));
     const int token = token0 + local;
     const bool live = token < n_tokens;
     const int safe_token = live ? token : n_tokens - 1;
-    f32x4 row[NV];
+    // all of a round's loads are asked for before any is used, with no branch between them; the
+    // bias comes from a row of zeros' worth of the base if there is none (and is then not added)
+    f32x4 row[NV], bias_piece[NV];
+    const float* base_row = in.base + (size_t)safe_token * width;
+    const float* bias_row = in.bias ? in.bias : base_row;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         int piece = min(lane + WAVE * j, n_pieces - 1);
-        row[j] = load4(in.base + (size_t)safe_token * width + 4 * piece);
-        if (in.bias) row[j] += load4(in.bias + 4 * piece);
-        if (sub != 0) row[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        row[j] = load16<f32x4>(base_row, 16 * piece);
+        bias_piece[j] = load16<f32x4>(bias_row, 16 * piece);
     }
     f32x4 part[ROWS_AT_ONCE][NV];
     auto ask_for_partial_rows = [&](int s0) {
 #pragma unroll
         for (int u = 0; u < ROWS_AT_ONCE; u++) {
             int s = max(0, min(s0 + waves_per_token * u, in.n_partials - 1));
+            // the row's address is the same in every lane (a scalar), the lanes differ by a 32-bit offset
+            const int partial_index = __builtin_amdgcn_readfirstlane(s * in.rows + safe_token);  // partial rows number fewer than 2^31
+            const float* partial_row = (in.n_partials ? in.partials : in.base) + (size_t)partial_index * width;
 #pragma unroll
-            for (int j = 0; j < NV; j++)
-                part[u][j] = load4((in.n_partials ? in.partials : in.base) + ((size_t)s * in.rows + safe_token) * width + 4 * min(lane + WAVE * j, n_pieces - 1));
+            for (int j = 0; j < NV; j++) part[u][j] = load16<f32x4>(partial_row, 16 * min(lane + WAVE * j, n_pieces - 1));
         }
     };
+    auto add_partial_rows = [&](int s0) {
+#pragma unroll
+        for (int u = 0; u < ROWS_AT_ONCE; u++) {
+            // a row that does not count was asked for again (a finite one): times zero, not a branch,
+            // which would make the compiler wait for every load under way
+            const float counts = s0 + waves_per_token * u < in.n_partials ? 1.0f : 0.0f;
+#pragma unroll
+            for (int j = 0; j < NV; j++) row[j] += part[u][j] * counts;
+        }
+    };
+    const int round_stride = waves_per_token * ROWS_AT_ONCE;
     ask_for_partial_rows(sub);
-
+    const float bias_counts = in.bias ? 1.0f : 0.0f, base_counts = sub == 0 ? 1.0f : 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) row[j] = (row[j] + bias_piece[j] * bias_counts) * base_counts;
+    // the up matrix: behind the partial rows in the order of the loads, so that the sums do not wait for it
     int up_at[UP_UNITS], up_part_of[UP_UNITS], up_tile[UP_UNITS];
-    bool up_valid[UP_UNITS];
     Vec16 up_piece[UP_UNITS][UP_ROUND];
+    float up_bias[BIAS_PER_THREAD];
+    auto ask_for_up_matrix = [&]() {
 #pragma unroll
-    for (int u = 0; u < UP_UNITS; u++) {
-        int unit = min(wave + DL_WAVES * u, TILES * DL_KSPLIT - 1);
-        up_tile[u] = unit % TILES, up_part_of[u] = unit / TILES;
-        int h = slice * U + up_tile[u] * 16 + row16;
-        up_valid[u] = h < inner;
-        up_at[u] = min(h, inner - 1) * width;
+        for (int u = 0; u < UP_UNITS; u++) {
+            int unit = min(wave + DL_WAVES * u, TILES * DL_KSPLIT - 1);
+            up_tile[u] = unit % TILES, up_part_of[u] = unit / TILES;
+            up_at[u] = min(slice * (U / 16) + up_tile[u], (inner + 15) / 16 - 1);  // row tile of w_up; beyond the last: zeros come out below
 #pragma unroll
-        for (int j = 0; j < UP_ROUND; j++) {
-            int k = (up_part_of[u] + DL_KSPLIT * j) * 32 + quad * 8;
-            up_piece[u][j] = *reinterpret_cast<const Vec16*>(w_up + (up_at[u] + min(k, width - 8)));
+            for (int j = 0; j < UP_ROUND; j++)
+                up_piece[u][j] = load16<Vec16>(w_up + packed_offset<bf16_t>(up_at[u], min(up_part_of[u] + DL_KSPLIT * j, n_steps - 1), n_steps, 0), lane * 16);
+        }
+        // and the bias of the hidden units this thread will finish, while nothing waits for it
+#pragma unroll
+        for (int i = 0; i < BIAS_PER_THREAD; i++) {
+            const int index = tid + DL_THREADS * i, tile = index / 256, r = (index / WAVE) % 4, l = index % WAVE;
+            const int h = slice * U + tile * 16 + 4 * (l / 16) + r;
+            up_bias[i] = (b_up ? b_up : gamma)[b_up && h < inner ? h : 0];
+        }
+    };
+    if (sub + round_stride >= in.n_partials) {  // one round of partial rows: the same for the whole wave
+        ask_for_up_matrix();
+        add_partial_rows(sub);
+    } else {
+        add_partial_rows(sub);
+        keep_order();
+        ask_for_partial_rows(sub + round_stride);
+        ask_for_up_matrix();
+        add_partial_rows(sub + round_stride);
+        for (int s0 = sub + 2 * round_stride; s0 < in.n_partials; s0 += round_stride) {  // many partial rows and few waves a token
+            ask_for_partial_rows(s0);
+            add_partial_rows(s0);
         }
     }
+    // the down matrix is needed last: asked for now, it has the norm and the up product to arrive in
+    keep_order();
+    const int down_tiles = (width + 15) / 16, down_k_steps = packed_k_steps<bf16_t>(inner);
     Vec16 down_piece[DOWN_GROUP][K_STEPS_DOWN];
 #pragma unroll
     for (int g = 0; g < DOWN_GROUP; g++) {
-        int out_col = min((wave + DL_WAVES * g) * 16 + row16, width - 1);
+        int out_tile = min(wave + DL_WAVES * g, down_tiles - 1);
 #pragma unroll
-        for (int s = 0; s < K_STEPS_DOWN; s++)
-            down_piece[g][s] = *reinterpret_cast<const Vec16*>(w_down + (size_t)out_col * inner + min(slice * U + s * 32 + quad * 8, inner - 8));
+        for (int s = 0; s < K_STEPS_DOWN; s++)  // chunks beyond the hidden units: read again, met by zeros of the hidden row
+            down_piece[g][s] = load16<Vec16>(w_down + packed_offset<bf16_t>(out_tile, min(slice * K_STEPS_DOWN + s, down_k_steps - 1), down_k_steps, 0), lane * 16);
     }
-
     {
-        for (int s0 = sub; s0 < in.n_partials; s0 += waves_per_token * ROWS_AT_ONCE) {
-            if (s0 != sub) ask_for_partial_rows(s0);
-#pragma unroll
-            for (int u = 0; u < ROWS_AT_ONCE; u++)
-                if (s0 + waves_per_token * u < in.n_partials) {
-#pragma unroll
-                    for (int j = 0; j < NV; j++) row[j] += part[u][j];
-                }
-        }
         if (waves_per_token > 1) {  // the same for the whole block
 #pragma unroll
             for (int j = 0; j < NV; j++)
@@ -550,17 +669,15 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
 #pragma unroll
                 for (int u = 0; u < UP_UNITS; u++)
 #pragma unroll
-                    for (int j = 0; j < UP_ROUND; j++) {
-                        int k = (up_part_of[u] + DL_KSPLIT * (i0 + j)) * 32 + quad * 8;
-                        up_piece[u][j] = *reinterpret_cast<const Vec16*>(w_up + (up_at[u] + min(k, width - 8)));
-                    }
+                    for (int j = 0; j < UP_ROUND; j++)
+                        up_piece[u][j] = load16<Vec16>(w_up + packed_offset<bf16_t>(up_at[u], min(up_part_of[u] + DL_KSPLIT * (i0 + j), n_steps - 1), n_steps, 0), lane * 16);
             }
 #pragma unroll
             for (int u = 0; u < UP_UNITS; u++)
 #pragma unroll
                 for (int j = 0; j < UP_ROUND; j++) {
                     int step = up_part_of[u] + DL_KSPLIT * (i0 + j);
-                    Vec16 w = mask16(up_piece[u][j], step * 32 + quad * 8 < width && up_valid[u]);
+                    Vec16 w = mask16(up_piece[u][j], step < n_steps);
                     bf16x8 x = *reinterpret_cast<const bf16x8*>(x_hat + row16 * x_stride + min(step, n_steps - 1) * 32 + quad * 8);
                     acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc[u], 0, 0, 0);
                 }
@@ -575,14 +692,17 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
     DL_STAMP(13);
     lds_barrier();
     // acc[r] of lane l in tile t is (token l % 16, hidden unit 16 t + 4 (l / 16) + r)
-    for (int index = tid; index < TILES * 256; index += DL_THREADS) {
+#pragma unroll
+    for (int i = 0; i < BIAS_PER_THREAD; i++) {
+        const int index = tid + DL_THREADS * i;
+        if (index >= TILES * 256) break;
         const int tile = index / 256, r = (index / WAVE) % 4, l = index % WAVE;
         float value = 0.0f;
 #pragma unroll
         for (int p = 0; p < DL_KSPLIT; p++) value += up_part[((p * TILES + tile) * 4 + r) * WAVE + l];
         const int unit = tile * 16 + 4 * (l / 16) + r, h = slice * U + unit;
         if (h < inner) {
-            if (b_up) value += b_up[h];
+            if (b_up) value += up_bias[i];
             if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
             else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
         } else {
@@ -595,16 +715,15 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
 
     // ---- this slice's share of the down product: rows of w_down in tiles of 16, columns slice*U ..
     {
-        const int n_tiles = (width + 15) / 16;
         const int token = token0 + row16;
-        for (int tile0 = wave; tile0 < n_tiles; tile0 += DL_WAVES * DOWN_GROUP) {
+        for (int tile0 = wave; tile0 < down_tiles; tile0 += DL_WAVES * DOWN_GROUP) {
             if (tile0 != wave) {  // wider than the rows asked for at the start cover
 #pragma unroll
                 for (int g = 0; g < DOWN_GROUP; g++) {
-                    int out_col = min((tile0 + DL_WAVES * g) * 16 + row16, width - 1);
+                    int out_tile = min(tile0 + DL_WAVES * g, down_tiles - 1);
 #pragma unroll
                     for (int s = 0; s < K_STEPS_DOWN; s++)
-                        down_piece[g][s] = *reinterpret_cast<const Vec16*>(w_down + (size_t)out_col * inner + min(slice * U + s * 32 + quad * 8, inner - 8));
+                        down_piece[g][s] = load16<Vec16>(w_down + packed_offset<bf16_t>(out_tile, min(slice * K_STEPS_DOWN + s, down_k_steps - 1), down_k_steps, 0), lane * 16);
                 }
             }
 #pragma unroll
@@ -613,12 +732,11 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
                 f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int s = 0; s < K_STEPS_DOWN; s++) {
-                    Vec16 w = mask16(down_piece[g][s], slice * U + s * 32 + quad * 8 < inner && tile * 16 + row16 < width);
                     bf16x8 x = *reinterpret_cast<const bf16x8*>(hidden + row16 * H_STRIDE + s * 32 + quad * 8);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&down_piece[g][s]), x, acc, 0, 0, 0);
                 }
                 int out_col = tile * 16 + 4 * quad;
-                if (token < n_tokens && out_col < width)
+                if (row16 < tokens_here && out_col < width)
                     *reinterpret_cast<f32x4*>(partial_out + ((size_t)slice * n_tokens + token) * width + out_col) = acc;
             }
         }
@@ -662,9 +780,13 @@ int launch_mlp_half(PendingSum in, float* summed, const float* gamma, const floa
         MLLM_REQUIRE(status == hipSuccess, "decode_mlp_half: cannot raise the LDS limit: %s", hipGetErrorString(status));
         raised = true;
     }
-    dim3 grid((inner + U - 1) / U, (n_tokens + DL_TOKENS - 1) / DL_TOKENS);
+    // Few tokens a block: more waves share a token's pending sums (one round of loads instead of
+    // several, each a trip to memory) and more blocks pull at the matrices; many tokens a block: the
+    // matrices are read fewer times.
+    const int tokens_per_block = stage_pieces == 0 ? DL_TOKENS : (n_tokens <= 16 ? 4 : (n_tokens <= 64 ? 8 : DL_TOKENS));
+    dim3 grid((inner + U - 1) / U, (n_tokens + tokens_per_block - 1) / tokens_per_block);
     decode_mlp_half_kernel<NV, U><<<grid, DL_THREADS, lds, stream>>>(in, summed, gamma, beta, eps, w_up, b_up, w_down, partial_out,
-                                                                      n_tokens, width, inner, epilogue, stage_pieces);
+                                                                      n_tokens, width, inner, epilogue, stage_pieces, tokens_per_block);
     return 0;
 }
 
@@ -719,7 +841,7 @@ MLLM_API int mllm_decode_mlp_half(const float* base, const float* partials, cons
                                   const float* b_up, const void* w_down, float* partial_out, int n_tokens, int width,
                                   int inner, int slice_units, int epilogue, hipStream_t stream) {
     if (check_pending("decode_mlp_half", base, partials, n_partials, width)) return 1;
-    MLLM_REQUIRE(n_tokens >= 0 && n_tokens <= 65535 * DL_TOKENS, "decode_mlp_half: %d tokens", n_tokens);
+    MLLM_REQUIRE(n_tokens >= 0 && n_tokens <= 65535 * 4, "decode_mlp_half: %d tokens", n_tokens);
     MLLM_REQUIRE(inner >= 8 && inner % 8 == 0, "decode_mlp_half: %d hidden units is not a multiple of 8", inner);
     MLLM_REQUIRE(slice_units == 64 || slice_units == 128, "decode_mlp_half: slices of %d hidden units; 64 or 128", slice_units);
     MLLM_REQUIRE(epilogue >= 0 && epilogue <= 2, "decode_mlp_half: unknown epilogue %d", epilogue);

@@ -1,7 +1,7 @@
 // Matrix products on the matrix cores: out[M,N] = act(A[M,K] . W[N,K]^T + bias[N]) (+ residual).
 //
-// W is kept [out, in] (rows contiguous in K), which is what an MFMA operand wants and what the
-// tied head's token table already is. 32-bit inputs use the 32-bit MFMA (no reduced-precision
+// W is [out, in], either row-major (rows contiguous in K: what the tied head's token table
+// already is) or in the packed layout (common.h), which the weights of the layers are kept in. 32-bit inputs use the 32-bit MFMA (no reduced-precision
 // matrix mode); bfloat16 inputs use the bf16 MFMA; sums are 32-bit in both. Replaces the
 // reference's mult_kernel + add_bias + gelu + vector_addition (engine/src/matrixmult.cu:7-34,
 // linear.cu:9-18) and its epilogue order sum -> +bias -> activation -> residual + that
@@ -70,7 +70,7 @@ __device__ __forceinline__ Vec16 mask_piece(Vec16 v, bool valid) {
 // Tiles of A and W go memory -> registers -> LDS; the loads run two tiles ahead of the products
 // (two register sets used in turn), so that one block per compute unit still hides the memory
 // latency: these products are small enough that the grid often is no more than that.
-template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED>
+template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, bool PACKED>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                    const float* __restrict__ bias,
                                                    const float* __restrict__ residual,
@@ -82,7 +82,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
     constexpr int VPR = BK / VEC;  // 16-byte pieces per tile row
     constexpr int THREADS = 64 * WAVES_M * WAVES_N;
     constexpr int A_PIECES = (BM * VPR + THREADS - 1) / THREADS, W_PIECES = (BN * VPR + THREADS - 1) / THREADS;
-    static_assert(TM >= 1 && TN >= 1, "tile layout");
+    constexpr int KC = 4 * VEC, CHUNKS_K = BK / KC;  // packed W: columns of a chunk, chunks along k in a tile
+    static_assert(TM >= 1 && TN >= 1 && BN % 16 == 0 && BK % KC == 0, "tile layout");
+    const int w_row_tiles = ceil_div(N, 16), w_k_steps = packed_k_steps<T>(K);
 
     __shared__ __attribute__((aligned(16))) T a_tiles[2][BM * LDK];  // two buffers: one is read while
     __shared__ __attribute__((aligned(16))) T w_tiles[2][BN * LDK];  // the next tile is written to the other
@@ -111,7 +113,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (BN * VPR % THREADS == 0 || piece < BN * VPR) w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, w_valid[set][i]);
+            if (BN * VPR % THREADS == 0 || piece < BN * VPR) {
+                if constexpr (PACKED) {
+                    // 64 consecutive pieces are one chunk: 1 KiB of contiguous memory
+                    int chunk = piece / 64, row_tile = n0 / 16 + chunk / CHUNKS_K, k_step = k0 / KC + chunk % CHUNKS_K;
+                    w_valid[set][i] = row_tile < w_row_tiles && k_step < w_k_steps;
+                    w_regs[set][i] = *reinterpret_cast<const Vec16*>(W + packed_offset<T>(min(row_tile, w_row_tiles - 1), min(k_step, w_k_steps - 1), w_k_steps, piece % 64));
+                } else {
+                    w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, w_valid[set][i]);
+                }
+            }
         }
     };
     auto stage = [&](int set) {  // register set `set` -> LDS buffer `set`
@@ -125,7 +136,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (piece < BN * VPR) *reinterpret_cast<Vec16*>(&w_tile[(piece / VPR) * LDK + (piece % VPR) * VEC]) = mask_piece(w_regs[set][i], w_valid[set][i]);
+            if (piece < BN * VPR) {
+                int row = piece / VPR, k = (piece % VPR) * VEC;
+                if constexpr (PACKED) {
+                    int chunk = piece / 64, l = piece % 64;
+                    row = (chunk / CHUNKS_K) * 16 + l % 16, k = (chunk % CHUNKS_K) * KC + (l / 16) * VEC;
+                }
+                *reinterpret_cast<Vec16*>(&w_tile[row * LDK + k]) = mask_piece(w_regs[set][i], w_valid[set][i]);
+            }
         }
     };
     auto products = [&](int buffer) {
@@ -224,7 +242,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 // 16 rows; the x rows of the same k come through the cache). out^T = W . x^T, so that W is the
 // 16-row operand. The waves' partial sums meet in LDS, where the epilogue runs.
 // ------------------------------------------------------------------------------------------------
-template <typename T, typename OutT, int MT, int KSPLIT>
+template <typename T, typename OutT, int MT, int KSPLIT, bool PACKED>
 __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     const T* __restrict__ A, const T* __restrict__ W, const float* __restrict__ bias,
     const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue,
@@ -264,7 +282,10 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         for (int u = 0; u < UNROLL; u++) {
             int k = (step0 + u) * KSTEP + quad * VEC;  // K is a multiple of VEC: a piece is whole or absent
             int safe_k = min(k, K - VEC);  // loads are unconditional, from a clamped address: no branch between them
-            w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + safe_k);
+            if constexpr (PACKED)  // a chunk of the packed layout is this wave's operand as it lies in memory
+                w_piece[u] = *reinterpret_cast<const Vec16*>(W + packed_offset<T>(blockIdx.x, min(step0 + u, n_steps - 1), n_steps, lane));
+            else
+                w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + safe_k);
 #pragma unroll
             for (int i = 0; i < MT; i++) x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + safe_k);
         }
@@ -333,36 +354,47 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 }
 
 template <typename T, typename OutT, int MT>
-void launch_skinny(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M,
+void launch_skinny(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M,
                    int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}) {
     constexpr int KSTEP = 4 * Tile<T>::VEC;
     int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
     int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
     while (split < 16 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
     dim3 grid(tiles);
-    if (split == 16)
-        gemm_skinny_kernel<T, OutT, MT, 16><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    else if (split == 1)
-        gemm_skinny_kernel<T, OutT, MT, 1><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    else if (split == 2)
-        gemm_skinny_kernel<T, OutT, MT, 2><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    else if (split == 4)
-        gemm_skinny_kernel<T, OutT, MT, 4><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    else
-        gemm_skinny_kernel<T, OutT, MT, 8><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    if (split == 16) {
+        if (packed) gemm_skinny_kernel<T, OutT, MT, 16, true><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+        else gemm_skinny_kernel<T, OutT, MT, 16, false><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    }
+    else if (split == 1) {
+        if (packed) gemm_skinny_kernel<T, OutT, MT, 1, true><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+        else gemm_skinny_kernel<T, OutT, MT, 1, false><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    }
+    else if (split == 2) {
+        if (packed) gemm_skinny_kernel<T, OutT, MT, 2, true><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+        else gemm_skinny_kernel<T, OutT, MT, 2, false><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    }
+    else if (split == 4) {
+        if (packed) gemm_skinny_kernel<T, OutT, MT, 4, true><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+        else gemm_skinny_kernel<T, OutT, MT, 4, false><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    }
+    else {
+        if (packed) gemm_skinny_kernel<T, OutT, MT, 8, true><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+        else gemm_skinny_kernel<T, OutT, MT, 8, false><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    }
 }
 
 int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
 
 template <typename T, typename OutT, bool ALIGNED, int BM, int BN, int WAVES_M, int WAVES_N>
-void launch_tile(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M, int N,
+void launch_tile(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
                  int K, int epilogue, hipStream_t stream) {
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
-    gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
 }
 
 template <typename T, typename OutT, bool ALIGNED>
-void launch_tiled(const T* a, const T* w, const float* bias, const float* residual, OutT* o, int M, int N,
+void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
                   int K, int epilogue, hipStream_t stream) {
     int tile = g_forced_tile;
     if (tile == 0) {
@@ -372,18 +404,18 @@ void launch_tiled(const T* a, const T* w, const float* bias, const float* residu
         else tile = 7;
     }
     switch (tile) {
-        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
-        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
     }
 }
 
 template <typename T, typename OutT>
-void launch_gemm(const void* A, const void* W, const float* bias, const float* residual, void* out,
+void launch_gemm(const void* A, const void* W, bool packed, const float* bias, const float* residual, void* out,
                  int M, int N, int K, int epilogue, hipStream_t stream) {
     const T* a = (const T*)A;
     const T* w = (const T*)W;
@@ -395,13 +427,13 @@ void launch_gemm(const void* A, const void* W, const float* bias, const float* r
     const bool wide = N >= 8192;
     const int skinny_rows = !wide ? 64 : (sizeof(T) == 2 ? 0 : 12);
     if (g_forced_tile == 0 && aligned && M <= skinny_rows) {
-        if (M <= 16) launch_skinny<T, OutT, 1>(a, w, bias, residual, o, M, N, K, epilogue, stream);
-        else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, bias, residual, o, M, N, K, epilogue, stream);
-        else launch_skinny<T, OutT, 4>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+        if (M <= 16) launch_skinny<T, OutT, 1>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
+        else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
+        else launch_skinny<T, OutT, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
     } else if (aligned) {
-        launch_tiled<T, OutT, true>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+        launch_tiled<T, OutT, true>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
     } else {
-        launch_tiled<T, OutT, false>(a, w, bias, residual, o, M, N, K, epilogue, stream);
+        launch_tiled<T, OutT, false>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
     }
 }
 
@@ -410,7 +442,7 @@ void launch_gemm(const void* A, const void* W, const float* bias, const float* r
 // Tuning aid: forces one tile shape of the tiled kernel (0 gives the choice back to the sizes).
 MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
-MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const float* residual,
+MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* bias, const float* residual,
                        void* out, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,
                        hipStream_t stream) {
     MLLM_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -418,11 +450,11 @@ MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const fl
     MLLM_REQUIRE(ceil_div(M, 32) <= 65535, "gemm: M=%d has too many row tiles", M);
     if (M == 0) return 0;
     if (in_dtype == MLLM_F32 && out_dtype == MLLM_F32)
-        launch_gemm<float, float>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<float, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
     else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_BF16)
-        launch_gemm<bf16_t, bf16_t>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<bf16_t, bf16_t>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
     else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_F32)
-        launch_gemm<bf16_t, float>(A, W, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<bf16_t, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
     else
         MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
     return mllm_check_launch("gemm");
@@ -431,7 +463,7 @@ MLLM_API int mllm_gemm(const void* A, const void* W, const float* bias, const fl
 // The fused q/k/v projection of a decode step or a short portion (M <= 64 rows): q columns go
 // to out_q [M, q_width], key and value columns straight into the cache pages at slots[row]
 // (what the reference's decode block does with its fused matvec: engine/src/transformer_block.cu:223-242).
-MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, const float* bias, void* out_q, void* k_pages,
+MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, const float* bias, void* out_q, void* k_pages,
                                  void* v_pages, const int* slots, int M, int K, int q_width, int kv_width,
                                  int n_kv_heads, int head_size, int page_size, int dtype, hipStream_t stream) {
     MLLM_REQUIRE(M >= 0 && M <= 64, "gemm_qkv_cache: %d rows; this entry takes up to 64", M);
@@ -444,9 +476,9 @@ MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, const float* bias
     while ((1 << scatter.page_shift) < page_size) scatter.page_shift++;
     int N = q_width + 2 * kv_width;
 #define MLLM_QKV_CASE(T)                                                                                              \
-    if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
-    else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
-    else launch_skinny<T, T, 4>((const T*)A, (const T*)W, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
+    if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
+    else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
+    else launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
     if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
 #undef MLLM_QKV_CASE
     return mllm_check_launch("gemm_qkv_cache");

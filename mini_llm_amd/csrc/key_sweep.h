@@ -51,29 +51,53 @@ struct KeySweep {
         Raw kf[UNROLL], vf[UNROLL];
     };
 
-    // Asks for the keys base .. base+KPI-1 of the request whose block table is given, those from
-    // `end` on replaced by `spare_key` (any key whose page the table holds). No branch between the
-    // loads: all are in flight together, and nothing here waits for them. KEYS / VALUES: which of
-    // the two to ask for (a caller short of registers asks for the values later).
+    // The pages of the keys base .. base+KPI-1 of the request whose block table is given, those
+    // from `end` on replaced by `spare_key` (any key whose page the table holds): the first half of
+    // fetch(), for a caller that wants the table's answer under way before it asks for the rows.
+    __device__ __forceinline__ void look_up(int (&page)[UNROLL], const int* __restrict__ table, int page_shift,
+                                            int base, int end, int spare_key, int lane) const {
+        const int group = lane / LPR;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            int key = base + u * RPI + group;
+            page[u] = table[(key < end ? key : spare_key) >> page_shift];
+        }
+    }
+
+    // Asks for those keys and values, given their pages. No branch between the loads: all are in
+    // flight together, and nothing here waits for them. KEYS / VALUES: which of the two to ask for.
     template <bool KEYS = true, bool VALUES = true>
-    __device__ __forceinline__ void fetch(Fetched& f, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
-                                          const int* __restrict__ table, int kv_head, int n_kv_heads, int page_shift,
-                                          int base, int end, int spare_key, int lane) const {
+    __device__ __forceinline__ void fetch_rows(Fetched& f, const int (&page)[UNROLL], const T* __restrict__ k_pages,
+                                               const T* __restrict__ v_pages, int kv_head, int n_kv_heads, int page_shift,
+                                               int base, int end, int spare_key, int lane) const {
         const int sub = lane % LPR, group = lane / LPR;
         const int page_mask = (1 << page_shift) - 1;
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             int key = base + u * RPI + group;
             int safe_key = key < end ? key : spare_key;
-            int page = table[safe_key >> page_shift];
-            size_t row = ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask));
+            size_t row = ((((size_t)page[u] * n_kv_heads + kv_head) << page_shift) + (safe_key & page_mask));
             if constexpr (KEYS) f.kf[u] = *reinterpret_cast<const Raw*>(k_pages + row * HD + sub * VEC);
             if constexpr (VALUES) f.vf[u] = *reinterpret_cast<const Raw*>(v_pages + row * HD + sub * VEC);
         }
     }
 
-    // Takes the fetched keys base .. min(base+KPI, end)-1 (at least one) into the running softmax.
+    // Both halves at once.
+    template <bool KEYS = true, bool VALUES = true>
+    __device__ __forceinline__ void fetch(Fetched& f, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                                          const int* __restrict__ table, int kv_head, int n_kv_heads, int page_shift,
+                                          int base, int end, int spare_key, int lane) const {
+        int page[UNROLL];
+        look_up(page, table, page_shift, base, end, spare_key, lane);
+        fetch_rows<KEYS, VALUES>(f, page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, base, end, spare_key, lane);
+    }
+
+    // Takes the fetched keys base .. min(base+KPI, end)-1 (there may be none) into the running softmax.
     // qf: the lane's VEC dimensions of the query, already scaled.
+    // CLEAN_VALUES: a key that does not count may have been fetched from memory nobody has written
+    // yet (the spare key of a wave without keys); its value then is replaced by zero, as not even
+    // a weight of zero silences a NaN.
+    template <bool CLEAN_VALUES = false>
     __device__ __forceinline__ void consume(const Fetched& f, const float (&qf)[VEC], int base, int end, int lane) {
         const int group = lane / LPR;
         float score[UNROLL];
@@ -90,17 +114,23 @@ struct KeySweep {
         }
 #pragma unroll
         for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
-        float new_max = fmaxf(running_max, tile_max);  // finite: the first key of the tile is valid
-        float rescale = expf(running_max - new_max);
+        float new_max = fmaxf(running_max, tile_max);
+        float reference = new_max == -INFINITY ? 0.0f : new_max;  // no key so far (base >= end is allowed): nothing to rescale
+        float rescale = expf(running_max - reference);
         running_sum *= rescale;
 #pragma unroll
         for (int i = 0; i < VEC; i++) o[i] *= rescale;
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
-            float p = base + u * RPI + group < end ? expf(score[u] - new_max) : 0.0f;
+            const bool counts = base + u * RPI + group < end;
+            float p = counts ? expf(score[u] - reference) : 0.0f;
             running_sum += p;
 #pragma unroll
-            for (int i = 0; i < VEC; i++) o[i] += p * Chunk<T>::get(f.vf[u], i);
+            for (int i = 0; i < VEC; i++) {
+                float value = Chunk<T>::get(f.vf[u], i);
+                if (CLEAN_VALUES && !counts) value = 0.0f;
+                o[i] += p * value;
+            }
         }
         running_max = new_max;
     }

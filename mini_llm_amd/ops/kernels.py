@@ -105,16 +105,59 @@ def add(a, b, out=None):
     return out
 
 
+class PackedMatrix:
+    """A weight matrix [rows (out), cols (in)] in the packed layout of the matrix kernels: chunks
+    of 16 rows x 64 bytes, each chunk's 16-byte pieces in the order the lanes of a wave take them
+    as matrix-core operands, zeros beyond the matrix. ``data`` is the flat device tensor."""
+
+    def __init__(self, data: torch.Tensor, rows: int, cols: int):
+        self.data, self.rows, self.cols = data, rows, cols
+
+    @property
+    def shape(self):
+        return (self.rows, self.cols)
+
+    @property
+    def dtype(self):
+        return self.data.dtype
+
+    @property
+    def device(self):
+        return self.data.device
+
+
+def pack_matrix(src, dtype=None, transpose=False) -> PackedMatrix:
+    """A float32/bfloat16 matrix [out, in] (or, with ``transpose``, stored [in, out]) in the packed
+    layout, in element type ``dtype`` (default: its own). Load-time work on weights."""
+    _device_tensor(src, "src", dim=2)
+    dtype = src.dtype if dtype is None else dtype
+    rows, cols = (src.shape[1], src.shape[0]) if transpose else src.shape
+    _require(rows > 0 and cols > 0, "an empty matrix cannot be packed")
+    lib = library()
+    data = torch.empty((lib.mllm_packed_elements(rows, cols, _code(dtype)),), dtype=dtype, device=src.device)
+    check(lib.mllm_pack_matrix(_ptr(src), _ptr(data), rows, cols, _code(src.dtype), _code(dtype), int(bool(transpose)), _stream()))
+    return PackedMatrix(data, rows, cols)
+
+
+def _matrix(weight, name, dtype):
+    """(pointer, packed flag, rows, cols) of a weight given row-major or packed."""
+    if isinstance(weight, PackedMatrix):
+        _device_tensor(weight.data, name, dtype, 1)
+        return _ptr(weight.data), 1, weight.rows, weight.cols
+    _device_tensor(weight, name, dtype, 2)
+    return _ptr(weight), 0, weight.shape[0], weight.shape[1]
+
+
 def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None, out=None):
-    """act(x @ weight.T + bias) (+ residual). ``weight`` is [out, in]; sums are float32.
+    """act(x @ weight.T + bias) (+ residual). ``weight`` is [out, in], a row-major tensor or a
+    PackedMatrix; sums are float32.
 
     x and weight share their element type (float32: true 32-bit MFMA; bfloat16: bf16 MFMA);
     bias and residual are float32; a residual makes the output float32."""
     _device_tensor(x, "x", dim=2)
-    _device_tensor(weight, "weight", x.dtype, 2)
+    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
     m, k = x.shape
-    n = weight.shape[0]
-    _require(weight.shape[1] == k, f"x has {k} columns but weight has {weight.shape[1]}")
+    _require(w_cols == k, f"x has {k} columns but weight has {w_cols}")
     _require(activation in EPILOGUES, f"unknown activation {activation!r}")
     if bias is not None:
         _device_tensor(bias, "bias", torch.float32, 1)
@@ -130,7 +173,7 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
     _device_tensor(out, "out", out_dtype, 2)
     _require(tuple(out.shape) == (m, n), "out has the wrong shape")
     _require(x.dtype != torch.float32 or out_dtype == torch.float32, "float32 inputs give float32 outputs")
-    check(library().mllm_gemm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x.dtype), _code(out_dtype), EPILOGUES[activation], _stream()))
+    check(library().mllm_gemm(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x.dtype), _code(out_dtype), EPILOGUES[activation], _stream()))
     return out
 
 
@@ -179,21 +222,21 @@ def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_hea
     """The fused q/k/v projection of up to 64 rows: returns q [rows, n_heads*head_size] and writes
     the key and value columns straight into the cache pages at slots[row] (negative: skip)."""
     _device_tensor(x, "x", dim=2)
-    _device_tensor(weight, "weight", x.dtype, 2)
+    w_ptr, w_packed, w_rows, w_cols = _matrix(weight, "weight", x.dtype)
     num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     _require(k_pages.dtype == x.dtype, "pages and x differ in element type")
     m, k = x.shape
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
     _require(m <= FUSED_QKV_MAX_ROWS, f"{m} rows; the fused projection takes up to {FUSED_QKV_MAX_ROWS}")
-    _require(tuple(weight.shape) == (q_width + 2 * kv_width, k), "weight does not match the heads or x")
+    _require((w_rows, w_cols) == (q_width + 2 * kv_width, k), "weight does not match the heads or x")
     _require(k % (16 // x.element_size()) == 0, "the input width is not a multiple of a 16-byte piece")
     if bias is not None:
         _device_tensor(bias, "bias", torch.float32, 1)
-        _require(bias.shape[0] == weight.shape[0], "bias does not match weight")
+        _require(bias.shape[0] == w_rows, "bias does not match weight")
     _device_tensor(slots, "slots", torch.int32, 1)
     _require(slots.shape[0] >= m, "fewer slots than rows")
     q = torch.empty((m, q_width), dtype=x.dtype, device=x.device)
-    check(library().mllm_gemm_qkv_cache(_ptr(x), _ptr(weight), _ptr(bias), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(slots), m, k, q_width, kv_width, n_kv_heads, head_size, page_size, _code(x.dtype), _stream()))
+    check(library().mllm_gemm_qkv_cache(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(slots), m, k, q_width, kv_width, n_kv_heads, head_size, page_size, _code(x.dtype), _stream()))
     return q
 
 
@@ -304,7 +347,7 @@ class PendingRows:
 
 
 MLP_SLICE_UNITS = 64         # hidden units a block of the feed-forward kernel takes
-LAYER_KERNEL_MAX_ROWS = 0    # rows up to this many take the layer kernels (0: off until they beat the separate kernels)
+LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kernels
 
 
 def _pending(hidden):
@@ -349,7 +392,8 @@ def _norm_vectors(gamma, beta, width):
 def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, k_pages, v_pages, slots, token_request,
                           positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, write_cache=True):
     """norm, q/k/v, cache write, attention and output product of a pre-norm layer's first half, for
-    rows that are each the newest token of their request, in one kernel (bfloat16 only).
+    rows that are each the newest token of their request, in one kernel (bfloat16 only; the two
+    matrices as PackedMatrix).
 
     ``hidden``: float32 rows or PendingRows. Returns PendingRows: the stream before this half
     with its sums taken, one partial row per head, and the output product's bias."""
@@ -360,10 +404,11 @@ def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, 
     _require(k_pages.dtype == torch.bfloat16, "the layer kernels for decoding are bfloat16 only")
     _require(decode_layer_supported(width, head_size, page_size), f"no layer kernel for width {width}, head size {head_size}, pages of {page_size}")
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
-    _device_tensor(w_qkv, "w_qkv", torch.bfloat16, 2)
-    _device_tensor(w_out, "w_out", torch.bfloat16, 2)
-    _require(tuple(w_qkv.shape) == (q_width + 2 * kv_width, width), "w_qkv does not match the heads or the width")
-    _require(tuple(w_out.shape) == (width, q_width), "w_out does not match the heads or the width")
+    for w, name in ((w_qkv, "w_qkv"), (w_out, "w_out")):
+        _require(isinstance(w, PackedMatrix), f"{name} must be a PackedMatrix")
+        _device_tensor(w.data, name, torch.bfloat16, 1)
+    _require(w_qkv.shape == (q_width + 2 * kv_width, width), "w_qkv does not match the heads or the width")
+    _require(w_out.shape == (width, q_width), "w_out does not match the heads or the width")
     for t, name, n in ((b_qkv, "b_qkv", q_width + 2 * kv_width), (b_out, "b_out", width)):
         if t is not None:
             _device_tensor(t, name, torch.float32, 1)
@@ -375,8 +420,8 @@ def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, 
     summed = torch.empty_like(base)
     out = torch.empty((n_heads, rows, width), dtype=torch.float32, device=base.device)
     check(library().mllm_decode_attention_half(
-        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_qkv),
-        _ptr(b_qkv), _ptr(w_out), _ptr(k_pages), _ptr(v_pages), _ptr(slots), _ptr(token_request), _ptr(positions),
+        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_qkv.data),
+        _ptr(b_qkv), _ptr(w_out.data), _ptr(k_pages), _ptr(v_pages), _ptr(slots), _ptr(token_request), _ptr(positions),
         _ptr(block_tables), block_tables.shape[1], _ptr(out), rows, width, n_heads, n_kv_heads, head_size, page_size,
         int(window), float(scale), int(bool(write_cache)), _stream()))
     return PendingRows(summed, out, b_out)
@@ -384,17 +429,18 @@ def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, 
 
 def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activation=None, slice_units=MLP_SLICE_UNITS):
     """norm, up product, activation and down product of a pre-norm layer's second half in one
-    kernel (bfloat16 matrices). Returns PendingRows: the stream before this half with its sums
+    kernel (bfloat16 matrices as PackedMatrix). Returns PendingRows: the stream before this half with its sums
     taken, one partial row per slice of ``slice_units`` hidden units, and the down product's bias."""
     base, partials, bias, n_partials = _pending(hidden)
     rows, width = base.shape
     _norm_vectors(gamma, beta, width)
     _require(activation in EPILOGUES, f"unknown activation {activation!r}")
-    _device_tensor(w_up, "w_up", torch.bfloat16, 2)
-    _device_tensor(w_down, "w_down", torch.bfloat16, 2)
-    inner = w_up.shape[0]
+    for w, name in ((w_up, "w_up"), (w_down, "w_down")):
+        _require(isinstance(w, PackedMatrix), f"{name} must be a PackedMatrix")
+        _device_tensor(w.data, name, torch.bfloat16, 1)
+    inner = w_up.rows
     _require(decode_layer_supported(width, inner=inner), f"no layer kernel for width {width} with {inner} hidden units")
-    _require(tuple(w_up.shape) == (inner, width) and tuple(w_down.shape) == (width, inner), "the two matrices do not match the width")
+    _require(w_up.shape == (inner, width) and w_down.shape == (width, inner), "the two matrices do not match the width")
     for t, name, n in ((b_up, "b_up", inner), (b_down, "b_down", width)):
         if t is not None:
             _device_tensor(t, name, torch.float32, 1)
@@ -403,6 +449,6 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
     summed = torch.empty_like(base)
     out = torch.empty(((inner + slice_units - 1) // slice_units, rows, width), dtype=torch.float32, device=base.device)
     check(library().mllm_decode_mlp_half(
-        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_up),
-        _ptr(b_up), _ptr(w_down), _ptr(out), rows, width, inner, slice_units, EPILOGUES[activation], _stream()))
+        _ptr(base), _ptr(partials), _ptr(bias), n_partials, _ptr(summed), _ptr(gamma), _ptr(beta), float(eps), _ptr(w_up.data),
+        _ptr(b_up), _ptr(w_down.data), _ptr(out), rows, width, inner, slice_units, EPILOGUES[activation], _stream()))
     return PendingRows(summed, out, b_down)

@@ -18,9 +18,11 @@ _SIGNATURES = {
     "mllm_embed": [P, P, P, P, P, c_int, c_int, c_int, P],
     "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
-    "mllm_gemm": [P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_gemm_qkv_cache": [P, P, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_qkv_cache": [P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_convert": [P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_pack_matrix": [P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_packed_elements": [c_int, c_int, c_int],
     "mllm_probe_read": [P, c_longlong, P, c_int, P],
     "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
@@ -62,6 +64,7 @@ def library() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = c_int
+        lib.mllm_packed_elements.restype = c_longlong
         lib.mllm_last_error.restype = ctypes.c_char_p
         lib.mllm_last_error.argtypes = []
         lib.path = path

@@ -76,8 +76,10 @@ def place(tensor: torch.Tensor, spec: TensorSpec, precision, device) -> torch.Te
     else:
         raise ValueError(f"unknown tensor role {spec.role!r}")
     if tensor.is_cuda and tensor.dtype in (torch.float32, torch.bfloat16) and tensor.dim() in (1, 2):
-        from ..ops import kernels  # on the GPU the conversion and the transpose are this framework's kernel
+        from ..ops import kernels  # on the GPU the conversion and the transpose are this framework's kernels
 
+        if spec.role == MATRIX and tensor.dim() == 2:  # operands of matrix products are kept in the packed layout
+            return kernels.pack_matrix(tensor.contiguous(), target, transpose=spec.keep_transposed)
         return kernels.convert(tensor.contiguous(), target, transpose=spec.keep_transposed)
     tensor = tensor.to(target)  # other stored types (F16, F64) and host-only checks of the loader
     if spec.keep_transposed:

@@ -71,24 +71,57 @@ def test_layernorm_constant_row_gives_beta(K):
     np.testing.assert_allclose(host(out), np.stack([b, b]), atol=1e-6)
 
 
+def as_weight(K, w, dtype, packed):
+    """A weight on the device, row-major or in the packed layout of the matrix kernels."""
+    return K.pack_matrix(dev(w, dtype)) if packed else dev(w, dtype)
+
+
+def plain_packed(w, vec):
+    """The packed layout of a matrix, written out element by element: chunks of 16 rows x 4*vec
+    columns, row tiles outermost; piece p of a chunk is row p % 16, columns (p // 16) * vec .."""
+    rows, cols = w.shape
+    kc = 4 * vec
+    row_tiles, k_steps = -(-rows // 16), -(-cols // kc)
+    padded = np.zeros((row_tiles * 16, k_steps * kc), dtype=w.dtype)
+    padded[:rows, :cols] = w
+    out = np.zeros((row_tiles, k_steps, 64, vec), dtype=w.dtype)
+    for p in range(64):
+        out[:, :, p, :] = padded.reshape(row_tiles, 16, k_steps, kc)[:, p % 16, :, (p // 16) * vec : (p // 16 + 1) * vec]
+    return out.reshape(-1)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (16, 32), (33, 65), (96, 288), (50, 777)])
+@pytest.mark.parametrize("src,dst", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_pack_matrix(K, rows, cols, src, dst, transpose):
+    rng = np.random.default_rng(rows * 7 + cols)
+    w = bf16_round(rng.standard_normal((rows, cols)))  # exact in every element type here
+    stored = w.T if transpose else w
+    packed = K.pack_matrix(dev(np.ascontiguousarray(stored), src), dst, transpose=transpose)
+    assert packed.shape == (rows, cols) and packed.dtype == dst
+    np.testing.assert_array_equal(host(packed.data), plain_packed(w, 4 if dst == torch.float32 else 8))
+
+
 GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
                (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20)]
 
 
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
 @pytest.mark.parametrize("activation", [None, "gelu_new", "gelu"])
-def test_linear_f32(K, m, n, k, activation):
+def test_linear_f32(K, m, n, k, activation, packed):
     rng = np.random.default_rng(m * 1000 + n)
     x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
     res = rng.standard_normal((m, n))
     y = x.astype(np.float32).astype(np.float64) @ w.astype(np.float32).astype(np.float64).T + b.astype(np.float32)
     if activation:
         y = P.ACTIVATIONS[activation](y)
-    out = K.linear(dev(x), dev(w), dev(b), activation=activation)
+    weight = as_weight(K, w, torch.float32, packed)
+    out = K.linear(dev(x), weight, dev(b), activation=activation)
     np.testing.assert_allclose(host(out), y, rtol=1e-5, atol=1e-5)
-    out = K.linear(dev(x), dev(w), dev(b), activation=activation, residual=dev(res))
+    out = K.linear(dev(x), weight, dev(b), activation=activation, residual=dev(res))
     np.testing.assert_allclose(host(out), y + res.astype(np.float32), rtol=1e-5, atol=1e-5)
-    out = K.linear(dev(x), dev(w))
+    out = K.linear(dev(x), weight)
     np.testing.assert_allclose(host(out), x.astype(np.float32).astype(np.float64) @ w.astype(np.float32).astype(np.float64).T, rtol=1e-5, atol=1e-5)
 
 
@@ -101,18 +134,20 @@ def test_linear_f32_is_true_32_bit(K):
     assert (out == k * (1.0 + 2.0**-12)).all()  # exact in float32; a reduced mode gives 64.0
 
 
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_linear_bf16(K, m, n, k, out_dtype):
+def test_linear_bf16(K, m, n, k, out_dtype, packed):
     rng = np.random.default_rng(m * 1000 + n + 1)
     x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
     y = bf16_round(x) @ bf16_round(w).T + b.astype(np.float32)
-    out = K.linear(dev(x, torch.bfloat16), dev(w, torch.bfloat16), dev(b), activation="gelu_new", out_dtype=out_dtype)
+    weight = as_weight(K, w, torch.bfloat16, packed)
+    out = K.linear(dev(x, torch.bfloat16), weight, dev(b), activation="gelu_new", out_dtype=out_dtype)
     tol = 1e-2 if out_dtype == torch.bfloat16 else 2e-5
     np.testing.assert_allclose(host(out), P.gelu_new(y), rtol=tol, atol=tol)
     if out_dtype == torch.float32:
         res = rng.standard_normal((m, n)).astype(np.float32)
-        out = K.linear(dev(x, torch.bfloat16), dev(w, torch.bfloat16), dev(b), residual=dev(res))
+        out = K.linear(dev(x, torch.bfloat16), weight, dev(b), residual=dev(res))
         np.testing.assert_allclose(host(out), y + res, rtol=2e-5, atol=2e-5)
 
 
@@ -308,7 +343,8 @@ def test_operands_are_checked_on_the_host(K):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16)])
-def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size):
+@pytest.mark.parametrize("packed", [False, True])
+def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, packed):
     rng = np.random.default_rng(rows)
     width = 72
     qw, kvw = n_heads * head_size, n_kv_heads * head_size
@@ -319,7 +355,7 @@ def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_hea
     slots = rng.permutation(num_pages * page_size)[:rows].astype(np.int32)
     if rows > 2:
         slots[1] = -1  # a padding row writes nothing
-    q = K.linear_qkv_cache(dev(x, dtype), dev(w, dtype), dev(b), kp, vp, dev(slots, torch.int32), n_heads, n_kv_heads, head_size)
+    q = K.linear_qkv_cache(dev(x, dtype), as_weight(K, w, dtype, packed), dev(b), kp, vp, dev(slots, torch.int32), n_heads, n_kv_heads, head_size)
     xr, wr = (x.astype(np.float32).astype(np.float64), w.astype(np.float32).astype(np.float64)) if dtype == torch.float32 else (bf16_round(x), bf16_round(w))
     ref = xr @ wr.T + b.astype(np.float32)
     tol = 2e-5 if dtype == torch.float32 else 2e-2
@@ -422,7 +458,8 @@ def test_decode_attention_half(K, width, n_heads, n_kv_heads, head_size, page_si
     rng = np.random.default_rng(width + head_size)
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
     eps = 3e-5
-    contexts = [0, 1, page_size - 1, page_size, 150, 700, -1, 333]  # -1: a padding row
+    # -1: a padding row; 700 and 1500 reach beyond the keys the kernel asks for in its first go
+    contexts = [0, 1, page_size - 1, page_size, 150, 700, -1, 333, 1500]
     rows = len(contexts)
     hidden, total = _pending_rows(K, rng, rows, width, n_partials, with_bias)
     gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
@@ -459,7 +496,7 @@ def test_decode_attention_half(K, width, n_heads, n_kv_heads, head_size, page_si
         expected[r] = total[r] + mixed[0] @ w_out.T + b_out
     k_before, v_before = kp.clone(), vp.clone()
     out = K.decode_attention_half(
-        hidden, dev(gamma), dev(beta), eps, dev(w_qkv, torch.bfloat16), dev(b_qkv), dev(w_out, torch.bfloat16), dev(b_out), kp, vp,
+        hidden, dev(gamma), dev(beta), eps, as_weight(K, w_qkv, torch.bfloat16, True), dev(b_qkv), as_weight(K, w_out, torch.bfloat16, True), dev(b_out), kp, vp,
         dev(new_slots, torch.int32), dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
         n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window)
     assert out.partials.shape == (n_heads, rows, width)
@@ -483,8 +520,8 @@ def test_decode_attention_half_reads_a_cache_it_does_not_write(K):
     hidden, total = _pending_rows(K, rng, 1, width, 0, False)
     kp = torch.zeros((2, n_heads, page_size, head_size), device=DEV).bfloat16()
     vp = torch.zeros_like(kp)
-    args = (dev(np.ones(width)), dev(np.zeros(width)), 1e-5, dev(rng.standard_normal((3 * width, width)) * 0.2, torch.bfloat16), None,
-            dev(rng.standard_normal((width, width)) * 0.2, torch.bfloat16), None, kp, vp, dev([3], torch.int32), dev([0], torch.int32),
+    args = (dev(np.ones(width)), dev(np.zeros(width)), 1e-5, as_weight(K, rng.standard_normal((3 * width, width)) * 0.2, torch.bfloat16, True), None,
+            as_weight(K, rng.standard_normal((width, width)) * 0.2, torch.bfloat16, True), None, kp, vp, dev([3], torch.int32), dev([0], torch.int32),
             dev([3], torch.int32), dev([[0]], torch.int32), n_heads, n_heads, head_size, 0.25)
     reading = K.settle(K.decode_attention_half(hidden, *args, write_cache=False))
     assert not kp.any() and not vp.any()
@@ -508,7 +545,7 @@ def test_decode_mlp_half(K, width, inner, rows, activation, slice_units, n_parti
     act = {"gelu": P.gelu_erf, "gelu_new": P.gelu_new, None: lambda x: x}[activation]
     normed = bf16_round(P.layernorm(total, gamma, beta, eps))
     expected = total + bf16_round(act(normed @ w_up.T + b_up)) @ w_down.T + b_down
-    out = K.decode_mlp_half(hidden, dev(gamma), dev(beta), eps, dev(w_up, torch.bfloat16), dev(b_up), dev(w_down, torch.bfloat16),
+    out = K.decode_mlp_half(hidden, dev(gamma), dev(beta), eps, as_weight(K, w_up, torch.bfloat16, True), dev(b_up), as_weight(K, w_down, torch.bfloat16, True),
                             dev(b_down), activation=activation, slice_units=slice_units)
     assert out.partials.shape == ((inner + slice_units - 1) // slice_units, rows, width)
     np.testing.assert_allclose(host(out.base), total, rtol=1e-5, atol=1e-5)
@@ -524,4 +561,4 @@ def test_layer_kernels_refuse_what_they_do_not_take(K):
     x = torch.zeros((1, 96), device=DEV)
     ones = torch.ones(96, device=DEV)
     with pytest.raises(K.OperandError):
-        K.decode_mlp_half(x, ones, ones, 1e-5, torch.zeros((100, 96), device=DEV).bfloat16(), None, torch.zeros((96, 100), device=DEV).bfloat16(), None)
+        K.decode_mlp_half(x, ones, ones, 1e-5, K.pack_matrix(torch.zeros((100, 96), device=DEV).bfloat16()), None, K.pack_matrix(torch.zeros((96, 100), device=DEV).bfloat16()), None)

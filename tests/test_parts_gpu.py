@@ -29,8 +29,11 @@ def bind_random(part, seed, dtype="float32"):
     for name, spec in part.named_tensor_specs().items():
         value = (spec.init.mean + 5 * spec.init.std * rng.standard_normal(spec.shape)).astype(np.float32)
         placed[name] = place(torch.from_numpy(value), spec, precision, DEV)
-        kept = placed[name].float().cpu().numpy()
-        stored[name] = (kept.T if spec.keep_transposed else kept).astype(np.float64)
+        if isinstance(placed[name], torch.Tensor):
+            kept = placed[name].float().cpu().numpy()
+            stored[name] = (kept.T if spec.keep_transposed else kept).astype(np.float64)
+        else:  # a matrix in the packed layout of the kernels: the stored values, rounded as it keeps them
+            stored[name] = torch.from_numpy(value).to(placed[name].dtype).float().numpy().astype(np.float64)
     part.bind_named(placed)
     return stored
 
