@@ -744,15 +744,66 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
     DL_STAMP(15);
 }
 
+// Four columns of a pending row with their sums taken: eight partial rows asked for at a time.
+__device__ __forceinline__ f32x4 pending_piece(const PendingSum& in, int row_index, int width, int piece) {
+    f32x4 value = load4(in.base + (size_t)row_index * width + 4 * piece);
+    if (in.bias) value += load4(in.bias + 4 * piece);
+    for (int s0 = 0; s0 < in.n_partials; s0 += 8) {
+        f32x4 part[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            part[u] = load4(in.partials + ((size_t)min(s0 + u, in.n_partials - 1) * in.rows + row_index) * width + 4 * piece);
+#pragma unroll
+        for (int u = 0; u < 8; u++) value += part[u] * (s0 + u < in.n_partials ? 1.0f : 0.0f);
+    }
+    return value;
+}
+
 // out = base + bias + the partial rows: the pending stream as plain rows, for whatever does not
 // take it pending. grid (pieces of 256 x 4 columns, rows).
 __global__ __launch_bounds__(256) void pending_sum_kernel(PendingSum in, float* __restrict__ out, int width) {
     const int piece = blockIdx.x * 256 + threadIdx.x, row_index = blockIdx.y;
     if (piece * 4 >= width) return;
-    f32x4 row = load4(in.base + (size_t)row_index * width + 4 * piece);
-    if (in.bias) row += load4(in.bias + 4 * piece);
-    for (int s = 0; s < in.n_partials; s++) row += load4(in.partials + ((size_t)s * in.rows + row_index) * width + 4 * piece);
-    *reinterpret_cast<f32x4*>(out + (size_t)row_index * width + 4 * piece) = row;
+    *reinterpret_cast<f32x4*>(out + (size_t)row_index * width + 4 * piece) = pending_piece(in, row_index, width, piece);
+}
+
+// Row LayerNorm of pending rows (the sums are taken on the way in): a block of four waves a row,
+// the row kept in LDS; row_index, if given, names the pending row of each output row. Centred, in
+// 32-bit, like the norm of plain rows (elementwise.hip).
+template <typename OutT>
+__global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, const int* __restrict__ row_index,
+                                                                const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                                OutT* __restrict__ out, int width, float eps) {
+    extern __shared__ f32x4 row_pieces[];  // width / 4
+    __shared__ float red[2][4];
+    const int tid = threadIdx.x, n_pieces = width / 4;
+    const int source = row_index ? row_index[blockIdx.x] : blockIdx.x;
+    float sum = 0.0f;
+    for (int piece = tid; piece < n_pieces; piece += 256) {
+        f32x4 value = pending_piece(in, source, width, piece);
+        row_pieces[piece] = value;
+        sum += (value[0] + value[1]) + (value[2] + value[3]);
+    }
+    sum = wave_total(sum);
+    if (tid % WAVE == 0) red[0][tid / WAVE] = sum;
+    __syncthreads();
+    const float n = (float)width;
+    const float mean = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / n;
+    float squares = 0.0f;
+    for (int piece = tid; piece < n_pieces; piece += 256) {
+        f32x4 d = row_pieces[piece] - mean;
+        squares += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+    }
+    squares = wave_total(squares);
+    if (tid % WAVE == 0) red[1][tid / WAVE] = squares;
+    __syncthreads();
+    const float inverse_stddev = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / n + eps);
+    for (int piece = tid; piece < n_pieces; piece += 256) {
+        f32x4 y = (row_pieces[piece] - mean) * inverse_stddev * load4(gamma + 4 * piece) + load4(beta + 4 * piece);
+        OutT* at = out + (size_t)blockIdx.x * width + 4 * piece;
+        if constexpr (sizeof(OutT) == 2) store_bf16x4(at, y);
+        else *reinterpret_cast<f32x4*>(at) = y;
+    }
 }
 
 int check_pending(const char* what, const float* base, const float* partials, int n_partials, int width) {
@@ -877,6 +928,27 @@ MLLM_API int mllm_pending_sum(const float* base, const float* partials, const fl
     dim3 grid((width / 4 + 255) / 256, n_rows);
     pending_sum_kernel<<<grid, 256, 0, stream>>>(in, out, width);
     return mllm_check_launch("pending_sum");
+}
+
+
+// LayerNorm of pending rows; row_index (or null) names the pending row of each of the n_rows output rows.
+MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, const float* pending_bias, int n_partials,
+                                    int pending_rows, const int* row_index, const float* gamma, const float* beta, void* out,
+                                    int n_rows, int width, float eps, int out_dtype, hipStream_t stream) {
+    MLLM_REQUIRE(base != nullptr && out != nullptr, "pending_layernorm: no rows");
+    MLLM_REQUIRE(n_partials >= 0 && (n_partials == 0 || partials != nullptr), "pending_layernorm: %d partial rows without memory", n_partials);
+    MLLM_REQUIRE(width > 0 && width % 4 == 0 && width <= 32768, "pending_layernorm: width %d is not a multiple of 4 up to 32768", width);
+    MLLM_REQUIRE(n_rows >= 0 && pending_rows >= 0 && eps > 0.0f, "pending_layernorm: bad sizes");
+    if (n_rows == 0) return 0;
+    PendingSum in{base, partials, pending_bias, n_partials, pending_rows};
+    const size_t lds = (size_t)width * 4;
+    if (out_dtype == MLLM_F32)
+        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, width, eps);
+    else if (out_dtype == MLLM_BF16)
+        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, width, eps);
+    else
+        MLLM_REQUIRE(false, "pending_layernorm: unknown output dtype %d", out_dtype);
+    return mllm_check_launch("pending_layernorm");
 }
 
 #ifdef MLLM_PHASE_STAMPS

@@ -4,13 +4,23 @@
 
 // out[t, :] = wte[token[t], :] + wpe[position[t], :]   (reference: engine/src/embedding.cu:7-27,
 // per-row positions as in embed_batch_kernel :89-104). One block per row; a negative token marks
-// a padding row, which is filled with zeros.
+// a padding row, which is filled with zeros. With `sources`, the token of a row whose source is
+// not negative is taken from token_slots[source] (a token the sampler left on the device, as the
+// reference's queued decode step does: engine/src/gpt2_gpu.cu:441-447) and written into tokens.
 template <typename T>
-__global__ void embed_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+__global__ void embed_kernel(int* __restrict__ tokens, const int* __restrict__ positions,
+                             const int* __restrict__ sources, const int* __restrict__ token_slots,
                              const T* __restrict__ wte, const T* __restrict__ wpe,
                              float* __restrict__ out, int width) {
     int row = blockIdx.x;
     int token = tokens[row];
+    if (sources) {
+        int source = sources[row];
+        if (source >= 0) {
+            token = token_slots[source];
+            if (threadIdx.x == 0) tokens[row] = token;
+        }
+    }
     float* out_row = out + (size_t)row * width;
     if (token < 0) {
         for (int i = threadIdx.x; i < width; i += blockDim.x) out_row[i] = 0.0f;
@@ -22,16 +32,18 @@ __global__ void embed_kernel(const int* __restrict__ tokens, const int* __restri
         out_row[i] = to_float(token_row[i]) + to_float(position_row[i]);
 }
 
-MLLM_API int mllm_embed(const int* tokens, const int* positions, const void* wte, const void* wpe,
-                        float* out, int n_rows, int width, int table_dtype, hipStream_t stream) {
+MLLM_API int mllm_embed(int* tokens, const int* positions, const int* sources, const int* token_slots,
+                        const void* wte, const void* wpe, float* out, int n_rows, int width, int table_dtype,
+                        hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "embed: bad sizes rows=%d width=%d", n_rows, width);
+    MLLM_REQUIRE(sources == nullptr || token_slots != nullptr, "embed: sources without token slots");
     if (n_rows == 0) return 0;
     int threads = width >= 256 ? 256 : 64;
     if (table_dtype == MLLM_F32)
-        embed_kernel<float><<<n_rows, threads, 0, stream>>>(tokens, positions, (const float*)wte,
+        embed_kernel<float><<<n_rows, threads, 0, stream>>>(tokens, positions, sources, token_slots, (const float*)wte,
                                                             (const float*)wpe, out, width);
     else if (table_dtype == MLLM_BF16)
-        embed_kernel<bf16_t><<<n_rows, threads, 0, stream>>>(tokens, positions, (const bf16_t*)wte,
+        embed_kernel<bf16_t><<<n_rows, threads, 0, stream>>>(tokens, positions, sources, token_slots, (const bf16_t*)wte,
                                                              (const bf16_t*)wpe, out, width);
     else
         MLLM_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);

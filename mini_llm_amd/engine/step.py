@@ -15,7 +15,6 @@ buffer per bucket that is overwritten before each replay."""
 from __future__ import annotations
 
 from ..cache import CacheManager, OutOfPages
-from ..ops import kernels
 from .batch import BatchStaging, DecodeBatchBuilder, StepBatch, StepEntry, build_step_batch
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -101,9 +100,7 @@ class ModelRunner:
 
     def forward(self, batch, resolve: bool = True):
         """Tokens that come from last-token slots are fetched on the device, then the model runs."""
-        if resolve:
-            kernels.resolve_tokens(batch.tokens, batch.token_sources, self.cache.last_token)
-        return self.model.forward(batch, self.cache)
+        return self.model.forward(batch, self.cache, resolve_tokens=resolve)
 
     def _graph_for(self, entries):
         if not self.use_graphs or len(entries) > GRAPH_BUCKETS[-1]:

@@ -101,10 +101,13 @@ class Model(Part):
                 out[call.cache] = need
         return out
 
-    def forward(self, batch, cache):
+    def forward(self, batch, cache, resolve_tokens: bool = False):
         """The whole step: embeds the batch's tokens, runs the schedule over the cache, and
-        returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only."""
-        hidden = self.embedding.forward(batch.tokens, batch.positions, self.position_encoding)
+        returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only. With
+        ``resolve_tokens`` the rows that name a last-token slot take their token from it."""
+        hidden = self.embedding.forward(batch.tokens, batch.positions, self.position_encoding,
+                                        token_sources=batch.token_sources if resolve_tokens else None,
+                                        token_slots=cache.last_token if resolve_tokens else None)
         for call in self.schedule:
             block = self.blocks[call.block]
             if not block.takes_pending:
@@ -112,7 +115,8 @@ class Model(Part):
             hidden = block.forward(hidden, cache.layer_context(batch, call))
         if batch.n_logit_rows == 0:
             return None
-        hidden = kernels.settle(hidden)
+        if not self.final_norm.takes_pending:
+            hidden = kernels.settle(hidden)
         # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
         normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
         return self.head.forward(normed)

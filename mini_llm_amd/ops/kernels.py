@@ -56,8 +56,10 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def embed(tokens, positions, wte, wpe, out=None):
-    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32. A negative token gives a zero row."""
+def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots=None):
+    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32. A negative token gives a zero row.
+    With ``token_sources`` and ``token_slots`` the token of a row whose source is not negative is
+    token_slots[source]; it is also written into ``tokens``."""
     _device_tensor(tokens, "tokens", torch.int32, 1)
     _device_tensor(positions, "positions", torch.int32, 1)
     _device_tensor(wte, "wte", dim=2)
@@ -65,30 +67,47 @@ def embed(tokens, positions, wte, wpe, out=None):
     n, width = tokens.shape[0], wte.shape[1]
     _require(positions.shape[0] == n, "tokens and positions differ in length")
     _require(wpe.shape[1] == width, "wte and wpe differ in width")
+    if token_sources is not None:
+        _device_tensor(token_sources, "token_sources", torch.int32, 1)
+        _device_tensor(token_slots, "token_slots", torch.int32, 1)
+        _require(token_sources.shape[0] >= n, "fewer sources than tokens")
     if out is None:
         out = torch.empty((n, width), dtype=torch.float32, device=tokens.device)
     _device_tensor(out, "out", torch.float32, 2)
     _require(tuple(out.shape) == (n, width), "out has the wrong shape")
-    check(library().mllm_embed(_ptr(tokens), _ptr(positions), _ptr(wte), _ptr(wpe), _ptr(out), n, width, _code(wte.dtype), _stream()))
+    check(library().mllm_embed(_ptr(tokens), _ptr(positions), _ptr(token_sources), _ptr(token_slots if token_sources is not None else None),
+                               _ptr(wte), _ptr(wpe), _ptr(out), n, width, _code(wte.dtype), _stream()))
     return out
 
 
 def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None):
-    """Row LayerNorm of float32 rows; ``row_index`` (int32) picks the input row of each output row."""
-    _device_tensor(x, "x", torch.float32, 2)
-    width = x.shape[1]
+    """Row LayerNorm of float32 rows, plain or pending (PendingRows: the sums are taken on the way
+    in); ``row_index`` (int32) picks the input row of each output row."""
+    pending = isinstance(x, PendingRows)
+    if pending and x.base.shape[1] % 4:
+        x, pending = settle(x), False
+    if pending:
+        base, partials, bias, n_partials = _pending(x)
+    else:
+        _device_tensor(x, "x", torch.float32, 2)
+        base = x
+    width = base.shape[1]
     _device_tensor(gamma, "gamma", torch.float32, 1)
     _device_tensor(beta, "beta", torch.float32, 1)
     _require(gamma.shape[0] == width and beta.shape[0] == width, "gamma/beta do not match the row width")
-    n = x.shape[0]
+    n = base.shape[0]
     if row_index is not None:
         _device_tensor(row_index, "row_index", torch.int32, 1)
         n = row_index.shape[0]
     if out is None:
-        out = torch.empty((n, width), dtype=out_dtype, device=x.device)
+        out = torch.empty((n, width), dtype=out_dtype, device=base.device)
     _device_tensor(out, "out", out_dtype, 2)
     _require(tuple(out.shape) == (n, width), "out has the wrong shape")
-    check(library().mllm_layernorm(_ptr(x), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
+    if pending:
+        check(library().mllm_pending_layernorm(_ptr(base), _ptr(partials), _ptr(bias), n_partials, base.shape[0], _ptr(row_index), _ptr(gamma),
+                                               _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
+    else:
+        check(library().mllm_layernorm(_ptr(base), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
     return out
 
 

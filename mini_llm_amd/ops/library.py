@@ -15,7 +15,7 @@ _library: ctypes.CDLL | None = None
 
 P = c_void_p
 _SIGNATURES = {
-    "mllm_embed": [P, P, P, P, P, c_int, c_int, c_int, P],
+    "mllm_embed": [P, P, P, P, P, P, P, c_int, c_int, c_int, P],
     "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
@@ -38,6 +38,7 @@ _SIGNATURES = {
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_decode_mlp_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pending_sum": [P, P, P, c_int, P, c_int, c_int, P],
+    "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_float, c_int, P],
 }
 
 

@@ -83,6 +83,9 @@ class LayerContext:
 
 
 class Norm(Part):
+    # True if ``forward`` also takes rows whose last sums are pending (ops.kernels.PendingRows)
+    takes_pending = False
+
     def forward(self, x, out_dtype, row_index=None):
         """x: [rows, width] float32 -> [rows or len(row_index), width] of out_dtype."""
         raise NotImplementedError

@@ -15,12 +15,13 @@ class TokenEmbedding(Part):
     def tensor_specs(self):
         return {"weight": TensorSpec((self.vocab_size, self.width), TABLE, Normal(0.02))}
 
-    def forward(self, tokens, positions, position_encoding: PositionEncoding | None):
+    def forward(self, tokens, positions, position_encoding: PositionEncoding | None, token_sources=None, token_slots=None):
         """[rows, width] float32: token rows, with the position rows added when the encoding
-        is one that enters at the embedding."""
+        is one that enters at the embedding. ``token_sources`` / ``token_slots``: rows whose token
+        is still on the device, in the slot the sampler left it in (kernels.embed)."""
         if position_encoding is None or position_encoding.stage != "embedding":
             raise NotImplementedError("only encodings added at the embedding have a kernel here")
-        return kernels.embed(tokens, positions, self.weight, position_encoding.weight)
+        return kernels.embed(tokens, positions, self.weight, position_encoding.weight, token_sources=token_sources, token_slots=token_slots)
 
 
 class TiedHead(Part):

@@ -9,6 +9,8 @@ from .base import Norm, register_part
 
 
 class LayerNorm(Norm):
+    takes_pending = True
+
     def __init__(self, width: int, eps: float):
         self.width, self.eps = width, eps
         self.weight = None

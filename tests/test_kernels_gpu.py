@@ -562,3 +562,30 @@ def test_layer_kernels_refuse_what_they_do_not_take(K):
     ones = torch.ones(96, device=DEV)
     with pytest.raises(K.OperandError):
         K.decode_mlp_half(x, ones, ones, 1e-5, K.pack_matrix(torch.zeros((100, 96), device=DEV).bfloat16()), None, K.pack_matrix(torch.zeros((96, 100), device=DEV).bfloat16()), None)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width,n_partials,with_bias", [(1, 64, 0, False), (5, 96, 3, True), (9, 768, 48, True), (3, 1032, 17, False), (2, 2500, 9, True)])
+def test_layernorm_of_pending_rows(K, out_dtype, rows, width, n_partials, with_bias):
+    # the sums are taken on the way into the norm; row_index picks and repeats rows
+    rng = np.random.default_rng(rows + width)
+    hidden, total = _pending_rows(K, rng, rows, width, n_partials, with_bias)
+    gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
+    index = np.array([rows - 1, 0, rows - 1], dtype=np.int32)
+    tol = 1e-5 if out_dtype == torch.float32 else 1e-2
+    out = K.layernorm(hidden, dev(gamma), dev(beta), 2e-5, out_dtype=out_dtype)
+    np.testing.assert_allclose(host(out), P.layernorm(total, gamma, beta, 2e-5), rtol=tol, atol=tol)
+    out = K.layernorm(hidden, dev(gamma), dev(beta), 2e-5, out_dtype=out_dtype, row_index=dev(index, torch.int32))
+    np.testing.assert_allclose(host(out), P.layernorm(total[index], gamma, beta, 2e-5), rtol=tol, atol=tol)
+    np.testing.assert_allclose(host(K.settle(hidden)), total, rtol=1e-5, atol=1e-5)
+
+
+def test_embed_takes_tokens_from_slots(K):
+    # rows whose source is not negative take their token from the slot the sampler left it in
+    rng = np.random.default_rng(4)
+    wte, wpe = rng.standard_normal((50, 96)).astype(np.float32), rng.standard_normal((16, 96)).astype(np.float32)
+    tokens = dev([7, -5, 9, 11], torch.int32)
+    out = K.embed(tokens, dev([0, 3, 1, 15], torch.int32), dev(wte), dev(wpe), token_sources=dev([-1, 2, -1, 0], torch.int32),
+                  token_slots=dev([40, 41, 42], torch.int32))
+    assert tokens.tolist() == [7, 42, 9, 40]
+    np.testing.assert_allclose(host(out), np.stack([wte[t] + wpe[p] for t, p in zip([7, 42, 9, 40], [0, 3, 1, 15])]), rtol=1e-6, atol=1e-6)
