@@ -6,7 +6,7 @@
 // per-row positions as in embed_batch_kernel :89-104). One block per row; a negative token marks
 // a padding row, which is filled with zeros. With `sources`, the token of a row whose source is
 // not negative is taken from token_slots[source] (a token the sampler left on the device, as the
-// reference's queued decode step does: engine/src/gpt2_gpu.cu:441-447) and written into tokens.
+// reference's queued decode reads its token: engine/src/gpt2_gpu_greedy.cu:94-107) and written into tokens.
 template <typename T>
 __global__ void embed_kernel(int* __restrict__ tokens, const int* __restrict__ positions,
                              const int* __restrict__ sources, const int* __restrict__ token_slots,
@@ -168,21 +168,4 @@ MLLM_API int mllm_add(const float* a, const void* b, float* out, long long n, in
     else
         MLLM_REQUIRE(false, "add: unknown dtype %d", b_dtype);
     return mllm_check_launch("add");
-}
-
-// tokens[row] = token_slots[sources[row]] where sources[row] >= 0: a request's next token taken from
-// its last-token slot on the device, where the sampler of the previous step left it (the
-// reference's queued decode reads its token the same way: engine/src/gpt2_gpu_greedy.cu:94-107).
-__global__ void resolve_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ sources,
-                                      const int* __restrict__ token_slots, int n_rows) {
-    int row = blockIdx.x * blockDim.x + threadIdx.x;
-    if (row < n_rows && sources[row] >= 0) tokens[row] = token_slots[sources[row]];
-}
-
-MLLM_API int mllm_resolve_tokens(int* tokens, const int* sources, const int* token_slots, int n_rows,
-                                 hipStream_t stream) {
-    MLLM_REQUIRE(n_rows >= 0, "resolve_tokens: negative size");
-    if (n_rows == 0) return 0;
-    resolve_tokens_kernel<<<ceil_div(n_rows, 256), 256, 0, stream>>>(tokens, sources, token_slots, n_rows);
-    return mllm_check_launch("resolve_tokens");
 }

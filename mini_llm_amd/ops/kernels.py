@@ -340,15 +340,6 @@ def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=N
     return out
 
 
-def resolve_tokens(tokens, sources, token_slots):
-    """tokens[row] = token_slots[sources[row]] where sources[row] >= 0 (in place)."""
-    _device_tensor(tokens, "tokens", torch.int32, 1)
-    _device_tensor(sources, "sources", torch.int32, 1)
-    _device_tensor(token_slots, "token_slots", torch.int32, 1)
-    _require(sources.shape[0] >= tokens.shape[0], "fewer sources than tokens")
-    check(library().mllm_resolve_tokens(_ptr(tokens), _ptr(sources), _ptr(token_slots), tokens.shape[0], _stream()))
-
-
 # -- a whole layer for rows that bring one token each -------------------------------------------------
 @dataclass
 class PendingRows:

@@ -32,7 +32,6 @@ _SIGNATURES = {
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
-    "mllm_resolve_tokens": [P, P, P, c_int, P],
     "mllm_decode_layer_supported": [c_int, c_int, c_int, c_int],
     "mllm_decode_attention_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, P, P, P, P, P, c_int, P,
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
