@@ -103,6 +103,43 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// The sum over each aligned group of N neighbouring lanes (N a power of two), in every lane of the
+// group: data-parallel steps inside rows of 16 lanes, the LDS crossbar only between rows.
+template <int N>
+__device__ __forceinline__ float lanes_sum(float v) {
+    if constexpr (N >= 2) v += dpp_moved<0xB1>(v);
+    if constexpr (N >= 4) v += dpp_moved<0x4E>(v);
+    if constexpr (N >= 8) v += dpp_moved<0x141>(v);
+    if constexpr (N >= 16) v += dpp_moved<0x140>(v);
+    if constexpr (N >= 32) v += __shfl_xor(v, 16, WAVE);
+    if constexpr (N >= 64) v += __shfl_xor(v, 32, WAVE);
+    return v;
+}
+
+// The sum over the lanes of a row of 16 that lie STEP apart (STEP a power of two), in each of
+// them: rotations of the row by STEP, 2 STEP, ...
+template <int STEP>
+__device__ __forceinline__ float row_strided_sum(float v) {
+    if constexpr (STEP <= 1) v += dpp_moved<0x121>(v);
+    if constexpr (STEP <= 2) v += dpp_moved<0x122>(v);
+    if constexpr (STEP <= 4) v += dpp_moved<0x124>(v);
+    if constexpr (STEP <= 8) v += dpp_moved<0x128>(v);
+    return v;
+}
+
+// The maximum over a wave, in every lane: four steps inside the rows, then the four rows' maxima.
+__device__ __forceinline__ float wave_max_total(float v) {
+    v = fmaxf(v, dpp_moved<0xB1>(v));
+    v = fmaxf(v, dpp_moved<0x4E>(v));
+    v = fmaxf(v, dpp_moved<0x141>(v));
+    v = fmaxf(v, dpp_moved<0x140>(v));
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 // tanh form of GELU, in the reference's order of operations (engine/include/gelu_math.h:6-11).
 __device__ __forceinline__ float gelu_tanh(float x) {
     const float coefficient = 0.7978845608f;

@@ -83,6 +83,73 @@ __device__ __forceinline__ void keep_order() { __builtin_amdgcn_sched_barrier(0)
 // data between the waves of a block here, so nothing more is needed.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// A wave's share of the q/k/v product of one (token, head): 3*HD rows of the matrix in tiles of 16,
+// each tile's k range cut into DL_KSPLIT shares; a (tile, share) pair is a unit. The wave owns the
+// units first_unit, first_unit + 8, ... (n_units of them), works on AT_ONCE at a time and keeps
+// ROUND k steps of each in flight. The shares' sums meet in LDS (qkv_part).
+template <int HD, int AT_ONCE>
+struct QkvShare {
+    static constexpr int ROW_TILES = 3 * HD / 16, ALL_UNITS = ROW_TILES * DL_KSPLIT, ROUND = 6;
+    const bf16_t* w_qkv;
+    int head, kv_head, q_width, kv_width, n_steps, lane, first_unit;
+    int w_at[AT_ONCE], part_of[AT_ONCE], tile_of[AT_ONCE];
+    Vec16 w_piece[AT_ONCE][ROUND];
+
+    __device__ __forceinline__ void choose(int u0) {
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++) {
+            int unit = min(first_unit + 8 * (u0 + u), ALL_UNITS - 1);  // beyond the last: computed again, not kept
+            tile_of[u] = unit % ROW_TILES, part_of[u] = unit / ROW_TILES;
+            int local = tile_of[u] * 16, which = local / HD, within = local % HD;  // HD is a multiple of 16: a tile lies in one of q, k, v
+            int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
+            w_at[u] = w_row / 16;
+        }
+    }
+    __device__ __forceinline__ void ask(int i0) {
+#pragma unroll
+        for (int u = 0; u < AT_ONCE; u++)
+#pragma unroll
+            for (int j = 0; j < ROUND; j++) {
+                int step = min(part_of[u] + DL_KSPLIT * (i0 + j), n_steps - 1);
+                w_piece[u][j] = load16<Vec16>(w_qkv + packed_offset<bf16_t>(w_at[u], step, n_steps, 0), lane * 16);
+            }
+    }
+    // All N_UNITS units; `asked`: choose(0) and ask(0) have been called already (the first round has
+    // been under way for a while). x_hat: the normed row in LDS, zeros beyond the width.
+    template <int N_UNITS>
+    __device__ __forceinline__ void run(bool asked, const bf16_t* x_hat, float (*qkv_part)[3 * HD]) {
+        const int row16 = lane % 16, quad = lane / 16;
+        const int steps_per_unit = (n_steps + DL_KSPLIT - 1) / DL_KSPLIT;
+#pragma unroll 1
+        for (int u0 = 0; u0 < N_UNITS; u0 += AT_ONCE) {
+            f32x4 acc[AT_ONCE];
+#pragma unroll
+            for (int u = 0; u < AT_ONCE; u++) acc[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (u0 > 0 || !asked) choose(u0);
+#pragma unroll 1
+            for (int i0 = 0; i0 < steps_per_unit; i0 += ROUND) {
+                if (u0 > 0 || i0 > 0 || !asked) ask(i0);
+#pragma unroll
+                for (int u = 0; u < AT_ONCE; u++)
+#pragma unroll
+                    for (int j = 0; j < ROUND; j++) {
+                        int step = part_of[u] + DL_KSPLIT * (i0 + j);
+                        Vec16 w = mask16(w_piece[u][j], step < n_steps);
+                        bf16x8 x = *reinterpret_cast<const bf16x8*>(x_hat + min(step, n_steps - 1) * 32 + quad * 8);
+                        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc[u], 0, 0, 0);
+                    }
+            }
+            // every column of the product is this one token; column 0 is kept
+#pragma unroll
+            for (int u = 0; u < AT_ONCE; u++)
+                if (row16 == 0 && first_unit + 8 * (u0 + u) < ALL_UNITS) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) qkv_part[part_of[u]][tile_of[u] * 16 + 4 * quad + r] = acc[u][r];
+                }
+        }
+    }
+};
+
 // ------------------------------------------------------------------------------------------------
 // norm -> q/k/v -> cache write -> attention over the cache -> this head's share of the output
 // product. grid (n_heads, tokens), 1024 threads in two roles:
@@ -111,21 +178,28 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     typedef KeySweep<bf16_t, HD> Sweep;
     constexpr int VEC = Sweep::VEC, LPR = Sweep::LPR, RPI = Sweep::RPI, KPI = Sweep::KPI;
     constexpr int ROW_TILES = 3 * HD / 16;
-    constexpr int UNITS = (ROW_TILES * DL_KSPLIT + DL_PROJECT_WAVES - 1) / DL_PROJECT_WAVES;  // (tile, k share) pairs a wave owns
-    constexpr int AT_ONCE = UNITS < 2 ? UNITS : 2;  // of which it works on so many at a time,
-    constexpr int ROUND = 12 / AT_ONCE;             // with so many k steps of each in flight
+    // the q/k/v product: two thirds of its units go to the waves that project, one third to the
+    // waves that attend (which have nothing else to do while they wait for the query)
+    constexpr int ALL_UNITS = ROW_TILES * DL_KSPLIT;
+    constexpr int UNITS_PROJECT = (2 * ALL_UNITS / 3 + 7) / 8, UNITS_ATTEND = (ALL_UNITS - 8 * UNITS_PROJECT + 7) / 8;
+    constexpr int AT_ONCE_PROJECT = UNITS_PROJECT < 2 ? UNITS_PROJECT : 2, AT_ONCE_ATTEND = UNITS_ATTEND < 2 ? UNITS_ATTEND : 2;
+    static_assert(UNITS_ATTEND >= 1 && 8 * (UNITS_PROJECT + UNITS_ATTEND) >= ALL_UNITS, "every unit of the q/k/v product has a wave");
     constexpr int HD_PAD = (HD + 31) / 32 * 32;
     constexpr int OUT_STEPS = HD_PAD / 32, OUT_GROUP = OUT_STEPS <= 2 ? 12 / OUT_STEPS : (OUT_STEPS <= 4 ? 2 : 1);
     constexpr int ROWS_PER_THREAD = (3 * HD + DL_PROJECT_THREADS - 1) / DL_PROJECT_THREADS;
     constexpr int MAX_PIECES = DL_MAX_WIDTH / 4, PIECES_PER_LANE = MAX_PIECES / WAVE;
     constexpr int NEAR_KEYS = DL_ATTEND_WAVES * KPI;  // keys the waves that attend can ask for in one go
+    // a wave leaves one (max, sum, output) triple for each of its rows of 16 lanes (for each group
+    // of lanes, if a group is wider): adding them up in LDS is cheaper than across the rows of a wave
+    constexpr int MERGE_SPAN = LPR < 16 ? 16 : LPR, MERGE_ENTRIES = WAVE / MERGE_SPAN;
 
     __shared__ f32x4 stage[DL_ATTEND_WAVES][MAX_PIECES];
     __shared__ f32x4 row_lds[MAX_PIECES];
     __shared__ __attribute__((aligned(16))) bf16_t x_hat[DL_MAX_WIDTH];
     __shared__ float qkv_part[DL_KSPLIT][3 * HD];
     __shared__ float qkv_row[3][HD];  // q, k, v of this token and head, rounded as the cache holds them
-    __shared__ float merged[DL_WAVES][HD + 2];
+    __shared__ float merged[DL_WAVES * MERGE_ENTRIES][HD + 2];
+    __shared__ float merge_weight[HD_PAD / WAVE > 0 ? HD_PAD / WAVE : 1][WAVE];
     __shared__ __attribute__((aligned(16))) bf16_t mixed[HD_PAD];
 
     const int tid = threadIdx.x, lane = tid % WAVE;
@@ -215,9 +289,14 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         sweep.look_up(key_page, table, page_shift, begin, end, spare_key, lane);  // the table's answer is under way early
         lds_barrier();  // 1: the eight sums are in LDS
         lds_barrier();  // 2
-        lds_barrier();  // 3
+        lds_barrier();  // 3: the normed row is in LDS
+        // ---- their share of the q/k/v product (measured: asking for the matrix before the meetings
+        // above, or for the keys before the matrix, only delays the other waves or costs registers)
+        QkvShare<HD, AT_ONCE_ATTEND> qkv{w_qkv, head, kv_head, q_width, kv_width, (width + 31) / 32, lane, 8 * UNITS_PROJECT + role_wave};
+        qkv.template run<UNITS_ATTEND>(false, x_hat, qkv_part);
         // ---- their shares of the cached keys and values, asked for now (the pages are known by
         // now); they ask for nothing else until they have used them
+        keep_order();
         typename Sweep::Fetched fetched;
         sweep.fetch_rows(fetched, key_page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
         DL_STAMP(20);
@@ -232,14 +311,17 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         // above down into a conditional block, behind the meetings of the waves
         sweep.template consume<true>(fetched, qf, begin, end, lane);
         if (wave == DL_PROJECT_WAVES) sweep.one_key(qf, qkv_row[1], qkv_row[2], lane);  // the token's own key and value, from LDS
-        sweep.merge_groups();
-        if (lane < LPR) {
+        sweep.merge_inside_rows();
+        {
+            const int entry = wave * MERGE_ENTRIES + lane / MERGE_SPAN;
+            if (lane % MERGE_SPAN < LPR) {
 #pragma unroll
-            for (int i = 0; i < VEC; i++) merged[wave][sub * VEC + i] = sweep.o[i];
-        }
-        if (lane == 0) {
-            merged[wave][HD] = sweep.running_max;
-            merged[wave][HD + 1] = sweep.running_sum;
+                for (int i = 0; i < VEC; i++) merged[entry][sub * VEC + i] = sweep.o[i];
+            }
+            if (lane % MERGE_SPAN == 0) {
+                merged[entry][HD] = sweep.running_max;
+                merged[entry][HD + 1] = sweep.running_sum;
+            }
         }
         DL_STAMP(22);
         lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
@@ -261,33 +343,9 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
         qkv_bias[i] = (b_qkv ? b_qkv : gamma)[b_qkv ? w_row : 0];
     }
-    // q, k, v of this head: 3*HD rows of the matrix in tiles of 16, each tile's k range shared by
-    // DL_KSPLIT waves; a wave owns UNITS (tile, share) pairs and works on AT_ONCE of them at a time
-    const int n_steps = (width + 31) / 32;
-    const int steps_per_unit = (n_steps + DL_KSPLIT - 1) / DL_KSPLIT;
-    int w_at[AT_ONCE], part_of[AT_ONCE], tile_of[AT_ONCE];
-    Vec16 w_piece[AT_ONCE][ROUND];
-    auto choose_units = [&](int u0) {
-#pragma unroll
-        for (int u = 0; u < AT_ONCE; u++) {
-            int unit = min(wave + DL_PROJECT_WAVES * (u0 + u), ROW_TILES * DL_KSPLIT - 1);  // beyond the last: computed again, not kept
-            tile_of[u] = unit % ROW_TILES, part_of[u] = unit / ROW_TILES;
-            int local = tile_of[u] * 16, which = local / HD, within = local % HD;  // HD is a multiple of 16: a tile lies in one of q, k, v
-            int w_row = which == 0 ? head * HD + within : q_width + (which - 1) * kv_width + kv_head * HD + within;
-            w_at[u] = w_row / 16;
-        }
-    };
-    auto ask_for_round = [&](int i0) {
-#pragma unroll
-        for (int u = 0; u < AT_ONCE; u++)
-#pragma unroll
-            for (int j = 0; j < ROUND; j++) {
-                int step = min(part_of[u] + DL_KSPLIT * (i0 + j), n_steps - 1);
-                w_piece[u][j] = load16<Vec16>(w_qkv + packed_offset<bf16_t>(w_at[u], step, n_steps, 0), lane * 16);
-            }
-    };
-    choose_units(0);
-    ask_for_round(0);
+    QkvShare<HD, AT_ONCE_PROJECT> qkv{w_qkv, head, kv_head, q_width, kv_width, (width + 31) / 32, lane, wave};
+    qkv.choose(0);
+    qkv.ask(0);
     if (request < 0) {
         leave_zeros();
         return;
@@ -339,33 +397,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     int far_page[Sweep::UNROLL];  // the pages of this wave's share of the far keys (of the spare key, if there are none)
     sweep.look_up(far_page, table, page_shift, begin, end, spare_key, lane);
 
-#pragma unroll 1
-    for (int u0 = 0; u0 < UNITS; u0 += AT_ONCE) {
-        f32x4 acc[AT_ONCE];
-#pragma unroll
-        for (int u = 0; u < AT_ONCE; u++) acc[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        if (u0 > 0) choose_units(u0);
-#pragma unroll 1
-        for (int i0 = 0; i0 < steps_per_unit; i0 += ROUND) {
-            if (u0 > 0 || i0 > 0) ask_for_round(i0);  // the first round has been under way since the start
-#pragma unroll
-            for (int u = 0; u < AT_ONCE; u++)
-#pragma unroll
-                for (int j = 0; j < ROUND; j++) {
-                    int step = part_of[u] + DL_KSPLIT * (i0 + j);
-                    Vec16 w = mask16(w_piece[u][j], step < n_steps);
-                    bf16x8 x = *reinterpret_cast<const bf16x8*>(x_hat + min(step, n_steps - 1) * 32 + quad * 8);
-                    acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&w), x, acc[u], 0, 0, 0);
-                }
-        }
-        // every column of the product is this one token; column 0 is kept
-#pragma unroll
-        for (int u = 0; u < AT_ONCE; u++)
-            if (row16 == 0 && wave + DL_PROJECT_WAVES * (u0 + u) < ROW_TILES * DL_KSPLIT) {
-#pragma unroll
-                for (int r = 0; r < 4; r++) qkv_part[part_of[u]][tile_of[u] * 16 + 4 * quad + r] = acc[u][r];
-            }
-    }
+    qkv.template run<UNITS_PROJECT>(true, x_hat, qkv_part);
     auto finish_qkv_rows = [&]() {  // sums of the k shares, bias, rounding; k and v go into their cache slot
 #pragma unroll
         for (int i = 0; i < ROWS_PER_THREAD; i++) {
@@ -397,7 +429,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         sweep.template consume<true>(fetched, qf, begin, end, lane);  // not under a further condition, as above
         if (begin + KPI < end)  // a context longer than one round of every wave of the block covers
             sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin + KPI, end, lane);
-        sweep.merge_groups();
+        sweep.merge_inside_rows();
     } else {
         lds_barrier();  // 4
         finish_qkv_rows();
@@ -405,13 +437,16 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         sweep.init();
     }
     DL_STAMP(4);
-    if (lane < LPR) {
+    {
+        const int entry = wave * MERGE_ENTRIES + lane / MERGE_SPAN;
+        if (lane % MERGE_SPAN < LPR) {
 #pragma unroll
-        for (int i = 0; i < VEC; i++) merged[wave][sub * VEC + i] = sweep.o[i];
-    }
-    if (lane == 0) {
-        merged[wave][HD] = sweep.running_max;
-        merged[wave][HD + 1] = sweep.running_sum;
+            for (int i = 0; i < VEC; i++) merged[entry][sub * VEC + i] = sweep.o[i];
+        }
+        if (lane % MERGE_SPAN == 0) {
+            merged[entry][HD] = sweep.running_max;
+            merged[entry][HD + 1] = sweep.running_sum;
+        }
     }
     // the output product's rows are asked for now: they are needed last
     keep_order();
@@ -429,21 +464,25 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     }
     lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
     DL_STAMP(5);
-    if (tid < HD_PAD) {  // HD_PAD <= 256 threads; the mixed row lies where its columns lie in the chunks of w_out, zeros around it
+    if (wave < (HD_PAD + WAVE - 1) / WAVE) {  // whole waves (the wave sums below need every lane); the mixed row lies where its columns lie in the chunks of w_out, zeros around it
+        // out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the triples s (one without keys has
+        // m = -inf, l = 0). Each wave works the weights out once, a lane a triple, and keeps them in
+        // LDS for itself.
+        constexpr int N_TRIPLES = DL_WAVES * MERGE_ENTRIES;
+        static_assert(N_TRIPLES <= WAVE, "a lane a triple");
+        const float triple_max = lane < N_TRIPLES ? merged[min(lane, N_TRIPLES - 1)][HD] : -INFINITY;
+        const float triple_sum = lane < N_TRIPLES ? merged[min(lane, N_TRIPLES - 1)][HD + 1] : 0.0f;
+        const float weight = expf(triple_max - wave_max_total(triple_max));
+        const float total = wave_total(triple_sum * weight);
+        merge_weight[wave][lane] = weight / total;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's own writes, read back below
         float value = 0.0f;
         const int d = tid - out_shift;
         if (d >= 0 && d < HD) {
-            float total_max = -INFINITY;
-            for (int s = 0; s < DL_WAVES; s++) total_max = fmaxf(total_max, merged[s][HD]);
-            float total = 0.0f;
-            for (int s = 0; s < DL_WAVES; s++) {
-                float weight = expf(merged[s][HD] - total_max);
-                total += merged[s][HD + 1] * weight;
-                value += merged[s][d] * weight;
-            }
-            value /= total;
+#pragma unroll 8
+            for (int s = 0; s < N_TRIPLES; s++) value += merged[s][d] * merge_weight[wave][s];
         }
-        mixed[tid] = static_cast<bf16_t>(value);
+        if (tid < HD_PAD) mixed[tid] = static_cast<bf16_t>(value);
     }
     lds_barrier();  // 7: the mixed row of this head is in LDS
     DL_STAMP(6);
@@ -834,7 +873,7 @@ int launch_mlp_half(PendingSum in, float* summed, const float* gamma, const floa
     // Few tokens a block: more waves share a token's pending sums (one round of loads instead of
     // several, each a trip to memory) and more blocks pull at the matrices; many tokens a block: the
     // matrices are read fewer times.
-    const int tokens_per_block = stage_pieces == 0 ? DL_TOKENS : (n_tokens <= 16 ? 4 : (n_tokens <= 64 ? 8 : DL_TOKENS));
+    const int tokens_per_block = stage_pieces == 0 ? DL_TOKENS : (n_tokens <= 4 ? 1 : (n_tokens <= 8 ? 2 : (n_tokens <= 16 ? 4 : (n_tokens <= 64 ? 8 : DL_TOKENS))));
     dim3 grid((inner + U - 1) / U, (n_tokens + tokens_per_block - 1) / tokens_per_block);
     decode_mlp_half_kernel<NV, U><<<grid, DL_THREADS, lds, stream>>>(in, summed, gamma, beta, eps, w_up, b_up, w_down, partial_out,
                                                                       n_tokens, width, inner, epilogue, stage_pieces, tokens_per_block);

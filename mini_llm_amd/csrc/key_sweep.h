@@ -107,13 +107,11 @@ struct KeySweep {
             float dot = 0.0f;
 #pragma unroll
             for (int i = 0; i < VEC; i++) dot += qf[i] * Chunk<T>::get(f.kf[u], i);
-#pragma unroll
-            for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
+            dot = lanes_sum<LPR>(dot);
             score[u] = base + u * RPI + group < end ? dot : -INFINITY;
             tile_max = fmaxf(tile_max, score[u]);
         }
-#pragma unroll
-        for (int offset = LPR; offset < WAVE; offset <<= 1) tile_max = fmaxf(tile_max, __shfl_xor(tile_max, offset, WAVE));
+        tile_max = wave_max_total(tile_max);
         float new_max = fmaxf(running_max, tile_max);
         float reference = new_max == -INFINITY ? 0.0f : new_max;  // no key so far (base >= end is allowed): nothing to rescale
         float rescale = expf(running_max - reference);
@@ -153,8 +151,7 @@ struct KeySweep {
         float dot = 0.0f;
 #pragma unroll
         for (int i = 0; i < VEC; i++) dot += qf[i] * key_row[sub * VEC + i];
-#pragma unroll
-        for (int offset = 1; offset < LPR; offset <<= 1) dot += __shfl_xor(dot, offset, WAVE);
+        dot = lanes_sum<LPR>(dot);
         float new_max = fmaxf(running_max, dot);
         float rescale = expf(running_max - new_max);
         running_sum *= rescale;
@@ -165,11 +162,23 @@ struct KeySweep {
         running_max = new_max;
     }
 
-    // Every lane of a row group counted the same keys: the groups' shares are added up, after
-    // which every lane holds the wave's sum and lanes 0..LPR-1 its output.
-    __device__ __forceinline__ void merge_groups() {
+    // Every lane of a row group counted the same keys: the shares of the groups inside each row of
+    // 16 lanes are added up (lanes LPR apart hold the same dimensions), after which the first LPR
+    // lanes of a row hold that row's output and every lane of the row its sum. A no-op for rows
+    // that are one group (LPR >= 16).
+    __device__ __forceinline__ void merge_inside_rows() {
+        if constexpr (LPR < 16) {
+            running_sum = row_strided_sum<LPR>(running_sum);
 #pragma unroll
-        for (int offset = LPR; offset < WAVE; offset <<= 1) {
+            for (int i = 0; i < VEC; i++) o[i] = row_strided_sum<LPR>(o[i]);
+        }
+    }
+
+    // All groups of the wave: after it every lane holds the wave's sum and lanes 0..LPR-1 its output.
+    __device__ __forceinline__ void merge_groups() {
+        merge_inside_rows();
+#pragma unroll
+        for (int offset = LPR < 16 ? 16 : LPR; offset < WAVE; offset <<= 1) {
             running_sum += __shfl_xor(running_sum, offset, WAVE);
 #pragma unroll
             for (int i = 0; i < VEC; i++) o[i] += __shfl_xor(o[i], offset, WAVE);
