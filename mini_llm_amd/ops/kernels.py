@@ -360,6 +360,13 @@ MLP_SLICE_UNITS = 64         # hidden units a block of the feed-forward kernel t
 LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kernels
 
 
+def layer_kernel_rows(width: int) -> int:
+    """Rows up to which the layer kernels for decoding beat the separate kernels (measured on
+    MI355X: at GPT-2 small's width up to 64 rows; at GPT-2 medium's they lose from 32 rows on, as
+    every (token, head) block reads its own copy of the partial rows and of the matrices)."""
+    return LAYER_KERNEL_MAX_ROWS if width <= 768 else min(16, LAYER_KERNEL_MAX_ROWS)
+
+
 def _pending(hidden):
     if isinstance(hidden, PendingRows):
         base, partials, bias = hidden.base, hidden.partials, hidden.bias

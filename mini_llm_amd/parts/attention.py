@@ -67,7 +67,7 @@ class CausalSelfAttention(Mixer):
 
     def forward_normed(self, hidden, norm, compute_dtype, ctx: LayerContext):
         # rows that are each the newest token of their request: the whole chain in one kernel
-        if (ctx.batch.max_q_len == 1 and hidden.shape[0] <= kernels.LAYER_KERNEL_MAX_ROWS and isinstance(norm, LayerNorm)
+        if (ctx.batch.max_q_len == 1 and hidden.shape[0] <= kernels.layer_kernel_rows(self.width) and isinstance(norm, LayerNorm)
                 and isinstance(self.qkv.weight, kernels.PackedMatrix) and isinstance(self.out.weight, kernels.PackedMatrix)
                 and self.qkv.weight.dtype == torch.bfloat16 and ctx.k_pages.dtype == torch.bfloat16
                 and kernels.decode_layer_supported(self.width, self.head_size, ctx.k_pages.shape[2])):
