@@ -79,22 +79,42 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const int row = blockIdx.x, tid = threadIdx.x;
     const float* x = logits + (size_t)row * vocab;
     const float temperature = temperatures ? temperatures[row] : 0.0f;
+    const int token_slot = token_slots ? slot_of_row[row] : -1;  // asked for now: at the end it would cost a trip to memory of its own
 
     float best = -INFINITY;
     int best_index = 0x7fffffff;
-    // eight loads in flight per thread before any is compared: the row is read in a few rounds
-    // of memory latency instead of one per element
+    // The row is read in 16-byte pieces, eight of them in flight per thread before any is compared:
+    // a few trips to memory for the whole row. A row starts wherever rows * vocab puts it, so the
+    // elements before the first 16-byte boundary and after the last one are read one by one.
+    const int head = min(vocab, (int)((16 - ((size_t)x & 15)) & 15) / 4);  // elements before the boundary
+    const int n_pieces = (vocab - head) / 4;
+    const f32x4* pieces = reinterpret_cast<const f32x4*>(x + head);
+    if (tid < head && beats(x[tid], tid, best, best_index)) {
+        best = x[tid];
+        best_index = tid;
+    }
+    for (int i = head + 4 * n_pieces + tid; i < vocab; i += SAMPLE_THREADS)
+        if (beats(x[i], i, best, best_index)) {
+            best = x[i];
+            best_index = i;
+        }
     constexpr int BATCH = 8;
-    for (int i0 = tid; i0 < vocab; i0 += SAMPLE_THREADS * BATCH) {
-        float values[BATCH];
+    for (int p0 = tid; p0 < n_pieces; p0 += SAMPLE_THREADS * BATCH) {
+        f32x4 values[BATCH];
 #pragma unroll
-        for (int u = 0; u < BATCH; u++) values[u] = x[min(i0 + u * SAMPLE_THREADS, vocab - 1)];
+        for (int u = 0; u < BATCH; u++) values[u] = pieces[min(p0 + u * SAMPLE_THREADS, n_pieces - 1)];
 #pragma unroll
         for (int u = 0; u < BATCH; u++) {
-            int i = i0 + u * SAMPLE_THREADS;
-            if (i < vocab && beats(values[u], i, best, best_index)) {
-                best = values[u];
-                best_index = i;
+            int p = p0 + u * SAMPLE_THREADS;
+            if (p < n_pieces) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int i = head + 4 * p + e;
+                    if (beats(values[u][e], i, best, best_index)) {
+                        best = values[u][e];
+                        best_index = i;
+                    }
+                }
             }
         }
     }
@@ -102,7 +122,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (!(temperature > 0.0f) || best != best) {  // greedy, or a NaN in the row
         if (tid == 0) {
             out_tokens[row] = best_index;
-            if (token_slots && slot_of_row[row] >= 0) token_slots[slot_of_row[row]] = best_index;
+            if (token_slot >= 0) token_slots[token_slot] = best_index;
         }
         return;
     }
@@ -149,7 +169,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     block_best(chosen, chosen_index, shared_values, shared_indices);
     if (tid == 0) {
         out_tokens[row] = chosen_index;
-        if (token_slots && slot_of_row[row] >= 0) token_slots[slot_of_row[row]] = chosen_index;
+        if (token_slot >= 0) token_slots[token_slot] = chosen_index;
     }
 }
 
