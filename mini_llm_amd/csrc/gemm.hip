@@ -75,7 +75,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                                                    const float* __restrict__ bias,
                                                    const float* __restrict__ residual,
                                                    OutT* __restrict__ out, int M, int N, int K,
-                                                   int epilogue) {
+                                                   int epilogue, CacheScatter scatter) {
     constexpr int BK = Tile<T>::BK, VEC = Tile<T>::VEC, PAD = Tile<T>::PAD;
     constexpr int LDK = BK + PAD;
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
@@ -220,6 +220,33 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
             int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
             if (col >= N) continue;
             float b = bias ? bias[col] : 0.0f;
+            if (scatter.enabled) {
+                // a fused q/k/v projection: the q columns go to out [M, q_width], this lane's key or
+                // value column into the cache pages at the rows' slots
+                OutT* pages = nullptr;
+                int kv_head = 0, d = 0;
+                if (col >= scatter.q_width) {
+                    int c = col - scatter.q_width;
+                    pages = (OutT*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
+                    if (c >= scatter.kv_width) c -= scatter.kv_width;
+                    kv_head = c / scatter.head_size, d = c % scatter.head_size;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    int row = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                    if (row >= M) continue;
+                    OutT value = from_float<OutT>(acc[i][j][v] + b);
+                    if (pages == nullptr) {
+                        out[(size_t)row * scatter.q_width + col] = value;
+                    } else {
+                        int slot = scatter.slots[row];
+                        if (slot < 0) continue;
+                        int page = slot >> scatter.page_shift, offset = slot & ((1 << scatter.page_shift) - 1);
+                        pages[((((size_t)page * scatter.n_kv_heads + kv_head) << scatter.page_shift) + offset) * scatter.head_size + d] = value;
+                    }
+                }
+                continue;
+            }
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 int row = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
@@ -387,15 +414,15 @@ int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tu
 
 template <typename T, typename OutT, bool ALIGNED, int BM, int BN, int WAVES_M, int WAVES_N>
 void launch_tile(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
-                 int K, int epilogue, hipStream_t stream) {
+                 int K, int epilogue, hipStream_t stream, CacheScatter scatter) {
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
-    if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
-    else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue);
+    if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+    else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
 }
 
 template <typename T, typename OutT, bool ALIGNED>
 void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
-                  int K, int epilogue, hipStream_t stream) {
+                  int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}) {
     int tile = g_forced_tile;
     if (tile == 0) {
         // measured on MI355X at GPT-2 sizes: many waves per block hide latency best
@@ -404,13 +431,13 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
         else tile = 7;
     }
     switch (tile) {
-        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
-        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream); break;
+        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
     }
 }
 
@@ -460,13 +487,13 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
     return mllm_check_launch("gemm");
 }
 
-// The fused q/k/v projection of a decode step or a short portion (M <= 64 rows): q columns go
-// to out_q [M, q_width], key and value columns straight into the cache pages at slots[row]
+// The fused q/k/v projection: q columns go to out_q [M, q_width], key and value columns straight
+// into the cache pages at slots[row] (few rows: the skinny kernel; more: the tiled one)
 // (what the reference's decode block does with its fused matvec: engine/src/transformer_block.cu:223-242).
 MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, const float* bias, void* out_q, void* k_pages,
                                  void* v_pages, const int* slots, int M, int K, int q_width, int kv_width,
                                  int n_kv_heads, int head_size, int page_size, int dtype, hipStream_t stream) {
-    MLLM_REQUIRE(M >= 0 && M <= 64, "gemm_qkv_cache: %d rows; this entry takes up to 64", M);
+    MLLM_REQUIRE(M >= 0 && ceil_div(M, 32) <= 65535, "gemm_qkv_cache: bad row count %d", M);
     MLLM_REQUIRE(K > 0 && q_width > 0 && kv_width == n_kv_heads * head_size && head_size > 0, "gemm_qkv_cache: bad sizes");
     MLLM_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "gemm_qkv_cache: page size %d is no power of two", page_size);
     MLLM_REQUIRE(dtype == MLLM_F32 || dtype == MLLM_BF16, "gemm_qkv_cache: unknown dtype %d", dtype);
@@ -478,7 +505,8 @@ MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, con
 #define MLLM_QKV_CASE(T)                                                                                              \
     if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
     else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
-    else launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
+    else if (M <= 64) launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
+    else launch_tiled<T, T, true>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
     if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
 #undef MLLM_QKV_CASE
     return mllm_check_launch("gemm_qkv_cache");

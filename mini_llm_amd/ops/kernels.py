@@ -234,19 +234,15 @@ def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
     check(library().mllm_cache_write(_ptr(k_src), _ptr(v_src), k_src.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(slots), n, n_kv_heads, head_size, page_size, _code(k_pages.dtype), _stream()))
 
 
-FUSED_QKV_MAX_ROWS = 64
-
-
 def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_heads, head_size):
-    """The fused q/k/v projection of up to 64 rows: returns q [rows, n_heads*head_size] and writes
-    the key and value columns straight into the cache pages at slots[row] (negative: skip)."""
+    """The fused q/k/v projection: returns q [rows, n_heads*head_size] and writes the key and value
+    columns straight into the cache pages at slots[row] (negative: skip)."""
     _device_tensor(x, "x", dim=2)
     w_ptr, w_packed, w_rows, w_cols = _matrix(weight, "weight", x.dtype)
     num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     _require(k_pages.dtype == x.dtype, "pages and x differ in element type")
     m, k = x.shape
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
-    _require(m <= FUSED_QKV_MAX_ROWS, f"{m} rows; the fused projection takes up to {FUSED_QKV_MAX_ROWS}")
     _require((w_rows, w_cols) == (q_width + 2 * kv_width, k), "weight does not match the heads or x")
     _require(k % (16 // x.element_size()) == 0, "the input width is not a multiple of a 16-byte piece")
     if bias is not None:

@@ -44,10 +44,10 @@ class CausalSelfAttention(Mixer):
         return KVNeed(self.n_kv_heads, self.head_size, self.window)
 
     def forward(self, x, residual, ctx: LayerContext):
-        fused = (ctx.write_cache and x.shape[0] <= kernels.FUSED_QKV_MAX_ROWS
-                 and x.shape[1] % (16 // x.element_size()) == 0 and ctx.k_pages.shape[2] & (ctx.k_pages.shape[2] - 1) == 0)
+        fused = (ctx.write_cache and x.shape[1] % (16 // x.element_size()) == 0
+                 and ctx.k_pages.shape[2] & (ctx.k_pages.shape[2] - 1) == 0)
         if fused:
-            # few rows: one kernel projects, keeps q and puts keys and values into their pages
+            # one kernel projects, keeps q and puts keys and values into their pages
             q = kernels.linear_qkv_cache(x, self.qkv.weight, self.qkv.bias, ctx.k_pages, ctx.v_pages, ctx.group.slots,
                                          self.n_heads, self.n_kv_heads, self.head_size)
         else:

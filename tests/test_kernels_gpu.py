@@ -342,14 +342,14 @@ def test_operands_are_checked_on_the_host(K):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16)])
+@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16), (65, 3, 3, 32, 16), (300, 5, 5, 48, 64)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, packed):
     rng = np.random.default_rng(rows)
     width = 72
     qw, kvw = n_heads * head_size, n_kv_heads * head_size
     x, w, b = rng.standard_normal((rows, width)), rng.standard_normal((qw + 2 * kvw, width)) / 8, rng.standard_normal(qw + 2 * kvw)
-    num_pages = 8
+    num_pages = max(8, rows // page_size + 2)
     kp = torch.full((num_pages, n_kv_heads, page_size, head_size), 7.0, device=DEV).to(dtype)
     vp = torch.full_like(kp, 7.0)
     slots = rng.permutation(num_pages * page_size)[:rows].astype(np.int32)
