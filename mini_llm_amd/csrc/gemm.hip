@@ -430,13 +430,9 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
         else if (M <= 64) tile = 2;
         else tile = 7;
     }
-    switch (tile) {
+    switch (tile) {  // other shapes (128x128, 256x128, fewer waves) were measured and lost at every size here
         case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
         case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        case 3: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        case 4: launch_tile<T, OutT, ALIGNED, 128, 128, 2, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        case 5: launch_tile<T, OutT, ALIGNED, 128, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        case 6: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
         default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
     }
 }
@@ -466,7 +462,7 @@ void launch_gemm(const void* A, const void* W, bool packed, const float* bias, c
 
 }  // namespace
 
-// Tuning aid: forces one tile shape of the tiled kernel (0 gives the choice back to the sizes).
+// Tuning aid: forces one tile shape of the tiled kernel (1: 32x128, 2: 64x64, another number: 128x64; 0 gives the choice back to the sizes).
 MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
 MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* bias, const float* residual,
