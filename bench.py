@@ -146,7 +146,7 @@ def measure_prefill(engine, runs: int = 5):
 MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
 
 
-def measure_serving(dtype: str, temperature: float):
+def measure_serving(dtype: str, temperature: float, step_ahead: bool = True):
     """Continuous batching through the scheduler: 64 concurrent requests on the GPT-2 medium shape,
     prompts of 32 to 768 uniform-random ids, 256 new tokens each, prompts cut into portions under a
     budget of 512 tokens a step and run beside the decodes."""
@@ -159,7 +159,8 @@ def measure_serving(dtype: str, temperature: float):
     from mini_llm_amd.sampling import SamplingParams
 
     config = config_from_dict(MEDIUM)
-    engine = Engine.from_random(config, 6, EngineOptions(dtype=dtype, max_sessions=64, max_tokens=64 * CONTEXT, max_tokens_per_step=512))
+    engine = Engine.from_random(config, 6, EngineOptions(dtype=dtype, max_sessions=64, max_tokens=64 * CONTEXT, max_tokens_per_step=512,
+                                                        step_ahead=step_ahead))
     rng = np.random.default_rng(6)
     prompts = [rng.integers(0, config.vocab_size, int(n)).tolist() for n in rng.integers(32, 769, 64)]
     counts = [0] * len(prompts)
@@ -185,7 +186,8 @@ def measure_serving(dtype: str, temperature: float):
     return {"model": "gpt2-medium shape", "dtype": dtype, "requests": len(prompts), "prompt_tokens": prompt_tokens,
             "generated_tokens": generated, "seconds": round(seconds, 3), "generated_tokens_per_s": round(generated / seconds, 1),
             "all_tokens_per_s": round((generated + prompt_tokens) / seconds, 1), "steps": after["steps"] - before["steps"],
-            "temperature": temperature, "preemptions": after["preemptions"] - before["preemptions"]}
+            "temperature": temperature, "preemptions": after["preemptions"] - before["preemptions"],
+            "step_ahead": step_ahead}
 
 
 def measure_peaks():
@@ -236,6 +238,7 @@ def main() -> int:
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
+    parser.add_argument("--step-by-step", action="store_true", help="--serving reads every step's tokens before it launches the next")
     parser.add_argument("--peaks", action="store_true", help="measure this machine's read bandwidth and matrix-core rate with the library's probes")
     args = parser.parse_args()
     if args.gpus != 1:
@@ -247,7 +250,7 @@ def main() -> int:
         return 0
 
     if args.serving:
-        print(json.dumps({"serving": measure_serving(args.dtype, args.temperature)}))
+        print(json.dumps({"serving": measure_serving(args.dtype, args.temperature, not args.step_by_step)}))
         return 0
 
     from mini_llm_amd.config import config_from_dict

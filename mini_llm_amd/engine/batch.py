@@ -46,6 +46,7 @@ class StepBatch:
     state_slots: object     # int32 [n_requests]
     logit_rows: object      # int32 [n_logit_rows]: rows whose logits are computed
     token_sources: object   # int32 [n_tokens]: last-token slot a row's token is taken from, -1 = as given
+    logit_slots: object     # int32 [n_logit_rows]: state slot of the request each logit row belongs to
     groups: list            # GroupStepData per cache group
     request_ids: list = field(default_factory=list)
     host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
@@ -146,22 +147,26 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
             slot[q_starts[i] : q_starts[i + 1]] = pages[pos // cache.page_size] * cache.page_size + pos % cache.page_size
         tables.append(table)
         slots.append(slot)
+    logit_slots = np.asarray([state_slots[i] for i, e in enumerate(entries) for _ in e.want], dtype=np.int32)
     n_logit_rows = len(logit_rows)
     if capacity is not None:
         logit_rows = _pad(logit_rows, cap_tokens, 0)
+        logit_slots = _pad(logit_slots, cap_tokens, 0)
 
     sections = [_pad(tokens, cap_tokens, -1), _pad(positions, cap_tokens, 0), _pad(token_request, cap_tokens, -1), q_starts,
                 _pad(np.asarray(contexts, dtype=np.int32), cap_requests, 0), _pad(state_slots, cap_requests, 0), logit_rows,
                 token_sources]
     for table, slot in zip(tables, slots):
         sections += [table.reshape(-1), slot]
+    sections.append(logit_slots)
     offsets, total = [], 0
     for section in sections:
         offsets.append(total)
         total += _aligned(len(section))
     host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts[: n_requests + 1],
             "context_lens": sections[4][:n_requests], "state_slots": state_slots, "logit_rows": logit_rows[:n_logit_rows],
-            "token_sources": token_sources[:n_tokens], "block_tables": tables, "slots": slots}
+            "token_sources": token_sources[:n_tokens], "logit_slots": logit_slots[:n_logit_rows],
+            "block_tables": tables, "slots": slots}
     if staging is None:
         views = sections
     else:
@@ -178,7 +183,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
         max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
-        state_slots=views[5], logit_rows=views[6], token_sources=views[7], groups=groups,
+        state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
         request_ids=[e.request_id for e in entries], host=host,
     )
 
@@ -250,5 +255,6 @@ class DecodeBatchBuilder:
             n_tokens=self.capacity, n_requests=self.capacity, n_logit_rows=self.capacity, max_q_len=1,
             max_total_len=self.cache.max_length, tokens=views[0], positions=views[1], token_request=views[2],
             q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], token_sources=views[7],
+            logit_slots=views[5],  # every request has one logit row, in its own place
             groups=groups, request_ids=[e.request_id for e in entries], host={},
         )

@@ -31,6 +31,7 @@ class EngineOptions:
     page_size: int = DEFAULT_PAGE_SIZE
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
     use_graphs: bool = True              # replay decode steps from captured HIP graphs
+    step_ahead: bool = True              # the scheduler launches a step before it has read the one before
     device: str = "cuda:0"
 
 
@@ -40,6 +41,7 @@ class _Executor:
     def __init__(self, engine: "Engine"):
         self._engine = engine
         self.page_size = engine.cache.page_size
+        self._hosts, self._turn = [], 0
 
     def max_positions(self):
         return self._engine.model.max_positions()
@@ -71,11 +73,40 @@ class _Executor:
         return self._engine.cache.free_pages()
 
     def run(self, entries, sampling, steps):
+        return self.collect(self.launch(entries, sampling, steps))
+
+    # One step ahead: launch() queues the step, the sampling (each token also goes to its request's
+    # last-token slot, where the next step finds it) and the copy of the tokens into pinned host
+    # memory; collect() waits for that copy alone, not for what was launched after it.
+    RING = 4
+
+    def launch(self, entries, sampling, steps):
+        import torch
+
+        engine = self._engine
         entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want, e.from_slot) for e in entries]
-        logits = self._engine.runner.step(entries)
+        logits = engine.runner.step(entries)
         if logits is None:
+            return None
+        n = logits.shape[0]
+        tokens = engine.sampler.sample(logits, sampling, steps, token_slots=engine.cache.last_token,
+                                       slot_of_row=engine.runner.last_batch.logit_slots)
+        if not self._hosts or self._hosts[0].shape[0] < n:
+            size = max(n, engine.options.max_sessions)
+            self._hosts = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+        host = self._hosts[self._turn % self.RING]
+        self._turn += 1
+        host[:n].copy_(tokens, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return host, n, event
+
+    def collect(self, handle):
+        if handle is None:
             return []
-        return self._engine.sampler.sample(logits, sampling, steps).cpu().tolist()
+        host, n, event = handle
+        event.synchronize()
+        return host[:n].tolist()
 
 
 class Session:
@@ -130,7 +161,8 @@ class Engine:
                                 max_requests=options.max_sessions, device=options.device)
         self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs)
         self.sampler = Sampler(self.runner.staging)
-        self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step)
+        self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step,
+                                   step_ahead=options.step_ahead)
         self._next_handle = 0
         self._queued = collections.deque()   # (pinned tokens, count, event) of steps whose tokens were not taken yet
         self._token_buffers, self._queue_turn = [], 0

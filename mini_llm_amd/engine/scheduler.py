@@ -19,6 +19,17 @@ Every iteration (`step`):
    fails;
 4. one step of the engine; each request whose prompt is complete gets one new token, sampled
    on the device; `emit(token, finish)`; a finished request leaves at once and frees its pages.
+
+One step ahead (an executor with `launch` / `collect`): the step planned in 2 is launched before
+the tokens of the step before it have been read. A request that was sampled in the step in
+flight brings "the token in my slot" (the sampler leaves it there on the device), so planning,
+batch layout and launch of step n+1 take place while the device still runs step n, and the device
+never waits for the host. What the host cannot know yet is whether token n was the request's end
+token: ends by length and context are counted ahead and never launched, an end token is seen one
+step late, and the one token computed past it is dropped. A finished request's pages go back at
+once all the same: everything the device does is in launch order, so whoever gets them next writes
+them after the step in flight has. A plan that would have to preempt first waits for the step in
+flight, so that a victim's tokens are all known.
 """
 
 from __future__ import annotations
@@ -51,6 +62,11 @@ class StepExecutor(Protocol):
     def pages_needed(self, request_id, n_new: int) -> list[int]: ...  # per layer group, for its next n_new tokens
     def free_pages(self) -> list[int]: ...                            # per layer group
     def run(self, entries: list, sampling: list, steps: list) -> list[int]: ...
+    # Optional, for running one step ahead: launch() queues the step and leaves each sampled token
+    # in its request's last-token slot; collect() waits for that step and returns its tokens. An
+    # entry with from_slot=True takes its one token from the request's slot.
+    # def launch(self, entries, sampling, steps) -> object: ...
+    # def collect(self, handle) -> list[int]: ...
 
 
 @dataclass(eq=False)
@@ -76,7 +92,10 @@ class _Running:
     request_id: int
     pending: list              # tokens not yet fed: the rest of the prompt, or the last sampled token
     history: list = field(default_factory=list)   # tokens fed since it was (re)admitted: what its pages hold
-    generated: int = 0
+    generated: int = 0         # tokens delivered
+    launched: int = 0          # tokens whose sampling has been launched (= generated, or one more)
+    awaiting: bool = False     # its next token is the output of the step in flight
+    fed_ahead: bool = False    # the step in flight takes the token of the step before it from the slot
     prompt_len: int = 0        # of the original prompt (a preempted request's recompute does not count)
     order: int = 0             # admission order; the largest is preempted first
     finished: bool = False
@@ -96,15 +115,29 @@ class _PagePlan:
         self.taken = [t + n for t, n in zip(self.taken, need)]
 
 
+@dataclass
+class _Flight:
+    """A step that has been launched and whose tokens have not been read."""
+
+    handle: object
+    sampled: list              # the _Running of each token, in the step's order
+
+
+class _SettleFirst(Exception):
+    """The plan has to preempt: the step in flight is collected first."""
+
+
 class Scheduler:
     def __init__(self, executor: StepExecutor, max_batch: int = 16, max_tokens_per_step: int = 2048,
-                 max_prefills_per_step: int | None = None):
+                 max_prefills_per_step: int | None = None, step_ahead: bool = True):
         if max_batch < 1 or max_tokens_per_step < 1:
             raise ValueError("max_batch and max_tokens_per_step must be at least 1")
         if max_prefills_per_step is not None and max_prefills_per_step < 1:
             raise ValueError("max_prefills_per_step must be at least 1")
         self._executor = executor
         self._max_batch, self._budget, self._max_prefills = max_batch, max_tokens_per_step, max_prefills_per_step
+        self._step_ahead = step_ahead and hasattr(executor, "launch") and hasattr(executor, "collect")
+        self._in_flight: _Flight | None = None
         self._waiting: collections.deque = collections.deque()   # Request, or _Running that was preempted
         self._running: list[_Running] = []
         self._wake = threading.Condition()
@@ -113,7 +146,7 @@ class Scheduler:
         self._next_id = 0
         self._order = 0
         self._steps = self._decode_steps = self._tokens = self._prefills = 0
-        self._batch_sizes = self._step_tokens = self._preemptions = 0
+        self._batch_sizes = self._step_tokens = self._preemptions = self._dropped_tokens = 0
 
     # --- called from other threads -------------------------------------------------------------
     def submit(self, request: Request) -> None:
@@ -133,6 +166,7 @@ class Scheduler:
             "steps": self._steps,
             "tokens_per_step": self._step_tokens / self._steps if self._steps else 0.0,
             "preemptions": self._preemptions,
+            "dropped_tokens": self._dropped_tokens,   # computed past an end token nobody had seen yet
         }
 
     def start(self) -> None:
@@ -152,7 +186,7 @@ class Scheduler:
 
     def has_work(self) -> bool:
         with self._wake:
-            return bool(self._running) or bool(self._waiting)
+            return bool(self._running) or bool(self._waiting) or self._in_flight is not None
 
     def run_until_idle(self) -> None:
         while self.step():
@@ -162,7 +196,7 @@ class Scheduler:
     def _loop(self) -> None:
         while True:
             with self._wake:
-                while not self._stopping and not self._running and not self._waiting:
+                while not self._stopping and not self._running and not self._waiting and self._in_flight is None:
                     self._wake.wait()
                 if self._stopping:
                     return
@@ -172,9 +206,16 @@ class Scheduler:
         """One iteration. Returns False if there was nothing to do."""
         try:
             self._drop_cancelled()
-            entries, owners = self._plan()
-            if entries:
-                self._run(entries, owners)
+            try:
+                entries, owners = self._plan()
+            except _SettleFirst:
+                self._collect()
+                entries, owners = self._plan()
+            launched = self._launch(entries, owners) if entries else None
+            self._collect()                 # the step launched before this one
+            self._in_flight = launched
+            if not self._step_ahead:
+                self._collect()
         except Exception as error:  # the engine is shared: every running request is affected
             logger.exception("engine error")
             self._fail_running(str(error))
@@ -186,6 +227,7 @@ class Scheduler:
         for running in [r for r in self._running if r.request.cancelled]:
             self._executor.close(running.request_id)
             self._running.remove(running)
+            running.finished = True   # a token of its that is still in flight is dropped
 
     def _portion_that_fits(self, running: _Running, plan: "_PagePlan", most: int):
         """(n, pages): the largest portion n <= most whose pages can be had beside what is planned
@@ -204,6 +246,7 @@ class Scheduler:
     def _preempt(self, victim: _Running) -> None:
         """The victim gives everything back and waits at the front of the queue; what it has been
         fed so far becomes prompt again, so that it is recomputed and goes on where it was."""
+        assert not victim.awaiting, "a victim's tokens are all known"
         self._executor.close(victim.request_id)
         self._running.remove(victim)
         victim.pending = victim.history + victim.pending
@@ -225,9 +268,13 @@ class Scheduler:
                 continue  # preempted while an older request was planned
             if budget < 1:
                 break
-            most = min(len(running.pending), budget)
+            if self._ends_in_flight(running):
+                continue
+            most = min(self._to_feed(running), budget)
             n, need = self._portion_that_fits(running, plan, most)
             while n == 0:
+                if self._in_flight is not None:
+                    raise _SettleFirst()   # nothing has been changed so far
                 victim = max(self._running, key=lambda r: r.order)
                 preempted = True
                 if victim is running:
@@ -267,9 +314,25 @@ class Scheduler:
             admitted += 1
         return entries, owners
 
+    @staticmethod
+    def _to_feed(running: _Running) -> int:
+        return 1 if running.awaiting else len(running.pending)
+
+    def _ends_in_flight(self, running: _Running) -> bool:
+        """The token being sampled in the step in flight is this request's last, whatever it is."""
+        if not running.awaiting:
+            return False
+        request, limit = running.request, self._executor.max_positions()
+        return ((limit is not None and running.prompt_len + running.launched >= limit)
+                or (request.max_new_tokens is not None and running.launched >= request.max_new_tokens))
+
     def _add_entry(self, entries, owners, plan, running, n, need) -> None:
-        completes = n == len(running.pending)
-        entries.append(StepEntry(running.request_id, list(running.pending[:n]), [n - 1] if completes else []))
+        if running.awaiting:
+            entry = StepEntry(running.request_id, [0], [0], from_slot=True)
+        else:
+            completes = n == len(running.pending)
+            entry = StepEntry(running.request_id, list(running.pending[:n]), [n - 1] if completes else [])
+        entries.append(entry)
         owners.append(running)
         plan.take(need)
 
@@ -318,26 +381,52 @@ class Scheduler:
             self._waiting.appendleft(item)
 
     # --- running and delivering ----------------------------------------------------------------
-    def _run(self, entries, owners) -> None:
-        sampled_owners = [o for o, e in zip(owners, entries) if e.want]
-        sampling = [o.request.sampling for o in sampled_owners]
-        steps = [o.generated for o in sampled_owners]
-        tokens = self._executor.run(entries, sampling, steps)
+    def _launch(self, entries, owners) -> _Flight:
+        sampled = [o for o, e in zip(owners, entries) if e.want]
+        sampling = [o.request.sampling for o in sampled]
+        steps = [o.launched for o in sampled]
+        if self._step_ahead:
+            handle = self._executor.launch(entries, sampling, steps)
+        else:
+            handle = self._executor.run(entries, sampling, steps)
         self._steps += 1
         self._step_tokens += sum(len(e.tokens) for e in entries)
-        decodes = sum(1 for o, e in zip(owners, entries) if o.generated > 0 and len(e.tokens) == 1)
+        decodes = sum(1 for o, e in zip(owners, entries) if o.launched > 0 and len(e.tokens) == 1)
         if decodes:
             self._decode_steps += 1
             self._batch_sizes += decodes
         for owner, entry in zip(owners, entries):
-            owner.history.extend(entry.tokens)
-            del owner.pending[: len(entry.tokens)]
-        for owner, token in zip(sampled_owners, tokens):
+            if entry.from_slot:
+                owner.fed_ahead = True     # the token joins its history when it is known
+            else:
+                owner.history.extend(entry.tokens)
+                del owner.pending[: len(entry.tokens)]
+        for owner in sampled:
+            owner.launched += 1
+            owner.awaiting = True
+        return _Flight(handle, sampled)
+
+    def _collect(self) -> None:
+        """Reads the tokens of the step in flight, if there is one, and delivers them."""
+        flight, self._in_flight = self._in_flight, None
+        if flight is None:
+            return
+        tokens = self._executor.collect(flight.handle) if self._step_ahead else flight.handle
+        for owner, token in zip(flight.sampled, tokens):
+            if owner.finished:
+                self._dropped_tokens += 1
+                continue
+            token = int(token)
             if owner.generated == 0:
                 self._prefills += 1
             owner.generated += 1
-            owner.pending = [int(token)]
-            self._deliver(owner, int(token))
+            if owner.fed_ahead:            # the step launched after this one has been fed it already
+                owner.history.append(token)
+                owner.fed_ahead = False
+            else:
+                owner.awaiting = False
+                owner.pending = [token]
+            self._deliver(owner, token)
         self._running = [r for r in self._running if not r.finished]
 
     def _finish_reason(self, running: _Running, token: int) -> FinishReason | None:
@@ -368,7 +457,9 @@ class Scheduler:
 
     def _fail_running(self, message: str) -> None:
         running, self._running = self._running, []
+        self._in_flight = None
         for item in running:
+            item.finished = True
             try:
                 self._executor.close(item.request_id)
             except Exception:

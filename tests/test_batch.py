@@ -25,7 +25,7 @@ def test_decode_builder_matches_the_general_one():
         general = build_step_batch(entries, cache, None, vocab_size=100, capacity=8)
         flat = builder.fill(entries)
         fast = builder.batch(flat, entries)
-        for field in ("tokens", "positions", "token_request", "q_starts", "context_lens", "state_slots", "logit_rows", "token_sources"):
+        for field in ("tokens", "positions", "token_request", "q_starts", "context_lens", "state_slots", "logit_rows", "token_sources", "logit_slots"):
             np.testing.assert_array_equal(getattr(fast, field), getattr(general, field), err_msg=field)
         for g in range(2):
             np.testing.assert_array_equal(fast.groups[g].block_tables, general.groups[g].block_tables)

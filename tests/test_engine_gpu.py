@@ -340,3 +340,45 @@ def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
     engine.release_cache(h)
     while engine._queued:
         engine.take()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dtype):
+    # nine requests in a pool that holds about three of them (requests wait, and some are preempted
+    # and recomputed), prompts in portions of 24 tokens beside decodes, an end token for every
+    # other request, greedy and sampled: the scheduler that launches a step before it has read the
+    # one before must deliver exactly what the step-by-step one delivers, and drop what it
+    # computed past an end token
+    from mini_llm_amd.engine.scheduler import Request
+    from mini_llm_amd.sampling import SamplingParams
+
+    _, config, weights = model_dirs["A"]
+    vocab = config["vocab_size"]
+    prompts = [random_tokens(200 + i, n, vocab) for i, n in enumerate((3, 40, 11, 64, 7, 29, 50, 2, 33))]
+    results = {}
+    for ahead in (False, True):
+        engine = engines("A", dtype, max_sessions=4, max_tokens=256, max_tokens_per_step=24, step_ahead=ahead)
+        for temperature in (0.0, 0.9):
+            if temperature == 0.0 and not ahead:
+                free = engine.generate(prompts, max_new_tokens=24)
+                ends = [tokens[5 + i] if i % 2 == 0 else None for i, tokens in enumerate(free)]
+            outputs, errors = [[] for _ in prompts], []
+            for i, prompt in enumerate(prompts):
+                def emit(token, finish, i=i):
+                    outputs[i].append((token, finish))
+                engine.submit(Request(prompt, 24, ends[i], emit, errors.append,
+                                      SamplingParams(temperature=temperature, seed=31 + i)))
+            before = engine.stats()
+            engine.scheduler.run_until_idle()
+            after = engine.stats()
+            results[ahead, temperature] = outputs
+            assert not errors
+            assert all(o and o[-1][1] is not None and all(f is None for _, f in o[:-1]) for o in outputs)
+            assert engine.cache.free_pages() == [engine.cache.pools[0].num_pages] and not engine.cache.requests
+            if ahead and temperature == 0.0:
+                assert after["dropped_tokens"] - before["dropped_tokens"] >= 1
+                assert any(f == "stop" for o in outputs for _, f in o)
+            if not ahead:
+                assert after["dropped_tokens"] == 0
+    for temperature in (0.0, 0.9):
+        assert results[True, temperature] == results[False, temperature]

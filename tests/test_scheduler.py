@@ -325,3 +325,147 @@ def test_options_are_checked():
         Scheduler(FakeExecutor(), max_batch=0)
     with pytest.raises(ValueError):
         Scheduler(FakeExecutor(), max_tokens_per_step=0)
+
+
+# --- one step ahead -----------------------------------------------------------------------------
+class AheadExecutor(FakeExecutor):
+    """The fake with launch / collect: a launched step is worked off at once, as a device would in
+    launch order, and leaves each sampled token in its request's slot; the host sees the tokens
+    at collect. It records how many steps were launched while another had not been collected."""
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.slot = {}
+        self.uncollected = 0
+        self.launched_ahead = 0
+        self.fail_next_collect = False
+
+    def launch(self, entries, sampling, steps):
+        for e in entries:
+            if e.from_slot:
+                assert e.tokens == [0] and e.want == [0]
+                e.tokens = [self.slot[e.request_id]]
+        tokens = self.run(entries, sampling, steps)
+        sampled = [e.request_id for e in entries if e.want]
+        self.slot.update(zip(sampled, tokens))
+        assert self.uncollected <= 1, "more than one step ahead"
+        self.launched_ahead += self.uncollected
+        self.uncollected += 1
+        return tokens
+
+    def collect(self, handle):
+        self.uncollected -= 1
+        if self.fail_next_collect:
+            self.fail_next_collect = False
+            raise RuntimeError("late boom")
+        return handle
+
+
+def test_a_step_is_launched_before_the_one_before_it_is_read():
+    ex = AheadExecutor()
+    s = Scheduler(ex)
+    a, _ = submit(s, [100, 5, 6], max_new=5)
+    b, _ = submit(s, [200], max_new=3)
+    s.run_until_idle()
+    assert a.tokens == [101, 102, 103, 104, 105] and b.tokens == [201, 202, 203]
+    assert (a.finish, b.finish) == ("length", "length") and ex.all_free()
+    # an end by length is counted ahead: no step runs for a token that nobody wants
+    assert composition(ex) == [[(0, 3), (1, 1)], [(0, 1), (1, 1)], [(0, 1), (1, 1)], [(0, 1)], [(0, 1)]]
+    assert ex.launched_ahead == 4 and s.stats()["dropped_tokens"] == 0
+    assert s.stats()["tokens"] == 8 and s.stats()["prefills"] == 2 and s.stats()["decode_steps"] == 4
+
+
+def test_an_end_token_is_seen_one_step_late_and_the_token_past_it_is_dropped():
+    ex = AheadExecutor()
+    s = Scheduler(ex)
+    stop, _ = submit(s, [100, 1], max_new=10, eos=103)
+    other, _ = submit(s, [200], max_new=6)
+    s.run_until_idle()
+    assert (stop.tokens, stop.finish) == ([101, 102, 103], "stop")
+    assert other.tokens == [201, 202, 203, 204, 205, 206] and ex.all_free()
+    assert sum(1 for step in ex.steps for r, _, _ in step if r == 0) == 4   # one step more than its 3 tokens
+    assert s.stats()["dropped_tokens"] == 1 and s.stats()["tokens"] == 9
+
+
+def test_ends_by_context_are_counted_ahead():
+    ex = AheadExecutor(positions=8)
+    s = Scheduler(ex)
+    context, _ = submit(s, [200, 1, 2, 3, 4], max_new=10)            # 5 + 3 >= 8
+    s.run_until_idle()
+    assert (context.tokens, context.finish) == ([201, 202, 203], "context")
+    assert composition(ex) == [[(0, 5)], [(0, 1)], [(0, 1)]] and s.stats()["dropped_tokens"] == 0
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_one_step_ahead_delivers_what_step_by_step_delivers(seed):
+    """Random requests (prompt lengths, limits, end tokens, arrival times) in a pool so small that
+    requests are preempted: the same tokens and finish reasons either way, and every page back."""
+    import random
+
+    def play(executor, **kw):
+        rng = random.Random(seed)
+        s = Scheduler(executor, max_batch=4, max_tokens_per_step=rng.choice([4, 7, 64]), **kw)
+        sinks = []
+        for i in range(12):
+            prompt = [500 * (i + 1)] + [rng.randrange(50) for _ in range(rng.randrange(0, 14))]
+            max_new = rng.randrange(1, 16)
+            eos = prompt[0] + rng.randrange(1, 20) if rng.random() < 0.5 else None
+            sinks.append(submit(s, prompt, max_new=max_new, eos=eos)[0])
+            for _ in range(rng.randrange(0, 4)):
+                s.step()
+        s.run_until_idle()
+        return s, sinks
+
+    plain_s, plain = play(FakeExecutor(num_pages=9, page_size=4, positions=24))
+    ex = AheadExecutor(num_pages=9, page_size=4, positions=24)
+    ahead_s, ahead = play(ex)
+    assert [(x.tokens, x.finish, x.error) for x in ahead] == [(x.tokens, x.finish, x.error) for x in plain]
+    assert all(x.finish is not None for x in plain)
+    assert ex.all_free() and ex.launched_ahead > 0
+    assert ahead_s.stats()["tokens"] == plain_s.stats()["tokens"]
+    if seed == 0:
+        assert plain_s.stats()["preemptions"] > 0 and ahead_s.stats()["preemptions"] > 0
+
+
+def test_a_plan_that_must_preempt_reads_the_step_in_flight_first():
+    ex = AheadExecutor(num_pages=6, page_size=4)
+    s = Scheduler(ex)
+    sinks = [submit(s, [100 * (i + 1)] + [0] * 6, max_new=12)[0] for i in range(3)]
+    s.run_until_idle()
+    assert [x.tokens for x in sinks] == [[100 * (i + 1) + k for k in range(1, 13)] for i in range(3)]
+    assert s.stats()["preemptions"] > 0 and ex.all_free()
+
+
+def test_cancel_with_a_step_in_flight():
+    ex = AheadExecutor()
+    s = Scheduler(ex)
+    a, ra = submit(s, [100], max_new=10)
+    b, _ = submit(s, [200], max_new=4)
+    s.step(); s.step()                                               # the second step is in flight
+    assert a.tokens == [101]
+    ra.cancel()
+    s.run_until_idle()
+    assert a.tokens == [101] and b.tokens == [201, 202, 203, 204] and ex.all_free()
+    assert s.stats()["dropped_tokens"] == 1
+
+
+def test_an_error_at_collect_fails_the_running_requests():
+    ex = AheadExecutor()
+    s = Scheduler(ex)
+    a, _ = submit(s, [100], max_new=5)
+    s.step(); s.step()
+    ex.fail_next_collect = True
+    assert s.step() is True
+    assert a.error == "late boom" and ex.all_free()
+    ex.uncollected = 0                                               # the failed step's successor is forgotten
+    c, _ = submit(s, [300], max_new=2)
+    s.run_until_idle()
+    assert c.tokens == [301, 302] and c.error is None
+
+
+def test_step_ahead_can_be_switched_off():
+    ex = AheadExecutor()
+    s = Scheduler(ex, step_ahead=False)
+    a, _ = submit(s, [100], max_new=3)
+    s.run_until_idle()
+    assert a.tokens == [101, 102, 103] and ex.launched_ahead == 0 and ex.uncollected == 0
