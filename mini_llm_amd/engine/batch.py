@@ -31,12 +31,21 @@ class GroupStepData:
     slots: object          # int32 [n_tokens]: cache row each token's key/value is written to
 
 
+# Portions up to this long are laid out before the longer ones, whatever the order of the
+# entries, so that a mixer can treat the two kinds apart (single decoded tokens over long
+# contexts beside long portions want different kernels) by cutting the batch at one row.
+SHORT_PORTION = 8
+
+
 @dataclass
 class StepBatch:
     n_tokens: int
     n_requests: int
     n_logit_rows: int
     max_q_len: int          # the longest portion in the batch
+    short_requests: int     # the first so many requests bring portions of at most SHORT_PORTION tokens,
+    short_rows: int         # which are the first so many rows; the requests after them bring longer ones
+    short_portion: int = field(default=SHORT_PORTION, init=False)
     max_total_len: int      # the longest sequence after this step
     tokens: object          # int32 [n_tokens]
     positions: object       # int32 [n_tokens]
@@ -111,9 +120,18 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
 
     ``capacity`` pads the batch to that many tokens and requests with rows that do nothing (token
     -1, request -1, slot -1), so that the layout depends on the capacity alone; ``device_buffer``
-    then is the fixed device buffer the batch is copied into (a captured graph reads it)."""
+    then is the fixed device buffer the batch is copied into (a captured graph reads it).
+
+    The requests are laid out short portions first (SHORT_PORTION); the logit rows keep the order
+    of the entries as given."""
     n_requests = len(entries)
+    given = entries
+    layout = sorted(range(n_requests), key=lambda i: len(given[i].tokens) > SHORT_PORTION)  # stable
+    place = {i: at for at, i in enumerate(layout)}   # entry as given -> its place in the layout
+    entries = [given[i] for i in layout]
     q_lens = [len(e.tokens) for e in entries]
+    short_requests = sum(1 for q in q_lens if q <= SHORT_PORTION)
+    short_rows = sum(q for q in q_lens if q <= SHORT_PORTION)
     n_tokens = sum(q_lens)
     contexts = [cache.length(e.request_id) for e in entries]
     n_groups = len(cache.groups)
@@ -130,7 +148,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     q_starts = np.full(cap_requests + 1, n_tokens, dtype=np.int32)
     q_starts[0] = 0
     q_starts[1 : n_requests + 1] = np.cumsum(q_lens)
-    logit_rows = np.asarray([q_starts[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
+    logit_rows = np.asarray([q_starts[place[i]] + w for i, e in enumerate(given) for w in e.want], dtype=np.int32)
     state_slots = np.asarray([cache.requests[e.request_id].state_slot for e in entries], dtype=np.int32)
     token_sources = np.full(cap_tokens, -1, dtype=np.int32)
     for i, e in enumerate(entries):
@@ -147,7 +165,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
             slot[q_starts[i] : q_starts[i + 1]] = pages[pos // cache.page_size] * cache.page_size + pos % cache.page_size
         tables.append(table)
         slots.append(slot)
-    logit_slots = np.asarray([state_slots[i] for i, e in enumerate(entries) for _ in e.want], dtype=np.int32)
+    logit_slots = np.asarray([state_slots[place[i]] for i, e in enumerate(given) for _ in e.want], dtype=np.int32)
     n_logit_rows = len(logit_rows)
     if capacity is not None:
         logit_rows = _pad(logit_rows, cap_tokens, 0)
@@ -181,6 +199,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     ]
     return StepBatch(
         n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
+        short_requests=short_requests, short_rows=short_rows,
         max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
@@ -253,6 +272,7 @@ class DecodeBatchBuilder:
                   for g in range(n_groups)]
         return StepBatch(
             n_tokens=self.capacity, n_requests=self.capacity, n_logit_rows=self.capacity, max_q_len=1,
+            short_requests=self.capacity, short_rows=self.capacity,
             max_total_len=self.cache.max_length, tokens=views[0], positions=views[1], token_request=views[2],
             q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], token_sources=views[7],
             logit_slots=views[5],  # every request has one logit row, in its own place

@@ -261,7 +261,8 @@ DECODE_MIN_SPLIT = 64       # keys a wave should at least have
 DECODE_MAX_SPLITS = 16      # waves per block
 
 
-def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None):
+def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
+                    short_rows=None, short_requests=None):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
@@ -270,7 +271,11 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     sequence after this step) only sets how many waves share a token's keys. ``q_starts``
     ([requests + 1], first row of each request's portion; its rows are contiguous) and
     ``context_lens`` ([requests], keys stored before this step) let long portions take the
-    matrix-core kernel, which walks tiles of one request's queries."""
+    matrix-core kernel, which walks tiles of one request's queries. ``short_rows`` and
+    ``short_requests``: the first so many rows are the portions of the first so many requests and
+    none of them is longer than DECODE_MAX_Q_LEN, while the rest are longer portions; a batch of
+    both kinds then runs as two launches, each kind in its own kernel (a single decoded token with
+    a long context would otherwise walk all its keys in one wave of the kernel for portions)."""
     _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     page_size = k_pages.shape[2]
     width = n_heads * head_size
@@ -289,6 +294,19 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     if n == 0:
         return out
     rows_aligned = q.data_ptr() % 16 == 0 and (q.stride(0) * q.element_size()) % 16 == 0  # 16-byte loads of q
+    if (short_rows is not None and short_requests is not None and 0 < short_rows < n and max_q_len is not None
+            and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None and rows_aligned
+            and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))
+            and lib.mllm_attention_prefill_supported(head_size, page_size)):
+        _require(0 < short_requests < context_lens.shape[0], "short_requests does not cut the batch in two")
+        common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len)
+        paged_attention(q[:short_rows], k_pages, v_pages, token_request, positions, block_tables, max_q_len=DECODE_MAX_Q_LEN,
+                        q_starts=q_starts[: short_requests + 1], context_lens=context_lens[:short_requests],
+                        out=out[:short_rows], **common)
+        # the longer portions: their requests' entries of q_starts still count rows from the top of q
+        paged_attention(q, k_pages, v_pages, token_request, positions, block_tables[short_requests:], max_q_len=max_q_len,
+                        q_starts=q_starts[short_requests:], context_lens=context_lens[short_requests:], out=out, **common)
+        return out
     if (max_q_len is not None and max_q_len <= DECODE_MAX_Q_LEN and rows_aligned
             and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))):
         # decoding and short portions: a block per (token, head) whose waves share the keys; more

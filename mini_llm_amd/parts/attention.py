@@ -62,6 +62,8 @@ class CausalSelfAttention(Mixer):
             self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
             max_q_len=ctx.batch.max_q_len, max_len=ctx.batch.max_total_len,
             q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens,
+            **({"short_rows": ctx.batch.short_rows, "short_requests": ctx.batch.short_requests}
+               if ctx.batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
         )
         return self.out.forward(mixed, residual=residual)
 

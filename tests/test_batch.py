@@ -34,3 +34,38 @@ def test_decode_builder_matches_the_general_one():
         assert (fast.n_tokens, fast.n_requests, fast.n_logit_rows, fast.max_q_len) == (8, 8, 8, 1)
         for e in entries:
             cache.commit(e.request_id, 1)
+
+
+def test_short_portions_are_laid_out_first_and_logit_rows_keep_the_given_order():
+    groups = [CacheGroupSpec("full", (0,), 2, 16, None)]
+    cache = CacheManager(groups, {}, num_pages=40, page_size=16, max_requests=8, max_length=200)
+    for name, length in (("a", 30), ("b", 0), ("c", 7), ("d", 50), ("e", 3)):
+        cache.open(name)
+        if length:
+            cache.reserve(name, length); cache.commit(name, length)
+    entries = [
+        StepEntry("b", list(range(100, 120)), [19]),     # a long portion, given first
+        StepEntry("a", [7], [0]),                        # a decoded token
+        StepEntry("d", list(range(200, 209)), []),       # nine tokens: long, nothing wanted
+        StepEntry("c", [1, 2, 3, 4, 5, 6, 7, 8], [7, 0]),  # eight tokens: still short
+        StepEntry("e", [9], [0], from_slot=True),
+    ]
+    for e in entries:
+        cache.reserve(e.request_id, len(e.tokens))
+    batch = build_step_batch(entries, cache, None, vocab_size=1000)
+    assert batch.request_ids == ["a", "c", "e", "b", "d"]
+    assert (batch.short_requests, batch.short_rows, batch.max_q_len) == (3, 10, 20)
+    assert batch.q_starts.tolist() == [0, 1, 9, 10, 30, 39]
+    assert batch.tokens.tolist() == [7] + [1, 2, 3, 4, 5, 6, 7, 8] + [9] + list(range(100, 120)) + list(range(200, 209))
+    assert batch.context_lens.tolist() == [30, 7, 3, 0, 50]
+    assert batch.positions.tolist() == [30] + list(range(7, 15)) + [3] + list(range(20)) + list(range(50, 59))
+    assert batch.token_request.tolist() == [0] + [1] * 8 + [2] + [3] * 20 + [4] * 9
+    # logits come in the order of the entries as given and of each want
+    assert batch.logit_rows.tolist() == [29, 0, 8, 1, 9]
+    slot = {name: cache.requests[name].state_slot for name in "abcde"}
+    assert batch.logit_slots.tolist() == [slot["b"], slot["a"], slot["c"], slot["c"], slot["e"]]
+    assert batch.state_slots.tolist() == [slot[n] for n in "acebd"]
+    assert batch.token_sources.tolist() == [-1] * 9 + [slot["e"]] + [-1] * 29
+    for i, name in enumerate("acebd"):
+        pages = cache.block_table(name, 0)
+        assert batch.groups[0].block_tables[i, : len(pages)].tolist() == list(pages)

@@ -175,7 +175,7 @@ def plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window):
     return out[total - nq :]
 
 
-@pytest.mark.parametrize("path", ["general", "split_keys", "split_keys_balanced", "matrix_cores"])
+@pytest.mark.parametrize("path", ["general", "split_keys", "split_keys_balanced", "matrix_cores", "two_kinds"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize(
     "n_heads,n_kv_heads,head_size,page_size,window",
@@ -186,14 +186,16 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     # general: a wave per (token, head). split_keys: the decode kernel (forced for every row by
     # promising short portions; it treats rows independently, so the promise costs only speed),
     # with the splits laid over the tables' whole reach or balanced over the longest sequence.
-    # matrix_cores: the prefill kernel, a block per tile of one request's queries.
+    # matrix_cores: the prefill kernel, a block per tile of one request's queries. two_kinds: short
+    # portions first, which take the decode kernel, then long ones, which take the prefill kernel
+    # (two launches where both kernels take the head size, else one as before).
     if path.startswith("split") and head_size not in (16, 32, 64, 128, 256):
         pytest.skip("the split-key kernel takes power-of-two head sizes; others go the general way")
     if path == "matrix_cores" and head_size > 128:
         pytest.skip("the matrix-core kernel takes head sizes up to 128; larger go the general way")
     rng = np.random.default_rng(n_heads * 100 + head_size)
     # three requests: (cached context, new tokens); pages handed out in a scrambled order
-    shapes = [(0, 70), (150, 1), (61, 9)]
+    shapes = [(150, 1), (200, 1), (61, 5), (0, 70), (40, 9)] if path == "two_kinds" else [(0, 70), (150, 1), (61, 9)]
     num_pages = 40
     order = rng.permutation(num_pages).tolist()
     kp = torch.full((num_pages, n_kv_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
@@ -206,7 +208,7 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
         total = ctx + new
         k_all, v_all = rnd(total, n_kv_heads * head_size), rnd(total, n_kv_heads * head_size)
         q = rnd(new, n_heads * head_size)
-        if r == 0:  # one far key stands out for the last query: a missed tile would show
+        if (ctx, new) == (0, 70):  # one far key stands out for the last query: a missed tile would show
             far = q[-1].reshape(n_heads, head_size)[:: n_heads // n_kv_heads].reshape(-1) * 4
             k_all[3] = bf16_round(far) if dtype == torch.bfloat16 else far
         n_blocks = (total + page_size - 1) // page_size
@@ -222,9 +224,11 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
         tpos += list(range(ctx, total))
         refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window or None))
     extra = {}
-    if path == "matrix_cores":
+    if path in ("matrix_cores", "two_kinds"):
         starts = np.cumsum([0] + [new for _, new in shapes])
         extra = dict(q_starts=dev(starts, torch.int32), context_lens=dev([c for c, _ in shapes], torch.int32))
+        if path == "two_kinds":
+            extra.update(short_rows=7, short_requests=3)
     else:  # a padding row in the middle
         q_rows.insert(1, np.zeros((1, n_heads * head_size)))
         treq.insert(shapes[0][1], -1)
@@ -233,7 +237,7 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     out = K.paged_attention(
         dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
         n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window,
-        max_q_len={"general": None, "matrix_cores": 70}.get(path, 1), max_len=151 if path == "split_keys_balanced" else None, **extra,
+        max_q_len={"general": None, "matrix_cores": 70, "two_kinds": 70}.get(path, 1), max_len=151 if path == "split_keys_balanced" else None, **extra,
     )
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)

@@ -130,6 +130,8 @@ def run_mixer_in_portions(mixer, cache, staging, sequences, cuts, layer=0):
         for e in entries:
             cache.reserve(e.request_id, len(e.tokens))
         batch = build_step_batch(entries, cache, staging, vocab_size=1)
+        sizes = dict(step)
+        step = [(name, sizes[name]) for name in batch.request_ids]  # the rows lie in the batch's order: short portions first
         x = np.concatenate([sequences[name][fed[name] : fed[name] + n] for name, n in step])
         ctx = cache.layer_context(batch, LayerCall(0, layer))
         out = host(mixer.forward(dev(x), torch.zeros((len(x), x.shape[1]), device=DEV), ctx))
