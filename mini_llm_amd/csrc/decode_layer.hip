@@ -812,7 +812,8 @@ __global__ __launch_bounds__(256) void pending_sum_kernel(PendingSum in, float* 
 template <typename OutT>
 __global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, const int* __restrict__ row_index,
                                                                 const float* __restrict__ gamma, const float* __restrict__ beta,
-                                                                OutT* __restrict__ out, int width, float eps) {
+                                                                OutT* __restrict__ out, float* __restrict__ summed, int width,
+                                                                float eps) {
     extern __shared__ f32x4 row_pieces[];  // width / 4
     __shared__ float red[2][4];
     const int tid = threadIdx.x, n_pieces = width / 4;
@@ -821,6 +822,7 @@ __global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, c
     for (int piece = tid; piece < n_pieces; piece += 256) {
         f32x4 value = pending_piece(in, source, width, piece);
         row_pieces[piece] = value;
+        if (summed) *reinterpret_cast<f32x4*>(summed + (size_t)blockIdx.x * width + 4 * piece) = value;  // the row with its sums taken
         sum += (value[0] + value[1]) + (value[2] + value[3]);
     }
     sum = wave_total(sum);
@@ -971,9 +973,10 @@ MLLM_API int mllm_pending_sum(const float* base, const float* partials, const fl
 
 
 // LayerNorm of pending rows; row_index (or null) names the pending row of each of the n_rows output rows.
+// summed (or null): [n_rows, width], also gets each of those rows with its sums taken, not normalised.
 MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, const float* pending_bias, int n_partials,
                                     int pending_rows, const int* row_index, const float* gamma, const float* beta, void* out,
-                                    int n_rows, int width, float eps, int out_dtype, hipStream_t stream) {
+                                    float* summed, int n_rows, int width, float eps, int out_dtype, hipStream_t stream) {
     MLLM_REQUIRE(base != nullptr && out != nullptr, "pending_layernorm: no rows");
     MLLM_REQUIRE(n_partials >= 0 && (n_partials == 0 || partials != nullptr), "pending_layernorm: %d partial rows without memory", n_partials);
     MLLM_REQUIRE(width > 0 && width % 4 == 0 && width <= 32768, "pending_layernorm: width %d is not a multiple of 4 up to 32768", width);
@@ -982,9 +985,9 @@ MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, co
     PendingSum in{base, partials, pending_bias, n_partials, pending_rows};
     const size_t lds = (size_t)width * 4;
     if (out_dtype == MLLM_F32)
-        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, width, eps);
+        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, summed, width, eps);
     else if (out_dtype == MLLM_BF16)
-        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, width, eps);
+        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, summed, width, eps);
     else
         MLLM_REQUIRE(false, "pending_layernorm: unknown output dtype %d", out_dtype);
     return mllm_check_launch("pending_layernorm");

@@ -273,7 +273,7 @@ template <typename T, typename OutT, int MT, int KSPLIT, bool PACKED>
 __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     const T* __restrict__ A, const T* __restrict__ W, const float* __restrict__ bias,
     const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue,
-    CacheScatter scatter) {
+    CacheScatter scatter, int steps_per_block) {
     constexpr int VEC = Tile<T>::VEC;
     constexpr int KSTEP = 4 * VEC;  // k covered by one load of the wave: 4 lane groups x 16 bytes
     // Loads in flight per wave before any is used. At decode sizes a wave's whole share of K fits
@@ -301,9 +301,15 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         x_row[i] = A + (size_t)(x_valid[i] ? t : 0) * K;
     }
 
-    // wave w takes k-steps w, w + KSPLIT, ... in groups of UNROLL
+    // The block takes the k-steps first_step .. last_step-1: all of them, or, when the launch has
+    // several blocks per 16 columns (gridDim.y), its part of K, whose sums then go to matrix
+    // blockIdx.y of `out` (partial products; the caller passes no bias, residual or epilogue).
+    // Wave w takes the steps in groups of UNROLL, every KSPLIT-th group.
     const int n_steps = (K + KSTEP - 1) / KSTEP;
-    for (int step0 = wave * UNROLL; step0 < n_steps; step0 += KSPLIT * UNROLL) {
+    const int first_step = blockIdx.y * steps_per_block;
+    const int last_step = min(n_steps, first_step + steps_per_block);
+    out += (size_t)blockIdx.y * M * N;
+    for (int step0 = first_step + wave * UNROLL; step0 < last_step; step0 += KSPLIT * UNROLL) {
         Vec16 w_piece[UNROLL], x_piece[UNROLL][MT];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
@@ -319,7 +325,7 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         // what lies outside the matrices is zeroed only now, so that nothing above waits for a load
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
-            bool k_valid = (step0 + u) * KSTEP + quad * VEC < K;
+            bool k_valid = (step0 + u) * KSTEP + quad * VEC < K && step0 + u < last_step;
             w_piece[u] = mask_piece(w_piece[u], k_valid && n_valid);
 #pragma unroll
             for (int i = 0; i < MT; i++) x_piece[u][i] = mask_piece(x_piece[u][i], k_valid && x_valid[i]);
@@ -382,32 +388,35 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 
 template <typename T, typename OutT, int MT>
 void launch_skinny(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M,
-                   int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}) {
+                   int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
     constexpr int KSTEP = 4 * Tile<T>::VEC;
+    constexpr int UNROLL = MT == 1 ? 8 : 4;
     int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
+    int steps_per_block = k_blocks == 1 ? steps : ceil_div(ceil_div(steps, k_blocks), UNROLL) * UNROLL;
     int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
-    while (split < 16 && tiles * split < 2048 && steps >= 8 * split) split *= 2;
-    dim3 grid(tiles);
-    if (split == 16) {
-        if (packed) gemm_skinny_kernel<T, OutT, MT, 16, true><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-        else gemm_skinny_kernel<T, OutT, MT, 16, false><<<grid, 1024, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    }
-    else if (split == 1) {
-        if (packed) gemm_skinny_kernel<T, OutT, MT, 1, true><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-        else gemm_skinny_kernel<T, OutT, MT, 1, false><<<grid, 64, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    }
-    else if (split == 2) {
-        if (packed) gemm_skinny_kernel<T, OutT, MT, 2, true><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-        else gemm_skinny_kernel<T, OutT, MT, 2, false><<<grid, 128, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    }
-    else if (split == 4) {
-        if (packed) gemm_skinny_kernel<T, OutT, MT, 4, true><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-        else gemm_skinny_kernel<T, OutT, MT, 4, false><<<grid, 256, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    }
-    else {
-        if (packed) gemm_skinny_kernel<T, OutT, MT, 8, true><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-        else gemm_skinny_kernel<T, OutT, MT, 8, false><<<grid, 512, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    }
+    while (split < 16 && tiles * k_blocks * split < 2048 && steps_per_block >= 8 * split) split *= 2;
+    dim3 grid(tiles, k_blocks);
+#define MLLM_SKINNY_CASE(SPLIT)                                                                                                   \
+    if (packed) gemm_skinny_kernel<T, OutT, MT, SPLIT, true><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block); \
+    else gemm_skinny_kernel<T, OutT, MT, SPLIT, false><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block);
+    if (split == 16) { MLLM_SKINNY_CASE(16) }
+    else if (split == 1) { MLLM_SKINNY_CASE(1) }
+    else if (split == 2) { MLLM_SKINNY_CASE(2) }
+    else if (split == 4) { MLLM_SKINNY_CASE(4) }
+    else { MLLM_SKINNY_CASE(8) }
+#undef MLLM_SKINNY_CASE
+}
+
+// Blocks along K that a product of few rows should be cut into, each leaving a partial product:
+// when the columns alone leave most compute units idle (every block reads all rows of x, so a
+// long K with few columns is slow however few bytes the matrix has) and every block still gets
+// eight steps. It depends on N and K only.
+template <typename T>
+int skinny_k_blocks(int N, int K) {
+    int tiles = ceil_div(N, 16), steps = ceil_div(K, 4 * Tile<T>::VEC);
+    int k_blocks = 1;
+    while (k_blocks < 8 && tiles * k_blocks < 256 && steps >= 16 * k_blocks) k_blocks *= 2;
+    return k_blocks;
 }
 
 int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
@@ -481,6 +490,34 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
     else
         MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
     return mllm_check_launch("gemm");
+}
+
+// How many partial products mllm_gemm_split should be asked for at these sizes (1: the product is
+// better left whole).
+MLLM_API int mllm_gemm_split_blocks(int N, int K, int in_dtype) {
+    if (N <= 0 || K <= 0) return 1;
+    if (in_dtype == MLLM_F32) return K % 4 ? 1 : skinny_k_blocks<float>(N, K);
+    if (in_dtype == MLLM_BF16) return K % 8 ? 1 : skinny_k_blocks<bf16_t>(N, K);
+    return 1;
+}
+
+// A . W^T of at most 64 rows as k_blocks partial products over consecutive parts of K:
+// partials [k_blocks, M, N] in 32-bit, whose sum (in any fixed order) is the product. For a long
+// K with few output columns; whoever takes the partial products adds bias and residual.
+MLLM_API int mllm_gemm_split(const void* A, const void* W, int w_packed, float* partials, int M, int N, int K,
+                             int in_dtype, int k_blocks, hipStream_t stream) {
+    MLLM_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_split: bad sizes M=%d N=%d K=%d (at most 64 rows)", M, N, K);
+    MLLM_REQUIRE(k_blocks >= 1 && k_blocks <= 16, "gemm_split: %d partial products is not in 1..16", k_blocks);
+    MLLM_REQUIRE(in_dtype == MLLM_F32 || in_dtype == MLLM_BF16, "gemm_split: unknown dtype %d", in_dtype);
+    MLLM_REQUIRE(K % (in_dtype == MLLM_F32 ? 4 : 8) == 0, "gemm_split: K=%d is not a multiple of a 16-byte piece", K);
+    if (M == 0) return 0;
+#define MLLM_SPLIT_CASE(T)                                                                                                     \
+    if (M <= 16) launch_skinny<T, float, 1>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);      \
+    else if (M <= 32) launch_skinny<T, float, 2>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks); \
+    else launch_skinny<T, float, 4>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);
+    if (in_dtype == MLLM_F32) { MLLM_SPLIT_CASE(float) } else { MLLM_SPLIT_CASE(bf16_t) }
+#undef MLLM_SPLIT_CASE
+    return mllm_check_launch("gemm_split");
 }
 
 // The fused q/k/v projection: q columns go to out_q [M, q_width], key and value columns straight

@@ -80,9 +80,15 @@ def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots
     return out
 
 
-def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None):
+def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None, with_sums=False):
     """Row LayerNorm of float32 rows, plain or pending (PendingRows: the sums are taken on the way
-    in); ``row_index`` (int32) picks the input row of each output row."""
+    in); ``row_index`` (int32) picks the input row of each output row. ``with_sums``: returns
+    (normalised rows, the rows with their sums taken) - what the residual stream goes on with."""
+    if with_sums:
+        _require(row_index is None, "the rows with their sums taken are not gathered")
+        if not isinstance(x, PendingRows) or x.base.shape[1] % 4 or (x.partials is None and x.bias is None):
+            x = settle(x)
+            return layernorm(x, gamma, beta, eps, out_dtype=out_dtype, out=out), x
     pending = isinstance(x, PendingRows)
     if pending and x.base.shape[1] % 4:
         x, pending = settle(x), False
@@ -104,8 +110,11 @@ def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=
     _device_tensor(out, "out", out_dtype, 2)
     _require(tuple(out.shape) == (n, width), "out has the wrong shape")
     if pending:
+        summed = torch.empty_like(base) if with_sums else None
         check(library().mllm_pending_layernorm(_ptr(base), _ptr(partials), _ptr(bias), n_partials, base.shape[0], _ptr(row_index), _ptr(gamma),
-                                               _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
+                                               _ptr(beta), _ptr(out), _ptr(summed), n, width, float(eps), _code(out_dtype), _stream()))
+        if with_sums:
+            return out, summed
     else:
         check(library().mllm_layernorm(_ptr(base), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
     return out
@@ -194,6 +203,27 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
     _require(x.dtype != torch.float32 or out_dtype == torch.float32, "float32 inputs give float32 outputs")
     check(library().mllm_gemm(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x.dtype), _code(out_dtype), EPILOGUES[activation], _stream()))
     return out
+
+
+def split_blocks(weight, dtype) -> int:
+    """Into how many partial products along K ``linear_split`` should cut a product of few rows
+    with this weight (1: better left whole): more than one for few output columns and a long K."""
+    _, _, n, k = _matrix(weight, "weight", dtype)
+    return int(library().mllm_gemm_split_blocks(n, k, _code(dtype)))
+
+
+def linear_split(x, weight, k_blocks: int):
+    """x @ weight.T of at most 64 rows as ``k_blocks`` partial products over consecutive parts of
+    K: float32 [k_blocks, rows, out]; their sum is the product. The blocks of a product with few
+    output columns each read every row of x; cut along K they read a part, and many more run."""
+    _device_tensor(x, "x", dim=2)
+    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
+    m, k = x.shape
+    _require(w_cols == k, f"x has {k} columns but weight has {w_cols}")
+    _require(m <= 64, "partial products are for at most 64 rows")
+    partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=x.device)
+    check(library().mllm_gemm_split(_ptr(x), w_ptr, w_packed, _ptr(partials), m, n, k, _code(x.dtype), int(k_blocks), _stream()))
+    return partials
 
 
 def convert(src, dtype, transpose=False):

@@ -19,6 +19,8 @@ _SIGNATURES = {
     "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_split": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_split_blocks": [c_int, c_int, c_int],
     "mllm_gemm_qkv_cache": [P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_convert": [P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pack_matrix": [P, P, c_int, c_int, c_int, c_int, c_int, P],
@@ -37,7 +39,7 @@ _SIGNATURES = {
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_decode_mlp_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pending_sum": [P, P, P, c_int, P, c_int, c_int, P],
-    "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, c_int, c_int, c_float, c_int, P],
+    "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, P],
 }
 
 

@@ -90,6 +90,15 @@ class Norm(Part):
         """x: [rows, width] float32 -> [rows or len(row_index), width] of out_dtype."""
         raise NotImplementedError
 
+    def forward_with_sums(self, hidden, out_dtype):
+        """hidden: float32 rows, or rows whose last sums are pending -> (the normalised rows, the
+        rows with their sums taken: what the residual stream goes on with). A norm that can take
+        the sums on its way in overrides this."""
+        from ..ops import kernels
+
+        hidden = kernels.settle(hidden)
+        return self.forward(hidden, out_dtype), hidden
+
 
 class Mixer(Part):
     """Mixes information between the positions of a sequence (attention here)."""
@@ -112,10 +121,8 @@ class Mixer(Part):
         """norm, then ``forward``, then the residual sum, as one call: a mixer that has a kernel
         for the whole chain overrides this. ``hidden`` and the result are float32 rows or rows
         whose last sums are pending (ops.kernels.PendingRows)."""
-        from ..ops import kernels
-
-        hidden = kernels.settle(hidden)
-        return self.forward(norm.forward(hidden, compute_dtype), hidden, ctx)
+        x, hidden = norm.forward_with_sums(hidden, compute_dtype)
+        return self.forward(x, hidden, ctx)
 
 
 class FeedForward(Part):
@@ -125,10 +132,8 @@ class FeedForward(Part):
 
     def forward_normed(self, hidden, norm: Norm, compute_dtype, ctx: LayerContext):
         """norm, then ``forward``, then the residual sum, as one call (see Mixer.forward_normed)."""
-        from ..ops import kernels
-
-        hidden = kernels.settle(hidden)
-        return self.forward(norm.forward(hidden, compute_dtype), hidden)
+        x, hidden = norm.forward_with_sums(hidden, compute_dtype)
+        return self.forward(x, hidden)
 
 
 class PositionEncoding(Part):

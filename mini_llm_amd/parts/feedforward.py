@@ -37,7 +37,9 @@ class DenseMLP(FeedForward):
                 and self.up.weight.dtype == torch.bfloat16 and kernels.decode_layer_supported(self.width, inner=self.inner)):
             return kernels.decode_mlp_half(hidden, norm.weight, norm.bias, norm.eps, self.up.weight, self.up.bias,
                                            self.down.weight, self.down.bias, activation=self.activation)
-        return super().forward_normed(hidden, norm, compute_dtype, ctx)
+        # else kernel by kernel; the down product of few rows may come back with its sums pending
+        x, hidden = norm.forward_with_sums(hidden, compute_dtype)
+        return self.down.forward_pending(self.up.forward(x, activation=self.activation), hidden)
 
 
 register_part("feed_forward", "dense_mlp", DenseMLP)

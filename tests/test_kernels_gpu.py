@@ -584,6 +584,49 @@ def test_layernorm_of_pending_rows(K, out_dtype, rows, width, n_partials, with_b
     np.testing.assert_allclose(host(K.settle(hidden)), total, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_layernorm_gives_the_summed_rows_too(K, out_dtype, with_bias):
+    rng = np.random.default_rng(12)
+    rows, width = 37, 200
+    gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
+    tol = 1e-5 if out_dtype == torch.float32 else 1e-2
+    for n_partials in (0, 1, 5):
+        hidden, total = _pending_rows(K, rng, rows, width, n_partials, with_bias)
+        out, summed = K.layernorm(hidden, dev(gamma), dev(beta), 2e-5, out_dtype=out_dtype, with_sums=True)
+        np.testing.assert_allclose(host(summed), total, rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(host(out), P.layernorm(total, gamma, beta, 2e-5), rtol=tol, atol=tol)
+    plain = dev(total)
+    out, summed = K.layernorm(plain, dev(gamma), dev(beta), 2e-5, out_dtype=out_dtype, with_sums=True)
+    assert summed is plain
+    np.testing.assert_allclose(host(out), P.layernorm(total, gamma, beta, 2e-5), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k,k_blocks", [(1, 40, 2048, 8), (20, 100, 1000, 3), (64, 1024, 1104, 4), (48, 200, 520, 2), (33, 16, 64, 16), (7, 50, 96, 1)])
+def test_linear_split_leaves_partial_products(K, m, n, k, k_blocks, dtype, packed):
+    # the product of few rows cut along K: the partial products add up to it, whatever the cut
+    # (also one that leaves the last blocks without any k)
+    rng = np.random.default_rng(m + n + k)
+    rounded = bf16_round if dtype == torch.bfloat16 else (lambda a: a.astype(np.float32).astype(np.float64))
+    x, w = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k)
+    partials = K.linear_split(dev(x, dtype), as_weight(K, w, dtype, packed), k_blocks)
+    assert tuple(partials.shape) == (k_blocks, m, n) and partials.dtype == torch.float32
+    np.testing.assert_allclose(host(partials).astype(np.float64).sum(axis=0), rounded(x) @ rounded(w).T, rtol=2e-5, atol=2e-5)
+    if k == 2048:
+        assert (host(partials) != 0).any(axis=(1, 2)).all()  # every block had its share
+    with pytest.raises(K.OperandError, match="64 rows"):
+        K.linear_split(dev(np.zeros((65, k)), dtype), as_weight(K, w, dtype, packed), 2)
+
+
+def test_split_blocks_follow_the_shape(K):
+    # few output columns and a long K are cut; many columns, or a short K, are not
+    big = lambda n, k, dtype: K.split_blocks(torch.empty((n, k), dtype=dtype, device=DEV), dtype)
+    assert big(1024, 4096, torch.bfloat16) == 4 and big(768, 3072, torch.float32) == 8
+    assert big(4096, 1024, torch.bfloat16) == 1 and big(1024, 96, torch.bfloat16) == 1 and big(64, 64, torch.float32) == 1
+
+
 def test_embed_takes_tokens_from_slots(K):
     # rows whose source is not negative take their token from the slot the sampler left it in
     rng = np.random.default_rng(4)

@@ -87,6 +87,42 @@ def test_dense_mlp_part(activation, dtype):
     np.testing.assert_allclose(host(out), ref, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [20, 64, 65])
+def test_dense_mlp_with_a_long_inner_side(dtype, rows):
+    # few rows, few output columns, a long inner side: the down product comes back cut along K,
+    # its sums pending, and the next norm takes them (65 rows: whole, as before)
+    from mini_llm_amd.engine.batch import StepBatch
+    from mini_llm_amd.ops import kernels
+    from mini_llm_amd.parts import make_part
+    from mini_llm_amd.parts.base import LayerContext
+
+    width, inner, eps = 48, 1024, 1e-5
+    part = make_part("feed_forward", "dense_mlp", width=width, inner=inner, activation="gelu_new")
+    norm = make_part("norm", "layernorm", width=width, eps=eps)
+    w, wn = bind_random(part, 14, dtype), bind_random(norm, 15)
+    rng = np.random.default_rng(16)
+    td = torch.float32 if dtype == "float32" else torch.bfloat16
+    hidden = rng.standard_normal((rows, width)).astype(np.float32)
+
+    class Portion:  # all the feed-forward asks of the batch: these rows are no single decoded tokens
+        max_q_len = rows
+
+    class Ctx:
+        batch = Portion()
+
+    out = part.forward_normed(dev(hidden), norm, td, Ctx())
+    assert isinstance(out, kernels.PendingRows) == (rows <= 64)
+    x = host(dev(P.layernorm(hidden.astype(np.float64), wn["weight"], wn["bias"], eps), td))
+    ref = hidden + P.linear(P.gelu_new(P.linear(x, w["c_fc.weight"], w["c_fc.bias"])), w["c_proj.weight"], w["c_proj.bias"])
+    tol = 3e-5 if dtype == "float32" else 3e-2
+    np.testing.assert_allclose(host(kernels.settle(out)), ref, atol=tol, rtol=tol)
+    # and the norm that reads them next gives the sums back beside its own rows
+    normed, summed = norm.forward_with_sums(out, torch.float32)
+    np.testing.assert_allclose(host(summed), ref, atol=tol, rtol=tol)
+    np.testing.assert_allclose(host(normed), P.layernorm(host(summed).astype(np.float64), wn["weight"], wn["bias"], eps), atol=1e-4, rtol=1e-4)
+
+
 def test_embedding_positions_and_tied_head():
     from mini_llm_amd.parts import TiedHead, TokenEmbedding, make_part
 
