@@ -65,7 +65,7 @@ class CausalSelfAttention(Mixer):
             **({"short_rows": ctx.batch.short_rows, "short_requests": ctx.batch.short_requests}
                if ctx.batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
         )
-        return self.out.forward(mixed, residual=residual)
+        return self.out.forward_pending(mixed, residual)
 
     def forward_normed(self, hidden, norm, compute_dtype, ctx: LayerContext):
         # rows that are each the newest token of their request: the whole chain in one kernel

@@ -113,7 +113,7 @@ class Mixer(Part):
 
     def forward(self, x, residual, ctx: LayerContext):
         """x: [rows, width] normed input in the compute dtype; returns residual + mix(x) in
-        float32. Rows belong to several requests and may be a portion of a prompt or one decoded
+        float32 (plain rows, or rows whose last sums are pending: ops.kernels.PendingRows). Rows belong to several requests and may be a portion of a prompt or one decoded
         token; what came before is in the cache / the state slot."""
         raise NotImplementedError
 
@@ -127,7 +127,8 @@ class Mixer(Part):
 
 class FeedForward(Part):
     def forward(self, x, residual):
-        """x: [rows, width] in the compute dtype; returns residual + f(x) in float32."""
+        """x: [rows, width] in the compute dtype; returns residual + f(x) in float32 (plain rows, or
+        rows whose last sums are pending)."""
         raise NotImplementedError
 
     def forward_normed(self, hidden, norm: Norm, compute_dtype, ctx: LayerContext):
