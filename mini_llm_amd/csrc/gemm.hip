@@ -41,22 +41,23 @@ struct Tile<bf16_t> {
 // when the piece goes to LDS (mask_piece). Nothing then depends on a load until the tile is
 // staged, so all loads of two tiles stay in flight. Otherwise (unaligned K) the piece is gathered
 // element by element, zero where the matrix ends.
+// k_end: where the block's part of K ends (K itself unless several blocks share a tile along K).
 template <typename T, bool ALIGNED>
-__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k, int K, bool& valid) {
+__device__ __forceinline__ Vec16 load_piece(const T* __restrict__ base, int row, int n_rows, int k, int K, int k_end, bool& valid) {
     constexpr int VEC = Tile<T>::VEC;
     if constexpr (ALIGNED) {
-        valid = row < n_rows && k < K;
+        valid = row < n_rows && k < k_end;
         int safe_row = min(row, n_rows - 1), safe_k = min(k, K - VEC);
         return *reinterpret_cast<const Vec16*>(base + (size_t)safe_row * K + safe_k);
     } else {
         valid = true;
         Vec16 v = {{0u, 0u, 0u, 0u}};
-        if (row >= n_rows || k >= K) return v;
+        if (row >= n_rows || k >= k_end) return v;
         const T* p = base + (size_t)row * K + k;
         T* e = reinterpret_cast<T*>(&v);
 #pragma unroll
         for (int i = 0; i < VEC; i++)
-            if (k + i < K) e[i] = p[i];
+            if (k + i < k_end) e[i] = p[i];
         return v;
     }
 }
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                                                    const float* __restrict__ bias,
                                                    const float* __restrict__ residual,
                                                    OutT* __restrict__ out, int M, int N, int K,
-                                                   int epilogue, CacheScatter scatter) {
+                                                   int epilogue, CacheScatter scatter, int k_per_block) {
     constexpr int BK = Tile<T>::BK, VEC = Tile<T>::VEC, PAD = Tile<T>::PAD;
     constexpr int LDK = BK + PAD;
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
@@ -93,6 +94,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int half = lane / 32, lane32 = lane % 32;
+    // The block's part of K: all of it, or, when several blocks share the tile (gridDim.z), a run
+    // of k_per_block (a multiple of two LDS tiles), whose sums go to matrix blockIdx.z of `out`
+    // (partial products: the caller passes no bias, residual or epilogue).
+    const int k_begin = blockIdx.z * k_per_block, k_end = min(K, k_begin + k_per_block);
+    out += (size_t)blockIdx.z * M * N;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 #pragma unroll
         for (int i = 0; i < A_PIECES; i++) {
             int piece = tid + i * THREADS;
-            if (BM * VPR % THREADS == 0 || piece < BM * VPR) a_regs[set][i] = load_piece<T, ALIGNED>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K, a_valid[set][i]);
+            if (BM * VPR % THREADS == 0 || piece < BM * VPR) a_regs[set][i] = load_piece<T, ALIGNED>(A, m0 + piece / VPR, M, k0 + (piece % VPR) * VEC, K, k_end, a_valid[set][i]);
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; i++) {
@@ -117,10 +123,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                 if constexpr (PACKED) {
                     // 64 consecutive pieces are one chunk: 1 KiB of contiguous memory
                     int chunk = piece / 64, row_tile = n0 / 16 + chunk / CHUNKS_K, k_step = k0 / KC + chunk % CHUNKS_K;
-                    w_valid[set][i] = row_tile < w_row_tiles && k_step < w_k_steps;
+                    w_valid[set][i] = row_tile < w_row_tiles && k_step * KC < k_end;  // k_end is K or a multiple of the chunk
                     w_regs[set][i] = *reinterpret_cast<const Vec16*>(W + packed_offset<T>(min(row_tile, w_row_tiles - 1), min(k_step, w_k_steps - 1), w_k_steps, piece % 64));
                 } else {
-                    w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, w_valid[set][i]);
+                    w_regs[set][i] = load_piece<T, ALIGNED>(W, n0 + piece / VPR, N, k0 + (piece % VPR) * VEC, K, k_end, w_valid[set][i]);
                 }
             }
         }
@@ -196,12 +202,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
     // no branch around the loads, the wait before a tile is staged counts exactly the loads of the
     // other set that may still be in flight. One barrier a tile: while buffer b is multiplied, the
     // next tile goes into buffer 1-b, which every wave left before the barrier above.
-    fetch(0, 0);
-    fetch(1, BK);
+    fetch(0, k_begin);
+    fetch(1, k_begin + BK);
     stage(0);
-    fetch(0, 2 * BK);
+    fetch(0, k_begin + 2 * BK);
     __syncthreads();
-    for (int k0 = 0; k0 < K; k0 += 2 * BK) {
+    for (int k0 = k_begin; k0 < k_end; k0 += 2 * BK) {
         stage(1);  // tile k0 + BK (zeros beyond K)
         fetch(1, k0 + 3 * BK);
         products(0);
@@ -419,19 +425,32 @@ int skinny_k_blocks(int N, int K) {
     return k_blocks;
 }
 
+// The same for more rows (the tiled kernel, 128 x 64 tiles): cut while the tiles of the cut
+// product are no more than one and a half to a compute unit (measured: beyond that the partial
+// products cost more to write and add than the cut saves) and every block keeps eight LDS tiles of K.
+template <typename T>
+int tiled_k_blocks(int M, int N, int K) {
+    int tiles = ceil_div(M, 128) * ceil_div(N, 64);
+    int k_blocks = 1;
+    while (k_blocks < 8 && tiles * k_blocks * 2 <= 384 && K >= 8 * Tile<T>::BK * k_blocks * 2) k_blocks *= 2;
+    return k_blocks;
+}
+
 int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
 
 template <typename T, typename OutT, bool ALIGNED, int BM, int BN, int WAVES_M, int WAVES_N>
 void launch_tile(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
-                 int K, int epilogue, hipStream_t stream, CacheScatter scatter) {
-    dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
-    if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
-    else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter);
+                 int K, int epilogue, hipStream_t stream, CacheScatter scatter, int k_blocks) {
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM), k_blocks);
+    constexpr int PAIR = 2 * Tile<T>::BK;  // the kernel's loop takes two LDS tiles a turn
+    int k_per_block = k_blocks == 1 ? ceil_div(K, PAIR) * PAIR : ceil_div(ceil_div(K, k_blocks), PAIR) * PAIR;
+    if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block);
+    else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block);
 }
 
 template <typename T, typename OutT, bool ALIGNED>
 void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
-                  int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}) {
+                  int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
     int tile = g_forced_tile;
     if (tile == 0) {
         // measured on MI355X at GPT-2 sizes: many waves per block hide latency best
@@ -440,9 +459,9 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
         else tile = 7;
     }
     switch (tile) {  // other shapes (128x128, 256x128, fewer waves) were measured and lost at every size here
-        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
-        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter); break;
+        case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
+        case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
+        default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
     }
 }
 
@@ -494,19 +513,19 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
 
 // How many partial products mllm_gemm_split should be asked for at these sizes (1: the product is
 // better left whole).
-MLLM_API int mllm_gemm_split_blocks(int N, int K, int in_dtype) {
-    if (N <= 0 || K <= 0) return 1;
-    if (in_dtype == MLLM_F32) return K % 4 ? 1 : skinny_k_blocks<float>(N, K);
-    if (in_dtype == MLLM_BF16) return K % 8 ? 1 : skinny_k_blocks<bf16_t>(N, K);
+MLLM_API int mllm_gemm_split_blocks(int M, int N, int K, int in_dtype) {
+    if (M <= 0 || N <= 0 || K <= 0) return 1;
+    if (in_dtype == MLLM_F32) return K % 4 ? 1 : (M <= 64 ? skinny_k_blocks<float>(N, K) : tiled_k_blocks<float>(M, N, K));
+    if (in_dtype == MLLM_BF16) return K % 8 ? 1 : (M <= 64 ? skinny_k_blocks<bf16_t>(N, K) : tiled_k_blocks<bf16_t>(M, N, K));
     return 1;
 }
 
-// A . W^T of at most 64 rows as k_blocks partial products over consecutive parts of K:
-// partials [k_blocks, M, N] in 32-bit, whose sum (in any fixed order) is the product. For a long
-// K with few output columns; whoever takes the partial products adds bias and residual.
+// A . W^T as k_blocks partial products over consecutive parts of K: partials [k_blocks, M, N] in
+// 32-bit, whose sum (in any fixed order) is the product. For a long K with few output columns;
+// whoever takes the partial products adds bias and residual.
 MLLM_API int mllm_gemm_split(const void* A, const void* W, int w_packed, float* partials, int M, int N, int K,
                              int in_dtype, int k_blocks, hipStream_t stream) {
-    MLLM_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_split: bad sizes M=%d N=%d K=%d (at most 64 rows)", M, N, K);
+    MLLM_REQUIRE(M >= 0 && N > 0 && K > 0 && ceil_div(M, 32) <= 65535, "gemm_split: bad sizes M=%d N=%d K=%d", M, N, K);
     MLLM_REQUIRE(k_blocks >= 1 && k_blocks <= 16, "gemm_split: %d partial products is not in 1..16", k_blocks);
     MLLM_REQUIRE(in_dtype == MLLM_F32 || in_dtype == MLLM_BF16, "gemm_split: unknown dtype %d", in_dtype);
     MLLM_REQUIRE(K % (in_dtype == MLLM_F32 ? 4 : 8) == 0, "gemm_split: K=%d is not a multiple of a 16-byte piece", K);
@@ -514,7 +533,8 @@ MLLM_API int mllm_gemm_split(const void* A, const void* W, int w_packed, float* 
 #define MLLM_SPLIT_CASE(T)                                                                                                     \
     if (M <= 16) launch_skinny<T, float, 1>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);      \
     else if (M <= 32) launch_skinny<T, float, 2>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks); \
-    else launch_skinny<T, float, 4>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);
+    else if (M <= 64) launch_skinny<T, float, 4>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks); \
+    else launch_tiled<T, float, true>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);
     if (in_dtype == MLLM_F32) { MLLM_SPLIT_CASE(float) } else { MLLM_SPLIT_CASE(bf16_t) }
 #undef MLLM_SPLIT_CASE
     return mllm_check_launch("gemm_split");

@@ -205,22 +205,23 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
     return out
 
 
-def split_blocks(weight, dtype) -> int:
-    """Into how many partial products along K ``linear_split`` should cut a product of few rows
-    with this weight (1: better left whole): more than one for few output columns and a long K."""
+def split_blocks(weight, dtype, rows: int = 1) -> int:
+    """Into how many partial products along K ``linear_split`` should cut the product of ``rows``
+    rows with this weight (1: better left whole): more than one where few rows and few output
+    columns meet a long K. The same for all row counts up to 64, and for all that need the same
+    number of 128-row tiles."""
     _, _, n, k = _matrix(weight, "weight", dtype)
-    return int(library().mllm_gemm_split_blocks(n, k, _code(dtype)))
+    return int(library().mllm_gemm_split_blocks(int(rows), n, k, _code(dtype)))
 
 
 def linear_split(x, weight, k_blocks: int):
-    """x @ weight.T of at most 64 rows as ``k_blocks`` partial products over consecutive parts of
-    K: float32 [k_blocks, rows, out]; their sum is the product. The blocks of a product with few
-    output columns each read every row of x; cut along K they read a part, and many more run."""
+    """x @ weight.T as ``k_blocks`` partial products over consecutive parts of K: float32
+    [k_blocks, rows, out]; their sum is the product. The blocks of a product with few output
+    columns each read whole rows of x; cut along K they read a part, and many more run."""
     _device_tensor(x, "x", dim=2)
     w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
     m, k = x.shape
     _require(w_cols == k, f"x has {k} columns but weight has {w_cols}")
-    _require(m <= 64, "partial products are for at most 64 rows")
     partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=x.device)
     check(library().mllm_gemm_split(_ptr(x), w_ptr, w_packed, _ptr(partials), m, n, k, _code(x.dtype), int(k_blocks), _stream()))
     return partials

@@ -20,7 +20,7 @@ _SIGNATURES = {
     "mllm_add": [P, P, P, c_longlong, c_int, P],
     "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_gemm_split": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_gemm_split_blocks": [c_int, c_int, c_int],
+    "mllm_gemm_split_blocks": [c_int, c_int, c_int, c_int],
     "mllm_gemm_qkv_cache": [P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_convert": [P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pack_matrix": [P, P, c_int, c_int, c_int, c_int, c_int, P],

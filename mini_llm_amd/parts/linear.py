@@ -16,7 +16,7 @@ class Linear(Part):
         self.weight_std, self.bias_std = weight_std, bias_std
         self.weight = None
         self.bias = None
-        self._split_blocks = None
+        self._split_blocks = {}
 
     def tensor_specs(self):
         shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
@@ -28,15 +28,15 @@ class Linear(Part):
     def forward(self, x, activation=None, residual=None, out_dtype=None):
         return kernels.linear(x, self.weight, self.bias, activation=activation, residual=residual, out_dtype=out_dtype)
 
-    SPLIT_ROWS = 64
-
     def forward_pending(self, x, residual):
         """residual + x W + b, as float32 rows or, where few rows meet few output columns and a long
         K, as rows whose sums are pending: the product cut along K into partial products, which
         whoever reads the rows next adds up (kernels.PendingRows)."""
-        if x.shape[0] <= self.SPLIT_ROWS:
-            if self._split_blocks is None:
-                self._split_blocks = kernels.split_blocks(self.weight, x.dtype)
-            if self._split_blocks > 1:
-                return kernels.PendingRows(residual, kernels.linear_split(x, self.weight, self._split_blocks), self.bias)
+        rows = x.shape[0]
+        bucket = 0 if rows <= 64 else -(-rows // 128)  # the answer is the same inside a bucket
+        k_blocks = self._split_blocks.get((bucket, x.dtype))
+        if k_blocks is None:
+            k_blocks = self._split_blocks[bucket, x.dtype] = kernels.split_blocks(self.weight, x.dtype, rows)
+        if k_blocks > 1:
+            return kernels.PendingRows(residual, kernels.linear_split(x, self.weight, k_blocks), self.bias)
         return self.forward(x, residual=residual)

@@ -604,10 +604,11 @@ def test_layernorm_gives_the_summed_rows_too(K, out_dtype, with_bias):
 
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("m,n,k,k_blocks", [(1, 40, 2048, 8), (20, 100, 1000, 3), (64, 1024, 1104, 4), (48, 200, 520, 2), (33, 16, 64, 16), (7, 50, 96, 1)])
+@pytest.mark.parametrize("m,n,k,k_blocks", [(1, 40, 2048, 8), (20, 100, 1000, 3), (64, 1024, 1104, 4), (48, 200, 520, 2), (33, 16, 64, 16), (7, 50, 96, 1),
+                                            (65, 40, 2048, 4), (300, 130, 1000, 3), (129, 64, 520, 8), (200, 70, 96, 2)])
 def test_linear_split_leaves_partial_products(K, m, n, k, k_blocks, dtype, packed):
-    # the product of few rows cut along K: the partial products add up to it, whatever the cut
-    # (also one that leaves the last blocks without any k)
+    # the product cut along K: the partial products add up to it, whatever the cut (also one that
+    # leaves the last blocks without any k); up to 64 rows in the kernel for few rows, more in the tiled one
     rng = np.random.default_rng(m + n + k)
     rounded = bf16_round if dtype == torch.bfloat16 else (lambda a: a.astype(np.float32).astype(np.float64))
     x, w = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k)
@@ -616,15 +617,15 @@ def test_linear_split_leaves_partial_products(K, m, n, k, k_blocks, dtype, packe
     np.testing.assert_allclose(host(partials).astype(np.float64).sum(axis=0), rounded(x) @ rounded(w).T, rtol=2e-5, atol=2e-5)
     if k == 2048:
         assert (host(partials) != 0).any(axis=(1, 2)).all()  # every block had its share
-    with pytest.raises(K.OperandError, match="64 rows"):
-        K.linear_split(dev(np.zeros((65, k)), dtype), as_weight(K, w, dtype, packed), 2)
 
 
 def test_split_blocks_follow_the_shape(K):
     # few output columns and a long K are cut; many columns, or a short K, are not
-    big = lambda n, k, dtype: K.split_blocks(torch.empty((n, k), dtype=dtype, device=DEV), dtype)
+    big = lambda n, k, dtype, rows=1: K.split_blocks(torch.empty((n, k), dtype=dtype, device=DEV), dtype, rows)
     assert big(1024, 4096, torch.bfloat16) == 4 and big(768, 3072, torch.float32) == 8
     assert big(4096, 1024, torch.bfloat16) == 1 and big(1024, 96, torch.bfloat16) == 1 and big(64, 64, torch.float32) == 1
+    assert big(1024, 4096, torch.bfloat16, 64) == 4 and big(1024, 4096, torch.bfloat16, 512) == 4
+    assert big(1024, 4096, torch.bfloat16, 2048) == 1 and big(4096, 1024, torch.bfloat16, 512) == 1
 
 
 def test_embed_takes_tokens_from_slots(K):
