@@ -108,6 +108,24 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
+    // The residual rows of this lane's outputs are asked for now and arrive while the products
+    // run: asked for in the epilogue, every block would wait for them at the same time, with
+    // nothing left to overlap the trip with.
+    float early_residual[TM][TN][16];
+    float early_bias[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
+        early_bias[j] = bias && col < N ? bias[col] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                int row = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                early_residual[i][j][v] = residual && row < M && col < N ? residual[(size_t)row * N + col] : 0.0f;
+            }
+    }
+
     Vec16 a_regs[2][A_PIECES], w_regs[2][W_PIECES];
     bool a_valid[2][A_PIECES], w_valid[2][W_PIECES];
     auto fetch = [&](int set, int k0) {
@@ -225,7 +243,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
         for (int j = 0; j < TN; j++) {
             int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
             if (col >= N) continue;
-            float b = bias ? bias[col] : 0.0f;
+            float b = early_bias[j];
             if (scatter.enabled) {
                 // a fused q/k/v projection: the q columns go to out [M, q_width], this lane's key or
                 // value column into the cache pages at the rows' slots
@@ -261,7 +279,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                 if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
                 else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
                 size_t at = (size_t)row * N + col;
-                if (residual) value = residual[at] + value;
+                if (residual) value = early_residual[i][j][v] + value;
                 out[at] = from_float<OutT>(value);
             }
         }
@@ -425,13 +443,15 @@ int skinny_k_blocks(int N, int K) {
     return k_blocks;
 }
 
-// The same for more rows (the tiled kernel, 128 x 64 tiles): cut while the tiles of the cut
-// product are no more than one and a half to a compute unit (measured: beyond that the partial
-// products cost more to write and add than the cut saves) and every block keeps eight LDS tiles of K.
+// The same for more rows (the tiled kernel, 128 x 64 tiles): only a product whose tiles leave half
+// the compute units idle is cut, while the tiles of the cut product are no more than one and a
+// half to a compute unit and every block keeps eight LDS tiles of K (measured: a product that
+// nearly fills the chip gains less from the cut than adding the partial products up costs).
 template <typename T>
 int tiled_k_blocks(int M, int N, int K) {
     int tiles = ceil_div(M, 128) * ceil_div(N, 64);
     int k_blocks = 1;
+    if (tiles > 128) return 1;
     while (k_blocks < 8 && tiles * k_blocks * 2 <= 384 && K >= 8 * Tile<T>::BK * k_blocks * 2) k_blocks *= 2;
     return k_blocks;
 }
