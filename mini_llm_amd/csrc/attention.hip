@@ -201,7 +201,10 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const int position = positions[token];
     const int first_key = window > 0 ? max(0, position - window + 1) : 0;
     const int n_keys = position + 1 - first_key;
-    const int chunk = (((n_keys + n_splits - 1) / n_splits + RPI - 1) / RPI) * RPI;  // keys per wave
+    // keys per wave: whole rounds of the sweep (a round asks for KPI keys whether it needs them or
+    // not), so that a wave either has a full round to do or none
+    constexpr int KPI = KeySweep<T, HD>::KPI;
+    const int chunk = (((n_keys + n_splits - 1) / n_splits + KPI - 1) / KPI) * KPI;
     const int begin = first_key + split * chunk;
     const int end = min(position + 1, begin + chunk);  // exclusive
     const int sub = lane % LPR;

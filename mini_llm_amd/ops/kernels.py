@@ -287,7 +287,8 @@ def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_hea
 
 
 DECODE_MAX_Q_LEN = 8        # portions up to this many tokens take the split-key kernel
-DECODE_TARGET_WAVES = 4096  # waves that fill the chip (256 compute units, 16 each) and hide the latency of their loads
+DECODE_TARGET_WAVES = 4096  # the most waves a launch should have: 16 to each of 256 compute units are resident at once (measured: a
+                            # second round of blocks costs more than longer shares of the keys per wave)
 DECODE_MIN_SPLIT = 64       # keys a wave should at least have
 DECODE_MAX_SPLITS = 16      # waves per block
 
@@ -340,11 +341,12 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         return out
     if (max_q_len is not None and max_q_len <= DECODE_MAX_Q_LEN and rows_aligned
             and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))):
-        # decoding and short portions: a block per (token, head) whose waves share the keys; more
-        # waves per block when there are few blocks, never more than one per 64 keys of reach
+        # decoding and short portions: a block per (token, head) whose waves share the keys; as many
+        # waves per block as keep the launch within what is resident at once, never more than one
+        # per 64 keys of reach
         reach = block_tables.shape[1] * page_size if max_len is None else max(1, min(max_len, block_tables.shape[1] * page_size))
         n_splits = 1
-        while n_splits < DECODE_MAX_SPLITS and n * n_heads * n_splits < DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < reach:
+        while n_splits < DECODE_MAX_SPLITS and 2 * n * n_heads * n_splits <= DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < reach:
             n_splits *= 2
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), _stream()))
         return out
@@ -407,9 +409,10 @@ LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kerne
 
 def layer_kernel_rows(width: int) -> int:
     """Rows up to which the layer kernels for decoding beat the separate kernels (measured on
-    MI355X: at GPT-2 small's width up to 64 rows; at GPT-2 medium's they lose from 32 rows on, as
-    every (token, head) block reads its own copy of the partial rows and of the matrices)."""
-    return LAYER_KERNEL_MAX_ROWS if width <= 768 else min(16, LAYER_KERNEL_MAX_ROWS)
+    MI355X: at GPT-2 small's width up to 32 rows, at GPT-2 medium's up to 16; beyond, every
+    (token, head) block reading its own copy of the partial rows and of the matrices costs more
+    than the launches and round trips the fusion saves)."""
+    return min(32 if width <= 768 else 16, LAYER_KERNEL_MAX_ROWS)
 
 
 def _pending(hidden):
