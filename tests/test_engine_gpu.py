@@ -361,6 +361,7 @@ def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dt
         for temperature in (0.0, 0.9):
             if temperature == 0.0 and not ahead:
                 free = engine.generate(prompts, max_new_tokens=24)
+                assert engine.stats()["preemptions"] >= 1  # the pool is that small
                 ends = [tokens[5 + i] if i % 2 == 0 else None for i, tokens in enumerate(free)]
             outputs, errors = [[] for _ in prompts], []
             for i, prompt in enumerate(prompts):
