@@ -469,3 +469,26 @@ def test_step_ahead_can_be_switched_off():
     a, _ = submit(s, [100], max_new=3)
     s.run_until_idle()
     assert a.tokens == [101, 102, 103] and ex.launched_ahead == 0 and ex.uncollected == 0
+
+
+def test_thread_runs_one_step_ahead_and_stops_with_a_step_in_flight():
+    ex = AheadExecutor()
+    s = Scheduler(ex, max_batch=2)
+    s.start()
+    sinks = [submit(s, [100 * (i + 1)], max_new=5, eos=(203 if i == 1 else None))[0] for i in range(3)]
+    deadline = time.time() + 5
+    while any(x.finish is None for x in sinks) and time.time() < deadline:
+        time.sleep(0.01)
+    assert [x.tokens for x in sinks] == [[101, 102, 103, 104, 105], [201, 202, 203], [301, 302, 303, 304, 305]]
+    assert [x.finish for x in sinks] == ["length", "stop", "length"]
+    deadline = time.time() + 5
+    while s.has_work() and time.time() < deadline:   # the token past the end token is collected and dropped
+        time.sleep(0.01)
+    assert ex.all_free() and ex.launched_ahead > 0 and s.stats()["dropped_tokens"] == 1
+    slow_collect = ex.collect
+    ex.collect = lambda handle: (time.sleep(0.01), slow_collect(handle))[1]
+    endless, _ = submit(s, [400], max_new=None)                       # 63 tokens at 10 ms each
+    while len(endless.tokens) < 3:
+        time.sleep(0.001)
+    s.stop()                                                          # whatever is in flight is forgotten
+    assert endless.error is not None and "shutting down" in endless.error and ex.all_free()
