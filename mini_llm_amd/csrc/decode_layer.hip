@@ -742,8 +742,8 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
         const int unit = tile * 16 + 4 * (l / 16) + r, h = slice * U + unit;
         if (h < inner) {
             if (b_up) value += up_bias[i];
-            if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
-            else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+            if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh_for_bf16(value);
+            else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf_for_bf16(value);
         } else {
             value = 0.0f;
         }

@@ -276,8 +276,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                 int row = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
                 if (row >= M) continue;
                 float value = acc[i][j][v] + b;
-                if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
-                else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+                if (epilogue == MLLM_EPI_GELU_TANH) value = sizeof(OutT) == 2 ? gelu_tanh_for_bf16(value) : gelu_tanh(value);
+                else if (epilogue == MLLM_EPI_GELU_ERF) value = sizeof(OutT) == 2 ? gelu_erf_for_bf16(value) : gelu_erf(value);
                 size_t at = (size_t)row * N + col;
                 if (residual) value = early_residual[i][j][v] + value;
                 out[at] = from_float<OutT>(value);
@@ -387,8 +387,8 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 #pragma unroll
         for (int w = 0; w < KSPLIT; w++) value += sums[w][ir][l];  // the same order for every element
         if (bias) value += bias[col];
-        if (epilogue == MLLM_EPI_GELU_TANH) value = gelu_tanh(value);
-        else if (epilogue == MLLM_EPI_GELU_ERF) value = gelu_erf(value);
+        if (epilogue == MLLM_EPI_GELU_TANH) value = sizeof(OutT) == 2 ? gelu_tanh_for_bf16(value) : gelu_tanh(value);
+        else if (epilogue == MLLM_EPI_GELU_ERF) value = sizeof(OutT) == 2 ? gelu_erf_for_bf16(value) : gelu_erf(value);
         if (scatter.enabled) {
             if (col < scatter.q_width) {
                 out[(size_t)token * scatter.q_width + col] = from_float<OutT>(value);
