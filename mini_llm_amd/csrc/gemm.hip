@@ -473,14 +473,19 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
                   int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
     int tile = g_forced_tile;
     if (tile == 0) {
-        // measured on MI355X at GPT-2 sizes: many waves per block hide latency best
+        // measured on MI355X at GPT-2 sizes: many waves per block hide latency best; the large tile
+        // (sixteen waves, half the traffic from the cache of the chip for the same product) from
+        // about half a block a compute unit on, where it wins by 5 % (2,048 x 2,304 x 768) to 25 %
+        // (8,192 x 4,096 x 1,024)
         if (M <= 32) tile = 1;
         else if (M <= 64) tile = 2;
+        else if (k_blocks == 1 && ceil_div(M, 256) * ceil_div(N, 128) >= 128) tile = 3;
         else tile = 7;
     }
-    switch (tile) {  // other shapes (128x128, 256x128, fewer waves) were measured and lost at every size here
+    switch (tile) {  // other shapes (128x128, 256x128 with eight waves, fewer waves) were measured and lost at every size here
         case 1: launch_tile<T, OutT, ALIGNED, 32, 128, 1, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
         case 2: launch_tile<T, OutT, ALIGNED, 64, 64, 2, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
+        case 3: launch_tile<T, OutT, ALIGNED, 256, 128, 4, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
         default: launch_tile<T, OutT, ALIGNED, 128, 64, 4, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks); break;
     }
 }
@@ -510,7 +515,7 @@ void launch_gemm(const void* A, const void* W, bool packed, const float* bias, c
 
 }  // namespace
 
-// Tuning aid: forces one tile shape of the tiled kernel (1: 32x128, 2: 64x64, another number: 128x64; 0 gives the choice back to the sizes).
+// Tuning aid: forces one tile shape of the tiled kernel (1: 32x128, 2: 64x64, 3: 256x128, another number: 128x64; 0 gives the choice back to the sizes).
 MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
 MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* bias, const float* residual,

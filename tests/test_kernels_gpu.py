@@ -103,7 +103,8 @@ def test_pack_matrix(K, rows, cols, src, dst, transpose):
 
 
 GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
-               (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20)]
+               (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20),
+               (2100, 2010, 104)]  # many rows and columns: the large tile (256 x 128), with ragged edges
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -346,7 +347,8 @@ def test_operands_are_checked_on_the_host(K):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16), (65, 3, 3, 32, 16), (300, 5, 5, 48, 64)])
+@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16), (65, 3, 3, 32, 16), (300, 5, 5, 48, 64),
+                                                                         (2100, 14, 14, 48, 64)])  # enough rows and columns for the large tile
 @pytest.mark.parametrize("packed", [False, True])
 def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, packed):
     rng = np.random.default_rng(rows)
