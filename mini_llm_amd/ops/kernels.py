@@ -28,18 +28,24 @@ def _require(condition: bool, message: str) -> None:
 
 
 def _code(dtype: torch.dtype) -> int:
-    _require(dtype in _DTYPE_CODE, f"no kernel for element type {dtype}")
+    if not (dtype in _DTYPE_CODE):
+        raise OperandError(f"no kernel for element type {dtype}")
     return _DTYPE_CODE[dtype]
 
 
 def _device_tensor(t: torch.Tensor, name: str, dtype=None, dim=None) -> None:
-    _require(isinstance(t, torch.Tensor), f"{name} is not a tensor")
-    _require(t.is_cuda, f"{name} is not on the GPU: there is no CPU path")
+    if not (isinstance(t, torch.Tensor)):
+        raise OperandError(f"{name} is not a tensor")
+    if not (t.is_cuda):
+        raise OperandError(f"{name} is not on the GPU: there is no CPU path")
     if dtype is not None:
-        _require(t.dtype == dtype, f"{name} must be {dtype}, not {t.dtype}")
+        if not (t.dtype == dtype):
+            raise OperandError(f"{name} must be {dtype}, not {t.dtype}")
     if dim is not None:
-        _require(t.dim() == dim, f"{name} must have {dim} dimensions, not {t.dim()}")
-    _require(t.is_contiguous(), f"{name} must be contiguous")
+        if not (t.dim() == dim):
+            raise OperandError(f"{name} must have {dim} dimensions, not {t.dim()}")
+    if not (t.is_contiguous()):
+        raise OperandError(f"{name} must be contiguous")
 
 
 def _ptr(t: torch.Tensor | None):
@@ -185,8 +191,10 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
     _device_tensor(x, "x", dim=2)
     w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
     m, k = x.shape
-    _require(w_cols == k, f"x has {k} columns but weight has {w_cols}")
-    _require(activation in EPILOGUES, f"unknown activation {activation!r}")
+    if not (w_cols == k):
+        raise OperandError(f"x has {k} columns but weight has {w_cols}")
+    if not (activation in EPILOGUES):
+        raise OperandError(f"unknown activation {activation!r}")
     if bias is not None:
         _device_tensor(bias, "bias", torch.float32, 1)
         _require(bias.shape[0] == n, "bias does not match weight")
@@ -221,7 +229,8 @@ def linear_split(x, weight, k_blocks: int):
     _device_tensor(x, "x", dim=2)
     w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
     m, k = x.shape
-    _require(w_cols == k, f"x has {k} columns but weight has {w_cols}")
+    if not (w_cols == k):
+        raise OperandError(f"x has {k} columns but weight has {w_cols}")
     partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=x.device)
     check(library().mllm_gemm_split(_ptr(x), w_ptr, w_packed, _ptr(partials), m, n, k, _code(x.dtype), int(k_blocks), _stream()))
     return partials
@@ -256,8 +265,10 @@ def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
     num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     width = n_kv_heads * head_size
     for t, name in ((k_src, "k_src"), (v_src, "v_src")):
-        _require(t.is_cuda and t.dim() == 2 and t.dtype == k_pages.dtype, f"{name} must be a 2-D GPU tensor of the pages' type")
-        _require(t.shape[1] == width and t.stride(1) == 1, f"{name} must have {width} contiguous columns")
+        if not (t.is_cuda and t.dim() == 2 and t.dtype == k_pages.dtype):
+            raise OperandError(f"{name} must be a 2-D GPU tensor of the pages' type")
+        if not (t.shape[1] == width and t.stride(1) == 1):
+            raise OperandError(f"{name} must have {width} contiguous columns")
     _require(k_src.shape[0] == v_src.shape[0] and k_src.stride(0) == v_src.stride(0), "k_src and v_src differ in rows or stride")
     _device_tensor(slots, "slots", torch.int32, 1)
     n = k_src.shape[0]
@@ -312,7 +323,8 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     page_size = k_pages.shape[2]
     width = n_heads * head_size
     _require(q.is_cuda and q.dim() == 2 and q.dtype == k_pages.dtype, "q must be a 2-D GPU tensor of the pages' type")
-    _require(q.shape[1] == width and q.stride(1) == 1, f"q must have {width} contiguous columns")
+    if not (q.shape[1] == width and q.stride(1) == 1):
+        raise OperandError(f"q must have {width} contiguous columns")
     n = q.shape[0]
     _device_tensor(token_request, "token_request", torch.int32, 1)
     _device_tensor(positions, "positions", torch.int32, 1)
@@ -374,7 +386,8 @@ def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=N
     for t, name, dtype in ((temperatures, "temperatures", torch.float32), (top_ps, "top_ps", torch.float32), (seeds, "seeds", torch.int64), (steps, "steps", torch.int32)):
         if t is not None:
             _device_tensor(t, name, dtype, 1)
-            _require(t.shape[0] >= n, f"{name} has fewer entries than rows")
+            if not (t.shape[0] >= n):
+                raise OperandError(f"{name} has fewer entries than rows")
     if out is None:
         out = torch.empty((n,), dtype=torch.int32, device=logits.device)
     _device_tensor(out, "out", torch.int32, 1)
@@ -467,20 +480,24 @@ def decode_attention_half(hidden, gamma, beta, eps, w_qkv, b_qkv, w_out, b_out, 
     _norm_vectors(gamma, beta, width)
     num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     _require(k_pages.dtype == torch.bfloat16, "the layer kernels for decoding are bfloat16 only")
-    _require(decode_layer_supported(width, head_size, page_size), f"no layer kernel for width {width}, head size {head_size}, pages of {page_size}")
+    if not (decode_layer_supported(width, head_size, page_size)):
+        raise OperandError(f"no layer kernel for width {width}, head size {head_size}, pages of {page_size}")
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
     for w, name in ((w_qkv, "w_qkv"), (w_out, "w_out")):
-        _require(isinstance(w, PackedMatrix), f"{name} must be a PackedMatrix")
+        if not (isinstance(w, PackedMatrix)):
+            raise OperandError(f"{name} must be a PackedMatrix")
         _device_tensor(w.data, name, torch.bfloat16, 1)
     _require(w_qkv.shape == (q_width + 2 * kv_width, width), "w_qkv does not match the heads or the width")
     _require(w_out.shape == (width, q_width), "w_out does not match the heads or the width")
     for t, name, n in ((b_qkv, "b_qkv", q_width + 2 * kv_width), (b_out, "b_out", width)):
         if t is not None:
             _device_tensor(t, name, torch.float32, 1)
-            _require(t.shape[0] == n, f"{name} does not match its matrix")
+            if not (t.shape[0] == n):
+                raise OperandError(f"{name} does not match its matrix")
     for t, name in ((slots, "slots"), (token_request, "token_request"), (positions, "positions")):
         _device_tensor(t, name, torch.int32, 1)
-        _require(t.shape[0] >= rows, f"{name} has fewer entries than rows")
+        if not (t.shape[0] >= rows):
+            raise OperandError(f"{name} has fewer entries than rows")
     _device_tensor(block_tables, "block_tables", torch.int32, 2)
     summed = torch.empty_like(base)
     out = torch.empty((n_heads, rows, width), dtype=torch.float32, device=base.device)
@@ -499,17 +516,21 @@ def decode_mlp_half(hidden, gamma, beta, eps, w_up, b_up, w_down, b_down, activa
     base, partials, bias, n_partials = _pending(hidden)
     rows, width = base.shape
     _norm_vectors(gamma, beta, width)
-    _require(activation in EPILOGUES, f"unknown activation {activation!r}")
+    if not (activation in EPILOGUES):
+        raise OperandError(f"unknown activation {activation!r}")
     for w, name in ((w_up, "w_up"), (w_down, "w_down")):
-        _require(isinstance(w, PackedMatrix), f"{name} must be a PackedMatrix")
+        if not (isinstance(w, PackedMatrix)):
+            raise OperandError(f"{name} must be a PackedMatrix")
         _device_tensor(w.data, name, torch.bfloat16, 1)
     inner = w_up.rows
-    _require(decode_layer_supported(width, inner=inner), f"no layer kernel for width {width} with {inner} hidden units")
+    if not (decode_layer_supported(width, inner=inner)):
+        raise OperandError(f"no layer kernel for width {width} with {inner} hidden units")
     _require(w_up.shape == (inner, width) and w_down.shape == (width, inner), "the two matrices do not match the width")
     for t, name, n in ((b_up, "b_up", inner), (b_down, "b_down", width)):
         if t is not None:
             _device_tensor(t, name, torch.float32, 1)
-            _require(t.shape[0] == n, f"{name} does not match its matrix")
+            if not (t.shape[0] == n):
+                raise OperandError(f"{name} does not match its matrix")
     _require(slice_units in (64, 128), "slices of 64 or 128 hidden units")
     summed = torch.empty_like(base)
     out = torch.empty(((inner + slice_units - 1) // slice_units, rows, width), dtype=torch.float32, device=base.device)
