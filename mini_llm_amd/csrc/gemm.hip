@@ -479,7 +479,7 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
         // (8,192 x 4,096 x 1,024)
         if (M <= 32) tile = 1;
         else if (M <= 64) tile = 2;
-        else if (k_blocks == 1 && ceil_div(M, 256) * ceil_div(N, 128) >= 128) tile = 3;
+        else if (k_blocks == 1 && ceil_div(M, 256) * ceil_div(N, 128) >= (sizeof(T) == 4 ? 256 : 128)) tile = 3;  // 32-bit products are bound by the matrix cores: no compute unit may idle
         else tile = 7;
     }
     switch (tile) {  // other shapes (128x128, 256x128 with eight waves, fewer waves) were measured and lost at every size here

@@ -104,7 +104,7 @@ def test_pack_matrix(K, rows, cols, src, dst, transpose):
 
 GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
                (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20),
-               (2100, 2010, 104)]  # many rows and columns: the large tile (256 x 128), with ragged edges
+               (2100, 2010, 104), (4100, 2010, 40)]  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
 
 
 @pytest.mark.parametrize("packed", [False, True])
