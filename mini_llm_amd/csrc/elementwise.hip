@@ -27,6 +27,10 @@ __global__ void embed_kernel(int* __restrict__ tokens, const int* __restrict__ p
         return;
     }
     const T* token_row = wte + (size_t)token * width;
+    if (wpe == nullptr) {  // positions enter the model elsewhere (or nowhere)
+        for (int i = threadIdx.x; i < width; i += blockDim.x) out_row[i] = to_float(token_row[i]);
+        return;
+    }
     const T* position_row = wpe + (size_t)positions[row] * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x)
         out_row[i] = to_float(token_row[i]) + to_float(position_row[i]);

@@ -63,16 +63,18 @@ def _stream():
 
 
 def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots=None):
-    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32. A negative token gives a zero row.
+    """out[t] = wte[tokens[t]] + wpe[positions[t]] in float32 (``wpe`` None: the token row alone). A
+    negative token gives a zero row.
     With ``token_sources`` and ``token_slots`` the token of a row whose source is not negative is
     token_slots[source]; it is also written into ``tokens``."""
     _device_tensor(tokens, "tokens", torch.int32, 1)
     _device_tensor(positions, "positions", torch.int32, 1)
     _device_tensor(wte, "wte", dim=2)
-    _device_tensor(wpe, "wpe", wte.dtype, 2)
     n, width = tokens.shape[0], wte.shape[1]
     _require(positions.shape[0] == n, "tokens and positions differ in length")
-    _require(wpe.shape[1] == width, "wte and wpe differ in width")
+    if wpe is not None:
+        _device_tensor(wpe, "wpe", wte.dtype, 2)
+        _require(wpe.shape[1] == width, "wte and wpe differ in width")
     if token_sources is not None:
         _device_tensor(token_sources, "token_sources", torch.int32, 1)
         _device_tensor(token_slots, "token_slots", torch.int32, 1)

@@ -17,11 +17,12 @@ class TokenEmbedding(Part):
 
     def forward(self, tokens, positions, position_encoding: PositionEncoding | None, token_sources=None, token_slots=None):
         """[rows, width] float32: token rows, with the position rows added when the encoding
-        is one that enters at the embedding. ``token_sources`` / ``token_slots``: rows whose token
-        is still on the device, in the slot the sampler left it in (kernels.embed)."""
-        if position_encoding is None or position_encoding.stage != "embedding":
-            raise NotImplementedError("only encodings added at the embedding have a kernel here")
-        return kernels.embed(tokens, positions, self.weight, position_encoding.weight, token_sources=token_sources, token_slots=token_slots)
+        is one that enters at the embedding (a table ``weight`` [positions, width]); an encoding
+        of stage "mixer", or none, leaves the token rows as they are. ``token_sources`` /
+        ``token_slots``: rows whose token is still on the device, in the slot the sampler left it
+        in (kernels.embed)."""
+        table = position_encoding.weight if position_encoding is not None and position_encoding.stage == "embedding" else None
+        return kernels.embed(tokens, positions, self.weight, table, token_sources=token_sources, token_slots=token_slots)
 
 
 class TiedHead(Part):

@@ -630,6 +630,13 @@ def test_split_blocks_follow_the_shape(K):
     assert big(1024, 4096, torch.bfloat16, 2048) == 1 and big(4096, 1024, torch.bfloat16, 512) == 1
 
 
+def test_embed_without_a_position_table(K):
+    rng = np.random.default_rng(6)
+    wte = rng.standard_normal((30, 72)).astype(np.float32)
+    out = K.embed(dev([3, -1, 29], torch.int32), dev([5, 0, 900], torch.int32), dev(wte), None)
+    np.testing.assert_array_equal(host(out), np.stack([wte[3], np.zeros(72, dtype=np.float32), wte[29]]))
+
+
 def test_embed_takes_tokens_from_slots(K):
     # rows whose source is not negative take their token from the slot the sampler left it in
     rng = np.random.default_rng(4)

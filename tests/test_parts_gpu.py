@@ -373,3 +373,164 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
     cache.open("c")
     again = host(runner.step([StepEntry("c", seqs["a"], [69])]))
     np.testing.assert_allclose(again[0], ref["a"][69], atol=5e-5, rtol=2e-4)
+
+
+# ------------------------------------------------------------------------------------------------
+# a second toy, defined here: positions that enter inside a mixer (no table at the embedding) and
+# a feed-forward that routes each row to one of two experts built from the framework's own parts
+# ------------------------------------------------------------------------------------------------
+def define_routed_toy():
+    from mini_llm_amd.config import ModelConfig, register_architecture
+    from mini_llm_amd.models import LayerCall, Model
+    from mini_llm_amd.ops import kernels
+    from mini_llm_amd.parts import FeedForward, Mixer, PositionEncoding, TiedHead, TokenEmbedding, make_part, register_part
+    from mini_llm_amd.weights import VECTOR, Normal, TensorSpec
+
+    class PhaseEncoding(PositionEncoding):
+        """x[t] * cos(position t * rate), applied by the mixer that holds it."""
+
+        stage = "mixer"
+
+        def __init__(self, n_positions, width):
+            self.n_positions, self.width = n_positions, width
+            self.rate = None
+
+        def tensor_specs(self):
+            return {"rate": TensorSpec((self.width,), VECTOR, Normal(0.05))}
+
+        def max_positions(self):
+            return self.n_positions
+
+        def apply(self, x, positions):
+            return x * torch.cos(positions[:, None].float() * self.rate)
+
+    class PhasedGate(Mixer):
+        def __init__(self, width, encoding):
+            self.width, self.encoding = width, encoding   # the encoding's tensor belongs to the model, not to this part
+            self.gain = None
+
+        def tensor_specs(self):
+            return {"gain": TensorSpec((self.width,), VECTOR, Normal(0.3, mean=1.0))}
+
+        def forward(self, x, residual, ctx):
+            positions = ctx.batch.positions[: x.shape[0]]
+            return kernels.add(residual, (self.encoding.apply(x.float(), positions) * self.gain).contiguous())
+
+    class TwoExperts(FeedForward):
+        graph_safe = False  # it plans on the host
+
+        def __init__(self, width, inner):
+            self.width = width
+            self.experts = [make_part("feed_forward", "dense_mlp", width=width, inner=inner, activation="gelu_new") for _ in range(2)]
+            self.router = None
+
+        def tensor_specs(self):
+            return {"router": TensorSpec((self.width,), VECTOR, Normal(1.0))}
+
+        def children(self):
+            return {f"experts.{e}.": expert for e, expert in enumerate(self.experts)}
+
+        def forward(self, x, residual):
+            chosen = (x.float() @ self.router) > 0   # router logits in 32-bit
+            out = torch.empty_like(residual)
+            for e, expert in enumerate(self.experts):
+                rows = torch.nonzero(chosen == bool(e)).flatten()
+                if rows.numel():
+                    out[rows] = kernels.settle(expert.forward(x[rows].contiguous(), residual[rows].contiguous()))
+            return out
+
+    register_part("position_encoding", "phase", PhaseEncoding)
+    register_part("mixer", "phased_gate", PhasedGate)
+    register_part("feed_forward", "two_experts", TwoExperts)
+
+    @dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        width: int
+        heads: int
+        inner: int
+        vocab: int
+        positions: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["architectures"][0], raw["width"], raw["heads"], raw["inner"], raw["vocab"], raw["positions"], raw["eps"])
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "width": self.width, "heads": self.heads, "inner": self.inner,
+                    "vocab": self.vocab, "positions": self.positions, "eps": self.eps}
+
+    def build(config, precision):
+        norm = lambda: make_part("norm", "layernorm", width=config.width, eps=config.eps)
+        encoding = make_part("position_encoding", "phase", n_positions=config.positions, width=config.width)
+        names = ("ln_1.", "mix.", "ln_2.", "mlp.")
+        blocks = [
+            make_part("block", "pre_norm", norm_1=norm(), mixer=make_part("mixer", "phased_gate", width=config.width, encoding=encoding),
+                      norm_2=norm(), feed_forward=make_part("feed_forward", "two_experts", width=config.width, inner=config.inner),
+                      compute_dtype=precision.compute, names=names),
+            make_part("block", "pre_norm", norm_1=norm(), mixer=make_part("mixer", "causal_attention", width=config.width, n_heads=config.heads),
+                      norm_2=norm(), feed_forward=make_part("feed_forward", "dense_mlp", width=config.width, inner=config.inner, activation="gelu"),
+                      compute_dtype=precision.compute, names=names),
+        ]
+        embedding = TokenEmbedding(config.vocab, config.width)
+        return Model(config, precision, embedding=embedding, position_encoding=encoding, blocks=blocks,
+                     schedule=[LayerCall(0, 0), LayerCall(1, 1)], final_norm=norm(), head=TiedHead(embedding),
+                     names={"embedding": "wte.", "position_encoding": "phase.", "block": "layers.{i}.", "final_norm": "norm."})
+
+    register_architecture("ToyRoutedLM", RoutedConfig, build)
+
+
+def plain_routed_toy(raw, w, tokens):
+    d, eps, H = raw["width"], raw["eps"], raw["heads"]
+    w = {k: v.astype(np.float64) for k, v in w.items()}
+    L = lambda i, n: w[f"layers.{i}.{n}"]
+    mlp = lambda x, prefix, act: P.linear(act(P.linear(x, w[prefix + "c_fc.weight"], w[prefix + "c_fc.bias"])), w[prefix + "c_proj.weight"], w[prefix + "c_proj.bias"])
+    h = w["wte.weight"][tokens]                                              # no position table
+    positions = np.arange(len(tokens))[:, None]
+    h = h + P.layernorm(h, L(0, "ln_1.weight"), L(0, "ln_1.bias"), eps) * np.cos(positions * w["phase.rate"]) * L(0, "mix.gain")
+    ln2 = P.layernorm(h, L(0, "ln_2.weight"), L(0, "ln_2.bias"), eps)
+    scores = ln2 @ L(0, "mlp.router")
+    assert np.abs(scores).min() > 1e-3, "a router score too close to the border for a comparison"
+    experts = [mlp(ln2, f"layers.0.mlp.experts.{e}.", P.gelu_new) for e in range(2)]
+    h = h + np.where((scores > 0)[:, None], experts[1], experts[0])
+    qkv = P.linear(P.layernorm(h, L(1, "ln_1.weight"), L(1, "ln_1.bias"), eps), L(1, "mix.c_attn.weight"), L(1, "mix.c_attn.bias"))
+    h = h + P.linear(P.multi_head_attention(qkv[:, :d], qkv[:, d : 2 * d], qkv[:, 2 * d :], H), L(1, "mix.c_proj.weight"), L(1, "mix.c_proj.bias"))
+    h = h + mlp(P.layernorm(h, L(1, "ln_2.weight"), L(1, "ln_2.bias"), eps), "layers.1.mlp.", P.ACTIVATIONS["gelu"])
+    return P.lm_head(P.layernorm(h, w["norm.weight"], w["norm.bias"], eps), w["wte.weight"])
+
+
+def test_toy_with_positions_inside_a_mixer_and_a_routed_feed_forward(tmp_path):
+    from mini_llm_amd.config import load_config
+    from mini_llm_amd.engine import ModelRunner, StepEntry
+    from mini_llm_amd.engine.loading import load_model, make_cache
+    from mini_llm_amd.weights import write_model_dir
+
+    define_routed_toy()
+    raw = {"architectures": ["ToyRoutedLM"], "width": 64, "heads": 2, "inner": 56, "vocab": 150, "positions": 80, "eps": 1e-5}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    config = load_config(tmp_path)
+    write_model_dir(config, 5, tmp_path)
+    weights = P.read_safetensors(tmp_path / "model.safetensors")
+    assert {"phase.rate", "layers.0.mix.gain", "layers.0.mlp.router", "layers.0.mlp.experts.1.c_proj.weight"} <= weights.keys()
+    assert not any(name.startswith("wpe") for name in weights)
+    model = load_model(tmp_path, "float32")
+    assert model.max_positions() == 80 and [g.layers for g in model.cache_groups()] == [(1,)]
+    cache = make_cache(model, max_tokens=256, page_size=16, max_requests=4)
+    runner = ModelRunner(model, cache, DEV)
+    assert not runner.use_graphs                          # the routed feed-forward plans on the host
+    seqs = {"a": random_tokens(3, 60, 150), "b": random_tokens(4, 25, 150)}
+    ref = {name: plain_routed_toy(raw, weights, t) for name, t in seqs.items()}
+    got, fed = {name: [] for name in seqs}, {name: 0 for name in seqs}
+    for name in seqs:
+        cache.open(name)
+    # portions of both kinds in one step, so that the rows are not laid out in the order given
+    for step in [[("a", 20), ("b", 3)], [("b", 1), ("a", 9)], [("a", 1), ("b", 1)], [("b", 20), ("a", 30)]]:
+        entries = [StepEntry(name, seqs[name][fed[name] : fed[name] + n], list(range(n))) for name, n in step]
+        logits = host(runner.step(entries))
+        at = 0
+        for name, n in step:
+            got[name].append(logits[at : at + n])
+            at += n
+            fed[name] += n
+    for name in seqs:
+        np.testing.assert_allclose(np.concatenate(got[name]), ref[name], atol=5e-5, rtol=2e-4, err_msg=name)
