@@ -424,10 +424,11 @@ LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kerne
 
 def layer_kernel_rows(width: int) -> int:
     """Rows up to which the layer kernels for decoding beat the separate kernels (measured on
-    MI355X: at GPT-2 small's width up to 32 rows, at GPT-2 medium's up to 16; beyond, every
-    (token, head) block reading its own copy of the partial rows and of the matrices costs more
-    than the launches and round trips the fusion saves)."""
-    return min(32 if width <= 768 else 16, LAYER_KERNEL_MAX_ROWS)
+    MI355X: at GPT-2 small's width up to 16 rows; at GPT-2 medium's the separate kernels, with
+    their products cut along K, win at every batch size: every (token, head) block reading its
+    own copy of the partial rows and of the matrices costs more than the launches and round trips
+    the fusion saves)."""
+    return min(16, LAYER_KERNEL_MAX_ROWS) if width <= 768 else 0
 
 
 def _pending(hidden):
