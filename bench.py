@@ -54,12 +54,12 @@ def prefill_flops(c, lengths, wanted_rows: int) -> float:
 
 
 class DecodeBench:
-    def __init__(self, engine, batch: int):
+    def __init__(self, engine, batch: int, prompt_len: int = PROMPT_LEN):
         import numpy as np
 
-        self.engine, self.batch = engine, batch
+        self.engine, self.batch, self.prompt_len = engine, batch, prompt_len
         rng = np.random.default_rng(SEED + 1)
-        self.prompts = [rng.integers(0, engine.config.vocab_size, PROMPT_LEN).tolist() for _ in range(batch)]
+        self.prompts = [rng.integers(0, engine.config.vocab_size, prompt_len).tolist() for _ in range(batch)]
         self.handles, self.last, self.length = [], [], 0
 
     def start(self):
@@ -71,10 +71,10 @@ class DecodeBench:
         self.handles = [self.engine.try_take_cache() for _ in range(self.batch)]
         self.last = []
         for i in range(0, self.batch, 4):
-            entries = [StepEntry(h, p, [PROMPT_LEN - 1]) for h, p in zip(self.handles[i : i + 4], self.prompts[i : i + 4])]
+            entries = [StepEntry(h, p, [self.prompt_len - 1]) for h, p in zip(self.handles[i : i + 4], self.prompts[i : i + 4])]
             logits = self.engine.runner.step(entries)
             self.last += self.engine.sampler.sample(logits, [SamplingParams()] * len(entries), [0] * len(entries)).cpu().tolist()
-        self.length = PROMPT_LEN
+        self.length = self.prompt_len
 
     def stop(self):
         for handle in self.handles:
@@ -144,6 +144,8 @@ def measure_prefill(engine, runs: int = 5):
 
 
 MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
+XL = dict(SMALL, n_layer=48, n_embd=1600, n_head=25, n_inner=6400)
+SHAPES = {"small": (SMALL, SEED), "medium": (MEDIUM, 6), "xl": (XL, 7)}  # the shapes and weight seeds the baseline names
 
 
 def measure_serving(dtype: str, temperature: float, step_ahead: bool = True):
@@ -233,6 +235,8 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--shape", default="small", choices=("small", "medium", "xl"), help="the GPT-2 shape that is run (the headline is small)")
+    parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of each sequence's prompt before decoding is timed")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
@@ -256,19 +260,22 @@ def main() -> int:
     from mini_llm_amd.config import config_from_dict
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
-    layers = args.layers or SMALL["n_layer"]
-    config = config_from_dict(dict(SMALL, n_layer=layers))
+    shape, seed = SHAPES[args.shape]
+    if not 1 <= args.prompt_len < CONTEXT:
+        parser.error(f"--prompt-len must be in 1..{CONTEXT - 1}")
+    layers = args.layers or shape["n_layer"]
+    config = config_from_dict(dict(shape, n_layer=layers))
     largest = max(args.batch, 1 if args.no_points else 64)
-    engine = Engine.from_random(config, SEED, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
+    engine = Engine.from_random(config, seed, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
 
     if args.prefill_only:
         print(json.dumps({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}))
         return 0
-    seconds, step_bytes = DecodeBench(engine, args.batch).run(args.steps, args.warmup)
+    seconds, step_bytes = DecodeBench(engine, args.batch, args.prompt_len).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
     achieved = step_bytes / (seconds / args.steps) / 1e9
     record = {
-        "metric": f"decode tokens/s at batch {args.batch}, GPT-2 small, 512-token prompts decoding towards 1024",
+        "metric": f"decode tokens/s at batch {args.batch}, GPT-2 {args.shape}, {args.prompt_len}-token prompts decoding towards 1024",
         "value": round(args.batch * args.steps / seconds, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -281,11 +288,11 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded random weights, uniform-random token ids",
         "config": {
-            "model": "gpt2-small", "n_layer": SMALL["n_layer"], "layers_run": layers, "n_embd": config.n_embd,
+            "model": f"gpt2-{args.shape}", "n_layer": shape["n_layer"], "layers_run": layers, "n_embd": config.n_embd,
             "n_head": config.n_head, "n_inner": config.n_inner, "vocab_size": config.vocab_size,
             "n_positions": config.n_positions, "activation_function": config.activation_function,
-            "global_batch": args.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT, "page_size": engine.cache.page_size,
-            "kv_cache_dtype": args.dtype, "sampling": "greedy", "parallelism": "single-gpu", "seed": SEED,
+            "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": CONTEXT, "page_size": engine.cache.page_size,
+            "kv_cache_dtype": args.dtype, "sampling": "greedy", "parallelism": "single-gpu", "seed": seed,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
     }
@@ -293,7 +300,7 @@ def main() -> int:
         record["prefill"] = measure_prefill(engine)
         points = {}
         for batch, steps in ((1, 128), (64, 64)):
-            s, _ = DecodeBench(engine, batch).run(steps, 8)
+            s, _ = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
             points[f"decode_b{batch}"] = round(batch * steps / s, 1)
         record["points"] = points
     print(json.dumps(record))

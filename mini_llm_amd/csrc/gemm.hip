@@ -500,8 +500,11 @@ void launch_gemm(const void* A, const void* W, bool packed, const float* bias, c
     // Few rows: the skinny kernel, except for a very wide matrix (the head over the vocabulary),
     // where a block of the skinny kernel would read the rows again for every 16 columns and the
     // tiled kernel with a short tile streams faster. The borders are measured on MI355X.
+    // A large bfloat16 matrix with more than 48 rows also goes to the tiled kernel (64 x 64 tile): its
+    // blocks read the rows once per 64 columns, not per 16 (4,800 x 1,600 at 64 rows: 14.0 against 16.7 us).
     const bool wide = N >= 8192;
-    const int skinny_rows = !wide ? 64 : (sizeof(T) == 2 ? 0 : 12);
+    const bool large = sizeof(T) == 2 && (long long)N * K >= 6000000;
+    const int skinny_rows = !wide ? (large ? 48 : 64) : (sizeof(T) == 2 ? 0 : 12);
     if (g_forced_tile == 0 && aligned && M <= skinny_rows) {
         if (M <= 16) launch_skinny<T, OutT, 1>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
         else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
@@ -583,7 +586,8 @@ MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, con
 #define MLLM_QKV_CASE(T)                                                                                              \
     if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
     else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
-    else if (M <= 64) launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
+    else if (M <= (sizeof(T) == 2 && (long long)N * K >= 6000000 ? 48 : 64))  /* a large matrix: as in mllm_gemm */                        \
+        launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);              \
     else launch_tiled<T, T, true>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
     if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
 #undef MLLM_QKV_CASE

@@ -126,6 +126,32 @@ def test_linear_f32(K, m, n, k, activation, packed):
     np.testing.assert_allclose(host(out), x.astype(np.float32).astype(np.float64) @ w.astype(np.float32).astype(np.float64).T, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("rows", [40, 49, 64])
+def test_few_rows_over_a_large_matrix(K, rows):
+    # more than 48 rows over a bfloat16 matrix of 6 M elements or more take the tiled kernel
+    # (64 x 64 tile) instead of the kernel for few rows: both sides of that border, plain and with
+    # the q/k/v epilogue that writes the cache
+    rng = np.random.default_rng(rows)
+    n, k = 2512, 2400
+    x, w, b = rng.standard_normal((rows, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
+    ref = bf16_round(x) @ bf16_round(w).T + b.astype(np.float32)
+    weight = as_weight(K, w, torch.bfloat16, True)
+    out = K.linear(dev(x, torch.bfloat16), weight, dev(b), out_dtype=torch.float32)
+    np.testing.assert_allclose(host(out), ref, rtol=2e-5, atol=2e-5)
+    n_heads, head_size, page_size = 13, 64, 64           # 3 x 832 = 2,496 columns
+    w = w[: 3 * n_heads * head_size]
+    kp = torch.full((3, n_heads, page_size, head_size), 7.0, device=DEV).to(torch.bfloat16)
+    vp = torch.full_like(kp, 7.0)
+    slots = rng.permutation(3 * page_size)[:rows].astype(np.int32)
+    q = K.linear_qkv_cache(dev(x, torch.bfloat16), as_weight(K, w, torch.bfloat16, True), dev(b[: len(w)]), kp, vp,
+                           dev(slots, torch.int32), n_heads, n_heads, head_size)
+    width = n_heads * head_size
+    np.testing.assert_allclose(host(q), ref[:, :width], rtol=2e-2, atol=2e-2)
+    for r, slot in enumerate(slots):
+        np.testing.assert_allclose(host(kp[slot // page_size, :, slot % page_size]).reshape(-1), ref[r, width : 2 * width], rtol=2e-2, atol=2e-2)
+        np.testing.assert_allclose(host(vp[slot // page_size, :, slot % page_size]).reshape(-1), ref[r, 2 * width : 3 * width], rtol=2e-2, atol=2e-2)
+
+
 def test_linear_f32_is_true_32_bit(K):
     # values that a reduced-precision matrix mode (tf32/bf16 inputs) would round away
     m, n, k = 8, 64, 64
