@@ -186,16 +186,20 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int page_shift, int window, float scale) {
+    int page_shift, int window, float scale, int out_packed) {
     constexpr int VEC = KeySweep<T, HD>::VEC, LPR = KeySweep<T, HD>::LPR, RPI = KeySweep<T, HD>::RPI;
     __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
 
     const int lane = threadIdx.x % WAVE, split = threadIdx.x / WAVE, n_splits = blockDim.x / WAVE;
     const int head = blockIdx.x, token = blockIdx.y;
     const int request = token_request[token];
-    T* out_row = out + (size_t)token * out_stride + head * HD;
+    // out_packed: the rows go out in the packed layout of a [tokens, n_heads * HD] matrix, for the
+    // output product of few rows that reads them next
+    auto out_at = [&](int d) -> T* {
+        return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
+    };
     if (request < 0) {  // a padding row; the whole block leaves together
-        for (int d = threadIdx.x; d < HD; d += blockDim.x) out_row[d] = from_float<T>(0.0f);
+        for (int d = threadIdx.x; d < HD; d += blockDim.x) *out_at(d) = from_float<T>(0.0f);
         return;
     }
     const int position = positions[token];
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     for (int d = threadIdx.x; d < HD; d += blockDim.x) {
         float value = 0.0f;
         for (int s = 0; s < n_splits; s++) value += partial[s][d] * expf(partial[s][HD] - total_max);
-        out_row[d] = from_float<T>(value * inverse);
+        *out_at(d) = from_float<T>(value * inverse);
     }
 }
 
@@ -251,13 +255,13 @@ template <typename T>
 int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                     void* out, int out_stride, const int* token_request, const int* positions,
                     const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
-                    int page_shift, int window, float scale, int n_splits, hipStream_t stream) {
+                    int page_shift, int window, float scale, int n_splits, int out_packed, hipStream_t stream) {
     dim3 grid(n_heads, n_tokens), block(WAVE * n_splits);
 #define MLLM_DECODE_CASE(HD)                                                                                   \
     case HD:                                                                                                   \
         attention_decode_kernel<T, HD><<<grid, block, 0, stream>>>(                                            \
             (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-            positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);              \
+            positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
@@ -283,7 +287,7 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    void* out, int out_stride, const int* token_request, const int* positions,
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
-                                   int n_splits, int dtype, hipStream_t stream) {
+                                   int n_splits, int dtype, int out_packed, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
@@ -299,10 +303,10 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
     int refused = 1;
     if (dtype == MLLM_F32)
         refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, stream);
+                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, stream);
     else
         refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, stream);
+                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, stream);
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }

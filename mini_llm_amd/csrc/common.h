@@ -47,6 +47,15 @@ __host__ __device__ __forceinline__ int packed_k_steps(int cols) {
     return (cols * (int)sizeof(T) + 63) / 64;
 }
 
+// Where element (row, col) of a [rows, cols] matrix lies in the packed layout. Rows of activations
+// are kept this way too when a product of few rows reads them next (its kernel loads whole chunks).
+template <typename T>
+__host__ __device__ __forceinline__ size_t packed_element(int row, int col, int cols) {
+    constexpr int VEC = 16 / (int)sizeof(T), KC = 4 * VEC;
+    const int in_chunk = col % KC;
+    return packed_offset<T>(row / 16, col / KC, packed_k_steps<T>(cols), (in_chunk / VEC) * 16 + row % 16) + in_chunk % VEC;
+}
+
 void mllm_set_error(const char* format, ...);
 int mllm_check_launch(const char* what);
 

@@ -813,7 +813,7 @@ template <typename OutT>
 __global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, const int* __restrict__ row_index,
                                                                 const float* __restrict__ gamma, const float* __restrict__ beta,
                                                                 OutT* __restrict__ out, float* __restrict__ summed, int width,
-                                                                float eps) {
+                                                                float eps, int packed_out) {
     extern __shared__ f32x4 row_pieces[];  // width / 4
     __shared__ float red[2][4];
     const int tid = threadIdx.x, n_pieces = width / 4;
@@ -841,7 +841,8 @@ __global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, c
     const float inverse_stddev = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / n + eps);
     for (int piece = tid; piece < n_pieces; piece += 256) {
         f32x4 y = (row_pieces[piece] - mean) * inverse_stddev * load4(gamma + 4 * piece) + load4(beta + 4 * piece);
-        OutT* at = out + (size_t)blockIdx.x * width + 4 * piece;
+        // four consecutive columns lie together in the packed layout too (inside one 16-byte piece)
+        OutT* at = out + (packed_out ? packed_element<OutT>(blockIdx.x, 4 * piece, width) : (size_t)blockIdx.x * width + 4 * piece);
         if constexpr (sizeof(OutT) == 2) store_bf16x4(at, y);
         else *reinterpret_cast<f32x4*>(at) = y;
     }
@@ -976,7 +977,8 @@ MLLM_API int mllm_pending_sum(const float* base, const float* partials, const fl
 // summed (or null): [n_rows, width], also gets each of those rows with its sums taken, not normalised.
 MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, const float* pending_bias, int n_partials,
                                     int pending_rows, const int* row_index, const float* gamma, const float* beta, void* out,
-                                    float* summed, int n_rows, int width, float eps, int out_dtype, hipStream_t stream) {
+                                    float* summed, int n_rows, int width, float eps, int out_dtype, int packed_out,
+                                    hipStream_t stream) {
     MLLM_REQUIRE(base != nullptr && out != nullptr, "pending_layernorm: no rows");
     MLLM_REQUIRE(n_partials >= 0 && (n_partials == 0 || partials != nullptr), "pending_layernorm: %d partial rows without memory", n_partials);
     MLLM_REQUIRE(width > 0 && width % 4 == 0 && width <= 32768, "pending_layernorm: width %d is not a multiple of 4 up to 32768", width);
@@ -985,9 +987,9 @@ MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, co
     PendingSum in{base, partials, pending_bias, n_partials, pending_rows};
     const size_t lds = (size_t)width * 4;
     if (out_dtype == MLLM_F32)
-        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, summed, width, eps);
+        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, summed, width, eps, packed_out);
     else if (out_dtype == MLLM_BF16)
-        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, summed, width, eps);
+        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, summed, width, eps, packed_out);
     else
         MLLM_REQUIRE(false, "pending_layernorm: unknown output dtype %d", out_dtype);
     return mllm_check_launch("pending_layernorm");

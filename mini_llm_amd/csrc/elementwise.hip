@@ -61,7 +61,7 @@ MLLM_API int mllm_embed(int* tokens, const int* positions, const int* sources, c
 template <typename OutT, int ROW_REGS>
 __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restrict__ row_index,
                                  const float* __restrict__ gamma, const float* __restrict__ beta,
-                                 OutT* __restrict__ out, int n_rows, int width, float eps) {
+                                 OutT* __restrict__ out, int n_rows, int width, float eps, int packed_out) {
     int lane = threadIdx.x % WAVE;
     int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
     if (row >= n_rows) return;
@@ -100,7 +100,7 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
         for (int r = 0; r < ROW_REGS; r++) {
             int i = lane + r * WAVE;
             if (i < width)
-                out_row[i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gains[r] + offsets[r]);
+                out[packed_out ? packed_element<OutT>(row, i, width) : (size_t)row * width + i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gains[r] + offsets[r]);
         }
     } else {
         float sum = 0.0f;
@@ -113,39 +113,41 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
         }
         float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) / n + eps);
         for (int i = lane; i < width; i += WAVE)
-            out_row[i] = from_float<OutT>((in_row[i] - mean) * inverse_stddev * gamma[i] + beta[i]);
+            out[packed_out ? packed_element<OutT>(row, i, width) : (size_t)row * width + i] = from_float<OutT>((in_row[i] - mean) * inverse_stddev * gamma[i] + beta[i]);
     }
 }
 
 template <typename OutT>
 static void launch_layernorm(const float* x, const int* row_index, const float* gamma,
                              const float* beta, void* out, int n_rows, int width, float eps,
-                             hipStream_t stream) {
+                             int packed_out, hipStream_t stream) {
     const int waves = 4;
     dim3 grid(ceil_div(n_rows, waves)), block(waves * WAVE);
     OutT* o = (OutT*)out;
     if (width <= 4 * WAVE)
-        layernorm_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+        layernorm_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
     else if (width <= 12 * WAVE)
-        layernorm_kernel<OutT, 12><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+        layernorm_kernel<OutT, 12><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
     else if (width <= 16 * WAVE)
-        layernorm_kernel<OutT, 16><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+        layernorm_kernel<OutT, 16><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
     else if (width <= 32 * WAVE)
-        layernorm_kernel<OutT, 32><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+        layernorm_kernel<OutT, 32><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
     else
-        layernorm_kernel<OutT, 0><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps);
+        layernorm_kernel<OutT, 0><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
 }
 
+// packed_out: out is in the packed layout of a [n_rows, width] matrix (room for whole chunks: rows up
+// to a multiple of 16, columns up to a multiple of 64 bytes; what lies beyond the rows is not written).
 MLLM_API int mllm_layernorm(const float* x, const int* row_index, const float* gamma,
                             const float* beta, void* out, int n_rows, int width, float eps,
-                            int out_dtype, hipStream_t stream) {
+                            int out_dtype, int packed_out, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && width > 0, "layernorm: bad sizes rows=%d width=%d", n_rows, width);
     MLLM_REQUIRE(eps > 0.0f, "layernorm: eps must be positive");
     if (n_rows == 0) return 0;
     if (out_dtype == MLLM_F32)
-        launch_layernorm<float>(x, row_index, gamma, beta, out, n_rows, width, eps, stream);
+        launch_layernorm<float>(x, row_index, gamma, beta, out, n_rows, width, eps, packed_out, stream);
     else if (out_dtype == MLLM_BF16)
-        launch_layernorm<bf16_t>(x, row_index, gamma, beta, out, n_rows, width, eps, stream);
+        launch_layernorm<bf16_t>(x, row_index, gamma, beta, out, n_rows, width, eps, packed_out, stream);
     else
         MLLM_REQUIRE(false, "layernorm: unknown output dtype %d", out_dtype);
     return mllm_check_launch("layernorm");

@@ -297,7 +297,7 @@ template <typename T, typename OutT, int MT, int KSPLIT, bool PACKED>
 __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     const T* __restrict__ A, const T* __restrict__ W, const float* __restrict__ bias,
     const float* __restrict__ residual, OutT* __restrict__ out, int M, int N, int K, int epilogue,
-    CacheScatter scatter, int steps_per_block) {
+    CacheScatter scatter, int steps_per_block, int x_packed, int out_packed) {
     constexpr int VEC = Tile<T>::VEC;
     constexpr int KSTEP = 4 * VEC;  // k covered by one load of the wave: 4 lane groups x 16 bytes
     // Loads in flight per wave before any is used. At decode sizes a wave's whole share of K fits
@@ -316,20 +316,29 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 #pragma unroll
     for (int i = 0; i < MT; i++) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const T* x_row[MT];
+    // Where this lane's piece of k-step s of row tile i lies: x_base[i] + min(s * x_stride + x_lane,
+    // x_limit), whether the rows of x are row-major or in the packed layout (x_packed: row tile i's
+    // chunk of a k-step is then the operand as it lies in memory; from row-major rows the same load
+    // touches 16 cache lines, and those loads are what a product of 48-64 rows spends most of its
+    // time on). Nothing inside the loop depends on which of the two it is.
+    const int n_steps = (K + KSTEP - 1) / KSTEP;
+    const int x_stride = x_packed ? 64 * VEC : KSTEP;
+    const int x_lane = x_packed ? lane * VEC : quad * VEC;
+    const int x_limit = x_packed ? ((n_steps - 1) * 64 + lane) * VEC : K - VEC;
+    const T* x_base[MT];
     bool x_valid[MT];
 #pragma unroll
     for (int i = 0; i < MT; i++) {
         int t = i * 16 + row16;
         x_valid[i] = t < M;
-        x_row[i] = A + (size_t)(x_valid[i] ? t : 0) * K;
+        // the packed matrix has (M + 15) / 16 row tiles, the kernel up to MT
+        x_base[i] = x_packed ? A + (size_t)min(i, (M - 1) / 16) * n_steps * (64 * VEC) : A + (size_t)(x_valid[i] ? t : 0) * K;
     }
 
     // The block takes the k-steps first_step .. last_step-1: all of them, or, when the launch has
     // several blocks per 16 columns (gridDim.y), its part of K, whose sums then go to matrix
     // blockIdx.y of `out` (partial products; the caller passes no bias, residual or epilogue).
     // Wave w takes the steps in groups of UNROLL, every KSPLIT-th group.
-    const int n_steps = (K + KSTEP - 1) / KSTEP;
     const int first_step = blockIdx.y * steps_per_block;
     const int last_step = min(n_steps, first_step + steps_per_block);
     out += (size_t)blockIdx.y * M * N;
@@ -344,7 +353,14 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
             else
                 w_piece[u] = *reinterpret_cast<const Vec16*>(w_row + safe_k);
 #pragma unroll
-            for (int i = 0; i < MT; i++) x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_row[i] + safe_k);
+            for (int i = 0; i < MT; i++) {
+                if constexpr (MT >= 4)  // measured: with four row tiles the two forms written out are faster (47 -> 54 k tokens/s at 64 rows in 32-bit), with one the common form (10.4 -> 11.9 k at 8 rows)
+                    x_piece[u][i] = *reinterpret_cast<const Vec16*>(
+                        x_packed ? A + packed_offset<T>(min(i, (M - 1) / 16), min(step0 + u, n_steps - 1), n_steps, lane)
+                                 : A + (size_t)(x_valid[i] ? i * 16 + row16 : 0) * K + safe_k);
+                else
+                    x_piece[u][i] = *reinterpret_cast<const Vec16*>(x_base[i] + min((step0 + u) * x_stride + x_lane, x_limit));
+            }
         }
         // what lies outside the matrices is zeroed only now, so that nothing above waits for a load
 #pragma unroll
@@ -406,13 +422,14 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         }
         size_t at = (size_t)token * N + col;
         if (residual) value = residual[at] + value;
-        out[at] = from_float<OutT>(value);
+        out[out_packed ? packed_element<OutT>(token, col, N) : at] = from_float<OutT>(value);
     }
 }
 
 template <typename T, typename OutT, int MT>
 void launch_skinny(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M,
-                   int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
+                   int N, int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1,
+                   int x_packed = 0, int out_packed = 0) {
     constexpr int KSTEP = 4 * Tile<T>::VEC;
     constexpr int UNROLL = MT == 1 ? 8 : 4;
     int tiles = ceil_div(N, 16), steps = ceil_div(K, KSTEP);
@@ -421,8 +438,8 @@ void launch_skinny(const T* a, const T* w, bool packed, const float* bias, const
     while (split < 16 && tiles * k_blocks * split < 2048 && steps_per_block >= 8 * split) split *= 2;
     dim3 grid(tiles, k_blocks);
 #define MLLM_SKINNY_CASE(SPLIT)                                                                                                   \
-    if (packed) gemm_skinny_kernel<T, OutT, MT, SPLIT, true><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block); \
-    else gemm_skinny_kernel<T, OutT, MT, SPLIT, false><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block);
+    if (packed) gemm_skinny_kernel<T, OutT, MT, SPLIT, true><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block, x_packed, out_packed); \
+    else gemm_skinny_kernel<T, OutT, MT, SPLIT, false><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block, x_packed, out_packed);
     if (split == 16) { MLLM_SKINNY_CASE(16) }
     else if (split == 1) { MLLM_SKINNY_CASE(1) }
     else if (split == 2) { MLLM_SKINNY_CASE(2) }
@@ -490,26 +507,29 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
     }
 }
 
+// Whether a product of M rows takes the kernel for few rows (which alone reads and writes rows in
+// the packed layout): up to 64 rows, except for a very wide matrix (the head over the vocabulary),
+// where a block of that kernel would read the rows again for every 16 columns and the tiled kernel
+// with a short tile streams faster. The borders are measured on MI355X.
+template <typename T>
+bool takes_few_row_kernel(int M, int N, int K) {
+    const bool aligned = K % Tile<T>::VEC == 0;
+    const bool wide = N >= 8192;
+    const int skinny_rows = !wide ? 64 : (sizeof(T) == 2 ? 0 : 12);
+    return g_forced_tile == 0 && aligned && M <= skinny_rows;
+}
+
 template <typename T, typename OutT>
 void launch_gemm(const void* A, const void* W, bool packed, const float* bias, const float* residual, void* out,
-                 int M, int N, int K, int epilogue, hipStream_t stream) {
+                 int M, int N, int K, int epilogue, int x_packed, int out_packed, hipStream_t stream) {
     const T* a = (const T*)A;
     const T* w = (const T*)W;
     OutT* o = (OutT*)out;
-    const bool aligned = K % Tile<T>::VEC == 0;
-    // Few rows: the skinny kernel, except for a very wide matrix (the head over the vocabulary),
-    // where a block of the skinny kernel would read the rows again for every 16 columns and the
-    // tiled kernel with a short tile streams faster. The borders are measured on MI355X.
-    // A large bfloat16 matrix with more than 48 rows also goes to the tiled kernel (64 x 64 tile): its
-    // blocks read the rows once per 64 columns, not per 16 (4,800 x 1,600 at 64 rows: 14.0 against 16.7 us).
-    const bool wide = N >= 8192;
-    const bool large = sizeof(T) == 2 && (long long)N * K >= 6000000;
-    const int skinny_rows = !wide ? (large ? 48 : 64) : (sizeof(T) == 2 ? 0 : 12);
-    if (g_forced_tile == 0 && aligned && M <= skinny_rows) {
-        if (M <= 16) launch_skinny<T, OutT, 1>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
-        else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
-        else launch_skinny<T, OutT, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
-    } else if (aligned) {
+    if (takes_few_row_kernel<T>(M, N, K)) {
+        if (M <= 16) launch_skinny<T, OutT, 1>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, CacheScatter{}, 1, x_packed, out_packed);
+        else if (M <= 32) launch_skinny<T, OutT, 2>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, CacheScatter{}, 1, x_packed, out_packed);
+        else launch_skinny<T, OutT, 4>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream, CacheScatter{}, 1, x_packed, out_packed);
+    } else if (K % Tile<T>::VEC == 0) {
         launch_tiled<T, OutT, true>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
     } else {
         launch_tiled<T, OutT, false>(a, w, packed, bias, residual, o, M, N, K, epilogue, stream);
@@ -521,19 +541,32 @@ void launch_gemm(const void* A, const void* W, bool packed, const float* bias, c
 // Tuning aid: forces one tile shape of the tiled kernel (1: 32x128, 2: 64x64, 3: 256x128, another number: 128x64; 0 gives the choice back to the sizes).
 MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
+// 1 if a product of M rows with an [N, K] matrix takes rows in the packed layout (x_packed, out_packed).
+MLLM_API int mllm_gemm_takes_packed_rows(int M, int N, int K, int in_dtype) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    if (in_dtype == MLLM_F32) return takes_few_row_kernel<float>(M, N, K) ? 1 : 0;
+    if (in_dtype == MLLM_BF16) return takes_few_row_kernel<bf16_t>(M, N, K) ? 1 : 0;
+    return 0;
+}
+
+// x_packed: A is in the packed layout of an [M, K] matrix; out_packed: out is written in the packed
+// layout of an [M, N] matrix (no residual then). Both only where mllm_gemm_takes_packed_rows says so.
 MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* bias, const float* residual,
                        void* out, int M, int N, int K, int in_dtype, int out_dtype, int epilogue,
-                       hipStream_t stream) {
+                       int x_packed, int out_packed, hipStream_t stream) {
     MLLM_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     MLLM_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
     MLLM_REQUIRE(ceil_div(M, 32) <= 65535, "gemm: M=%d has too many row tiles", M);
+    MLLM_REQUIRE((!x_packed && !out_packed) || mllm_gemm_takes_packed_rows(M, N, K, in_dtype),
+                 "gemm: rows in the packed layout are for the kernel for few rows, which M=%d N=%d K=%d do not take", M, N, K);
+    MLLM_REQUIRE(!out_packed || residual == nullptr, "gemm: a residual sum is not written in the packed layout");
     if (M == 0) return 0;
     if (in_dtype == MLLM_F32 && out_dtype == MLLM_F32)
-        launch_gemm<float, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<float, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, x_packed, out_packed, stream);
     else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_BF16)
-        launch_gemm<bf16_t, bf16_t>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<bf16_t, bf16_t>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, x_packed, out_packed, stream);
     else if (in_dtype == MLLM_BF16 && out_dtype == MLLM_F32)
-        launch_gemm<bf16_t, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, stream);
+        launch_gemm<bf16_t, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, x_packed, out_packed, stream);
     else
         MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
     return mllm_check_launch("gemm");
@@ -552,16 +585,17 @@ MLLM_API int mllm_gemm_split_blocks(int M, int N, int K, int in_dtype) {
 // 32-bit, whose sum (in any fixed order) is the product. For a long K with few output columns;
 // whoever takes the partial products adds bias and residual.
 MLLM_API int mllm_gemm_split(const void* A, const void* W, int w_packed, float* partials, int M, int N, int K,
-                             int in_dtype, int k_blocks, hipStream_t stream) {
+                             int in_dtype, int k_blocks, int x_packed, hipStream_t stream) {
+    MLLM_REQUIRE(!x_packed || M <= 64, "gemm_split: rows in the packed layout are for at most 64 rows, not %d", M);
     MLLM_REQUIRE(M >= 0 && N > 0 && K > 0 && ceil_div(M, 32) <= 65535, "gemm_split: bad sizes M=%d N=%d K=%d", M, N, K);
     MLLM_REQUIRE(k_blocks >= 1 && k_blocks <= 16, "gemm_split: %d partial products is not in 1..16", k_blocks);
     MLLM_REQUIRE(in_dtype == MLLM_F32 || in_dtype == MLLM_BF16, "gemm_split: unknown dtype %d", in_dtype);
     MLLM_REQUIRE(K % (in_dtype == MLLM_F32 ? 4 : 8) == 0, "gemm_split: K=%d is not a multiple of a 16-byte piece", K);
     if (M == 0) return 0;
 #define MLLM_SPLIT_CASE(T)                                                                                                     \
-    if (M <= 16) launch_skinny<T, float, 1>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);      \
-    else if (M <= 32) launch_skinny<T, float, 2>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks); \
-    else if (M <= 64) launch_skinny<T, float, 4>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks); \
+    if (M <= 16) launch_skinny<T, float, 1>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks, x_packed);      \
+    else if (M <= 32) launch_skinny<T, float, 2>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks, x_packed); \
+    else if (M <= 64) launch_skinny<T, float, 4>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks, x_packed); \
     else launch_tiled<T, float, true>((const T*)A, (const T*)W, w_packed != 0, nullptr, nullptr, partials, M, N, K, 0, stream, CacheScatter{}, k_blocks);
     if (in_dtype == MLLM_F32) { MLLM_SPLIT_CASE(float) } else { MLLM_SPLIT_CASE(bf16_t) }
 #undef MLLM_SPLIT_CASE
@@ -573,7 +607,7 @@ MLLM_API int mllm_gemm_split(const void* A, const void* W, int w_packed, float* 
 // (what the reference's decode block does with its fused matvec: engine/src/transformer_block.cu:223-242).
 MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, const float* bias, void* out_q, void* k_pages,
                                  void* v_pages, const int* slots, int M, int K, int q_width, int kv_width,
-                                 int n_kv_heads, int head_size, int page_size, int dtype, hipStream_t stream) {
+                                 int n_kv_heads, int head_size, int page_size, int dtype, int x_packed, hipStream_t stream) {
     MLLM_REQUIRE(M >= 0 && ceil_div(M, 32) <= 65535, "gemm_qkv_cache: bad row count %d", M);
     MLLM_REQUIRE(K > 0 && q_width > 0 && kv_width == n_kv_heads * head_size && head_size > 0, "gemm_qkv_cache: bad sizes");
     MLLM_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0, "gemm_qkv_cache: page size %d is no power of two", page_size);
@@ -583,12 +617,13 @@ MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, con
     CacheScatter scatter{k_pages, v_pages, slots, q_width, kv_width, n_kv_heads, head_size, 0, 1};
     while ((1 << scatter.page_shift) < page_size) scatter.page_shift++;
     int N = q_width + 2 * kv_width;
+    MLLM_REQUIRE(!x_packed || mllm_gemm_takes_packed_rows(M, N, K, dtype),
+                 "gemm_qkv_cache: rows in the packed layout are for the kernel for few rows, which M=%d N=%d K=%d do not take", M, N, K);
 #define MLLM_QKV_CASE(T)                                                                                              \
-    if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);      \
-    else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
-    else if (M <= (sizeof(T) == 2 && (long long)N * K >= 6000000 ? 48 : 64))  /* a large matrix: as in mllm_gemm */                        \
-        launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);              \
-    else launch_tiled<T, T, true>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter);
+    if (!takes_few_row_kernel<T>(M, N, K)) launch_tiled<T, T, true>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter); \
+    else if (M <= 16) launch_skinny<T, T, 1>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter, 1, x_packed);      \
+    else if (M <= 32) launch_skinny<T, T, 2>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter, 1, x_packed); \
+    else launch_skinny<T, T, 4>((const T*)A, (const T*)W, w_packed != 0, bias, nullptr, (T*)out_q, M, N, K, 0, stream, scatter, 1, x_packed);
     if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
 #undef MLLM_QKV_CASE
     return mllm_check_launch("gemm_qkv_cache");

@@ -88,15 +88,16 @@ def embed(tokens, positions, wte, wpe, out=None, token_sources=None, token_slots
     return out
 
 
-def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None, with_sums=False):
+def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=None, with_sums=False, packed_out=False):
     """Row LayerNorm of float32 rows, plain or pending (PendingRows: the sums are taken on the way
     in); ``row_index`` (int32) picks the input row of each output row. ``with_sums``: returns
-    (normalised rows, the rows with their sums taken) - what the residual stream goes on with."""
+    (normalised rows, the rows with their sums taken) - what the residual stream goes on with.
+    ``packed_out``: the normalised rows come as PackedRows, for a product of few rows."""
     if with_sums:
         _require(row_index is None, "the rows with their sums taken are not gathered")
         if not isinstance(x, PendingRows) or x.base.shape[1] % 4 or (x.partials is None and x.bias is None):
             x = settle(x)
-            return layernorm(x, gamma, beta, eps, out_dtype=out_dtype, out=out), x
+            return layernorm(x, gamma, beta, eps, out_dtype=out_dtype, out=out, packed_out=packed_out), x
     pending = isinstance(x, PendingRows)
     if pending and x.base.shape[1] % 4:
         x, pending = settle(x), False
@@ -113,19 +114,26 @@ def layernorm(x, gamma, beta, eps, out_dtype=torch.float32, row_index=None, out=
     if row_index is not None:
         _device_tensor(row_index, "row_index", torch.int32, 1)
         n = row_index.shape[0]
-    if out is None:
-        out = torch.empty((n, width), dtype=out_dtype, device=base.device)
-    _device_tensor(out, "out", out_dtype, 2)
-    _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+    if packed_out:
+        _require(out is None, "packed rows are allocated here")
+        result = empty_packed_rows(n, width, out_dtype, base.device)
+        out = result.data
+    else:
+        if out is None:
+            out = torch.empty((n, width), dtype=out_dtype, device=base.device)
+        _device_tensor(out, "out", out_dtype, 2)
+        _require(tuple(out.shape) == (n, width), "out has the wrong shape")
+        result = out
     if pending:
         summed = torch.empty_like(base) if with_sums else None
         check(library().mllm_pending_layernorm(_ptr(base), _ptr(partials), _ptr(bias), n_partials, base.shape[0], _ptr(row_index), _ptr(gamma),
-                                               _ptr(beta), _ptr(out), _ptr(summed), n, width, float(eps), _code(out_dtype), _stream()))
+                                               _ptr(beta), _ptr(out), _ptr(summed), n, width, float(eps), _code(out_dtype), int(packed_out), _stream()))
         if with_sums:
-            return out, summed
+            return result, summed
     else:
-        check(library().mllm_layernorm(_ptr(base), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype), _stream()))
-    return out
+        check(library().mllm_layernorm(_ptr(base), _ptr(row_index), _ptr(gamma), _ptr(beta), _ptr(out), n, width, float(eps), _code(out_dtype),
+                                       int(packed_out), _stream()))
+    return result
 
 
 def add(a, b, out=None):
@@ -162,6 +170,39 @@ class PackedMatrix:
         return self.data.device
 
 
+# Rows from which on activations are worth passing in the packed layout between the kernels of a
+# layer (measured on MI355X: from 17 rows the products of few rows gain up to a half; below, nothing
+# in bfloat16, and the 32-bit path loses 7 %).
+PACKED_ROWS_FROM = 17
+
+
+class PackedRows(PackedMatrix):
+    """Rows of activations [rows, cols] in the same packed layout, as a kernel left them for a
+    product of few rows to read (what lies beyond the rows and columns is not defined, and the
+    product does not use it)."""
+
+
+def empty_packed_rows(rows: int, cols: int, dtype, device) -> PackedRows:
+    per_piece = 16 // (4 if dtype == torch.float32 else 2)
+    chunks = -(-rows // 16) * -(-cols // (4 * per_piece))
+    return PackedRows(torch.empty(chunks * 64 * per_piece, dtype=dtype, device=device), rows, cols)
+
+
+def takes_packed_rows(rows: int, weight, dtype) -> bool:
+    """Whether ``linear`` / ``linear_qkv_cache`` of so many rows with this weight reads (and can
+    write) rows in the packed layout: where the product takes the kernel for few rows."""
+    _, _, n, k = _matrix(weight, "weight", dtype)
+    return bool(library().mllm_gemm_takes_packed_rows(int(rows), n, k, _code(dtype)))
+
+
+def _rows(x, name):
+    """(pointer, packed flag, rows, cols, dtype, device) of activations given plain or packed."""
+    if isinstance(x, PackedRows):
+        return _ptr(x.data), 1, x.rows, x.cols, x.data.dtype, x.data.device
+    _device_tensor(x, name, dim=2)
+    return _ptr(x), 0, x.shape[0], x.shape[1], x.dtype, x.device
+
+
 def pack_matrix(src, dtype=None, transpose=False) -> PackedMatrix:
     """A float32/bfloat16 matrix [out, in] (or, with ``transpose``, stored [in, out]) in the packed
     layout, in element type ``dtype`` (default: its own). Load-time work on weights."""
@@ -184,15 +225,15 @@ def _matrix(weight, name, dtype):
     return _ptr(weight), 0, weight.shape[0], weight.shape[1]
 
 
-def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None, out=None):
+def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None, out=None, packed_out=False):
     """act(x @ weight.T + bias) (+ residual). ``weight`` is [out, in], a row-major tensor or a
-    PackedMatrix; sums are float32.
+    PackedMatrix; sums are float32. x may be PackedRows, and with ``packed_out`` the result is,
+    where ``takes_packed_rows`` says so.
 
     x and weight share their element type (float32: true 32-bit MFMA; bfloat16: bf16 MFMA);
     bias and residual are float32; a residual makes the output float32."""
-    _device_tensor(x, "x", dim=2)
-    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
-    m, k = x.shape
+    x_ptr, x_packed, m, k, x_dtype, device = _rows(x, "x")
+    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x_dtype)
     if not (w_cols == k):
         raise OperandError(f"x has {k} columns but weight has {w_cols}")
     if not (activation in EPILOGUES):
@@ -201,18 +242,25 @@ def linear(x, weight, bias=None, activation=None, residual=None, out_dtype=None,
         _device_tensor(bias, "bias", torch.float32, 1)
         _require(bias.shape[0] == n, "bias does not match weight")
     if out_dtype is None:
-        out_dtype = torch.float32 if residual is not None else x.dtype
+        out_dtype = torch.float32 if residual is not None else x_dtype
     if residual is not None:
         _device_tensor(residual, "residual", torch.float32, 2)
         _require(tuple(residual.shape) == (m, n), "residual has the wrong shape")
         _require(out_dtype == torch.float32, "a residual sum is float32")
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _device_tensor(out, "out", out_dtype, 2)
-    _require(tuple(out.shape) == (m, n), "out has the wrong shape")
-    _require(x.dtype != torch.float32 or out_dtype == torch.float32, "float32 inputs give float32 outputs")
-    check(library().mllm_gemm(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x.dtype), _code(out_dtype), EPILOGUES[activation], _stream()))
-    return out
+    _require(x_dtype != torch.float32 or out_dtype == torch.float32, "float32 inputs give float32 outputs")
+    if packed_out:
+        _require(out is None and residual is None, "packed rows are allocated here, and hold no residual sum")
+        result = empty_packed_rows(m, n, out_dtype, device)
+        out = result.data
+    else:
+        if out is None:
+            out = torch.empty((m, n), dtype=out_dtype, device=device)
+        _device_tensor(out, "out", out_dtype, 2)
+        _require(tuple(out.shape) == (m, n), "out has the wrong shape")
+        result = out
+    check(library().mllm_gemm(x_ptr, w_ptr, w_packed, _ptr(bias), _ptr(residual), _ptr(out), m, n, k, _code(x_dtype), _code(out_dtype),
+                              EPILOGUES[activation], x_packed, int(packed_out), _stream()))
+    return result
 
 
 def split_blocks(weight, dtype, rows: int = 1) -> int:
@@ -227,14 +275,14 @@ def split_blocks(weight, dtype, rows: int = 1) -> int:
 def linear_split(x, weight, k_blocks: int):
     """x @ weight.T as ``k_blocks`` partial products over consecutive parts of K: float32
     [k_blocks, rows, out]; their sum is the product. The blocks of a product with few output
-    columns each read whole rows of x; cut along K they read a part, and many more run."""
-    _device_tensor(x, "x", dim=2)
-    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
-    m, k = x.shape
+    columns each read whole rows of x; cut along K they read a part, and many more run. x may be
+    PackedRows (up to 64 rows)."""
+    x_ptr, x_packed, m, k, x_dtype, device = _rows(x, "x")
+    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x_dtype)
     if not (w_cols == k):
         raise OperandError(f"x has {k} columns but weight has {w_cols}")
-    partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=x.device)
-    check(library().mllm_gemm_split(_ptr(x), w_ptr, w_packed, _ptr(partials), m, n, k, _code(x.dtype), int(k_blocks), _stream()))
+    partials = torch.empty((k_blocks, m, n), dtype=torch.float32, device=device)
+    check(library().mllm_gemm_split(x_ptr, w_ptr, w_packed, _ptr(partials), m, n, k, _code(x_dtype), int(k_blocks), x_packed, _stream()))
     return partials
 
 
@@ -280,22 +328,23 @@ def cache_write(k_src, v_src, k_pages, v_pages, slots, n_kv_heads, head_size):
 
 def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_heads, head_size):
     """The fused q/k/v projection: returns q [rows, n_heads*head_size] and writes the key and value
-    columns straight into the cache pages at slots[row] (negative: skip)."""
-    _device_tensor(x, "x", dim=2)
-    w_ptr, w_packed, w_rows, w_cols = _matrix(weight, "weight", x.dtype)
+    columns straight into the cache pages at slots[row] (negative: skip). x may be PackedRows where
+    ``takes_packed_rows`` says so."""
+    x_ptr, x_packed, m, k, x_dtype, device = _rows(x, "x")
+    w_ptr, w_packed, w_rows, w_cols = _matrix(weight, "weight", x_dtype)
     num_pages, page_size = _check_pages(k_pages, v_pages, n_kv_heads, head_size)
-    _require(k_pages.dtype == x.dtype, "pages and x differ in element type")
-    m, k = x.shape
+    _require(k_pages.dtype == x_dtype, "pages and x differ in element type")
     q_width, kv_width = n_heads * head_size, n_kv_heads * head_size
     _require((w_rows, w_cols) == (q_width + 2 * kv_width, k), "weight does not match the heads or x")
-    _require(k % (16 // x.element_size()) == 0, "the input width is not a multiple of a 16-byte piece")
+    _require(k % (16 // (4 if x_dtype == torch.float32 else 2)) == 0, "the input width is not a multiple of a 16-byte piece")
     if bias is not None:
         _device_tensor(bias, "bias", torch.float32, 1)
         _require(bias.shape[0] == w_rows, "bias does not match weight")
     _device_tensor(slots, "slots", torch.int32, 1)
     _require(slots.shape[0] >= m, "fewer slots than rows")
-    q = torch.empty((m, q_width), dtype=x.dtype, device=x.device)
-    check(library().mllm_gemm_qkv_cache(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(slots), m, k, q_width, kv_width, n_kv_heads, head_size, page_size, _code(x.dtype), _stream()))
+    q = torch.empty((m, q_width), dtype=x_dtype, device=device)
+    check(library().mllm_gemm_qkv_cache(x_ptr, w_ptr, w_packed, _ptr(bias), _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(slots), m, k, q_width,
+                                        kv_width, n_kv_heads, head_size, page_size, _code(x_dtype), x_packed, _stream()))
     return q
 
 
@@ -307,7 +356,7 @@ DECODE_MAX_SPLITS = 16      # waves per block
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
-                    short_rows=None, short_requests=None):
+                    short_rows=None, short_requests=None, packed_out=False):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
@@ -320,7 +369,9 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     ``short_requests``: the first so many rows are the portions of the first so many requests and
     none of them is longer than DECODE_MAX_Q_LEN, while the rest are longer portions; a batch of
     both kinds then runs as two launches, each kind in its own kernel (a single decoded token with
-    a long context would otherwise walk all its keys in one wave of the kernel for portions)."""
+    a long context would otherwise walk all its keys in one wave of the kernel for portions).
+    ``packed_out``: where the kernel for decoding and short portions runs, the rows come as
+    PackedRows (for the output product of few rows that reads them next); elsewhere as ever."""
     _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     page_size = k_pages.shape[2]
     width = n_heads * head_size
@@ -362,8 +413,14 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         n_splits = 1
         while n_splits < DECODE_MAX_SPLITS and 2 * n * n_heads * n_splits <= DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < reach:
             n_splits *= 2
-        check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), _stream()))
-        return out
+        result = out
+        if packed_out:
+            result = empty_packed_rows(n, width, q.dtype, q.device)
+            out = result.data
+        check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
+                                        _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
+                                        head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out), _stream()))
+        return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _device_tensor(q_starts, "q_starts", torch.int32, 1)

@@ -16,12 +16,13 @@ _library: ctypes.CDLL | None = None
 P = c_void_p
 _SIGNATURES = {
     "mllm_embed": [P, P, P, P, P, P, P, c_int, c_int, c_int, P],
-    "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, P],
+    "mllm_layernorm": [P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
     "mllm_add": [P, P, P, c_longlong, c_int, P],
-    "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_gemm_split": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_takes_packed_rows": [c_int, c_int, c_int, c_int],
+    "mllm_gemm_split": [P, P, c_int, P, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_gemm_split_blocks": [c_int, c_int, c_int, c_int],
-    "mllm_gemm_qkv_cache": [P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_gemm_qkv_cache": [P, P, c_int, P, P, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_convert": [P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pack_matrix": [P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_packed_elements": [c_int, c_int, c_int],
@@ -29,7 +30,7 @@ _SIGNATURES = {
     "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
-    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
@@ -39,7 +40,7 @@ _SIGNATURES = {
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_decode_mlp_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pending_sum": [P, P, P, c_int, P, c_int, c_int, P],
-    "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, P],
+    "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
 }
 
 

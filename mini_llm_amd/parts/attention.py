@@ -43,11 +43,15 @@ class CausalSelfAttention(Mixer):
     def kv_need(self):
         return KVNeed(self.n_kv_heads, self.head_size, self.window)
 
+    def _fused_qkv(self, ctx: LayerContext, dtype) -> bool:
+        """One kernel projects, keeps q and puts keys and values into their pages."""
+        page_size = ctx.k_pages.shape[2]
+        return bool(ctx.write_cache and self.width % (16 // (4 if dtype == torch.float32 else 2)) == 0 and page_size & (page_size - 1) == 0)
+
     def forward(self, x, residual, ctx: LayerContext):
-        fused = (ctx.write_cache and x.shape[1] % (16 // x.element_size()) == 0
-                 and ctx.k_pages.shape[2] & (ctx.k_pages.shape[2] - 1) == 0)
-        if fused:
-            # one kernel projects, keeps q and puts keys and values into their pages
+        """x: plain rows, or kernels.PackedRows where ``forward_normed`` asked the norm for them."""
+        rows = x.shape[0]
+        if self._fused_qkv(ctx, x.dtype):
             q = kernels.linear_qkv_cache(x, self.qkv.weight, self.qkv.bias, ctx.k_pages, ctx.v_pages, ctx.group.slots,
                                          self.n_heads, self.n_kv_heads, self.head_size)
         else:
@@ -62,6 +66,8 @@ class CausalSelfAttention(Mixer):
             self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
             max_q_len=ctx.batch.max_q_len, max_len=ctx.batch.max_total_len,
             q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens,
+            # few rows: the output product reads them faster in the packed layout
+            packed_out=kernels.PACKED_ROWS_FROM <= rows <= 64 and self.out.accepts_packed_rows(rows, q.dtype, pending=True),
             **({"short_rows": ctx.batch.short_rows, "short_requests": ctx.batch.short_requests}
                if ctx.batch.short_portion <= kernels.DECODE_MAX_Q_LEN else {}),
         )
@@ -77,7 +83,11 @@ class CausalSelfAttention(Mixer):
                 hidden, norm.weight, norm.bias, norm.eps, self.qkv.weight, self.qkv.bias, self.out.weight, self.out.bias,
                 ctx.k_pages, ctx.v_pages, ctx.group.slots, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
                 self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0, write_cache=ctx.write_cache)
-        return super().forward_normed(hidden, norm, compute_dtype, ctx)
+        # kernel by kernel; few rows go from the norm to the q/k/v product in the packed layout
+        rows = hidden.shape[0]
+        packed = kernels.PACKED_ROWS_FROM <= rows <= 64 and self._fused_qkv(ctx, compute_dtype) and self.qkv.accepts_packed_rows(rows, compute_dtype)
+        x, hidden = norm.forward_with_sums(hidden, compute_dtype, packed=packed)
+        return self.forward(x, hidden, ctx)
 
 
 register_part("mixer", "causal_attention", CausalSelfAttention)

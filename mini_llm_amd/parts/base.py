@@ -90,10 +90,11 @@ class Norm(Part):
         """x: [rows, width] float32 -> [rows or len(row_index), width] of out_dtype."""
         raise NotImplementedError
 
-    def forward_with_sums(self, hidden, out_dtype):
+    def forward_with_sums(self, hidden, out_dtype, packed=False):
         """hidden: float32 rows, or rows whose last sums are pending -> (the normalised rows, the
         rows with their sums taken: what the residual stream goes on with). A norm that can take
-        the sums on its way in overrides this."""
+        the sums on its way in overrides this. ``packed``: the caller would like the normalised
+        rows as kernels.PackedRows (it takes plain rows too: this default gives those)."""
         from ..ops import kernels
 
         hidden = kernels.settle(hidden)

@@ -37,9 +37,13 @@ class DenseMLP(FeedForward):
                 and self.up.weight.dtype == torch.bfloat16 and kernels.decode_layer_supported(self.width, inner=self.inner)):
             return kernels.decode_mlp_half(hidden, norm.weight, norm.bias, norm.eps, self.up.weight, self.up.bias,
                                            self.down.weight, self.down.bias, activation=self.activation)
-        # else kernel by kernel; the down product of few rows may come back with its sums pending
-        x, hidden = norm.forward_with_sums(hidden, compute_dtype)
-        return self.down.forward_pending(self.up.forward(x, activation=self.activation), hidden)
+        # else kernel by kernel; the down product of few rows may come back with its sums pending, and
+        # few rows go from kernel to kernel in the packed layout, which the products read faster
+        rows = hidden.shape[0]
+        few = kernels.PACKED_ROWS_FROM <= rows <= 64
+        x, hidden = norm.forward_with_sums(hidden, compute_dtype, packed=few and self.up.accepts_packed_rows(rows, compute_dtype))
+        packed_out = few and self.up.accepts_packed_rows(rows, compute_dtype) and self.down.accepts_packed_rows(rows, compute_dtype, pending=True)
+        return self.down.forward_pending(self.up.forward(x, activation=self.activation, packed_out=packed_out), hidden)
 
 
 register_part("feed_forward", "dense_mlp", DenseMLP)

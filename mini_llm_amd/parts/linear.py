@@ -17,6 +17,7 @@ class Linear(Part):
         self.weight = None
         self.bias = None
         self._split_blocks = {}
+        self._accepts_packed = {}
 
     def tensor_specs(self):
         shape = (self.in_features, self.out_features) if self.stored_in_out else (self.out_features, self.in_features)
@@ -25,8 +26,20 @@ class Linear(Part):
             specs["bias"] = TensorSpec((self.out_features,), VECTOR, Normal(self.bias_std))
         return specs
 
-    def forward(self, x, activation=None, residual=None, out_dtype=None):
-        return kernels.linear(x, self.weight, self.bias, activation=activation, residual=residual, out_dtype=out_dtype)
+    def forward(self, x, activation=None, residual=None, out_dtype=None, packed_out=False):
+        return kernels.linear(x, self.weight, self.bias, activation=activation, residual=residual, out_dtype=out_dtype, packed_out=packed_out)
+
+    def accepts_packed_rows(self, rows: int, dtype, pending: bool = False) -> bool:
+        """Whether ``forward`` (or, with ``pending``, ``forward_pending``) of so many rows reads them in
+        the packed layout (kernels.PackedRows): where the product takes the kernel for few rows."""
+        key = (rows, dtype, pending)
+        answer = self._accepts_packed.get(key)
+        if answer is None:
+            answer = kernels.takes_packed_rows(rows, self.weight, dtype)
+            if pending and rows <= 64 and kernels.split_blocks(self.weight, dtype, rows) > 1:
+                answer = True   # the partial products of few rows come from that kernel whatever the matrix
+            self._accepts_packed[key] = answer
+        return answer
 
     def forward_pending(self, x, residual):
         """residual + x W + b, as float32 rows or, where few rows meet few output columns and a long

@@ -90,6 +90,86 @@ def plain_packed(w, vec):
     return out.reshape(-1)
 
 
+def unpacked(packed_rows):
+    """The [rows, cols] matrix that a PackedMatrix / PackedRows holds (the inverse of plain_packed)."""
+    rows, cols = packed_rows.shape
+    vec = 16 // packed_rows.data.element_size()
+    kc = 4 * vec
+    row_tiles, k_steps = -(-rows // 16), -(-cols // kc)
+    flat = host(packed_rows.data.float()).reshape(row_tiles, k_steps, 64, vec)
+    out = np.zeros((row_tiles * 16, k_steps * kc))
+    for p in range(64):
+        out.reshape(row_tiles, 16, k_steps, kc)[:, p % 16, :, (p // 16) * vec : (p // 16 + 1) * vec] = flat[:, :, p, :]
+    return out[:rows, :cols]
+
+
+def packed_rows_of(K, x, dtype):
+    """Activations as a kernel would leave them in the packed layout (NaN where nothing is defined)."""
+    rows = K.empty_packed_rows(x.shape[0], x.shape[1], dtype, DEV)
+    rows.data.fill_(float("nan"))
+    vec = 16 // rows.data.element_size()
+    flat = plain_packed(np.asarray(x, dtype=np.float64), vec)
+    mask = plain_packed(np.ones_like(np.asarray(x, dtype=np.float64)), vec) > 0
+    values = torch.tensor(flat, dtype=torch.float64, device=DEV).to(dtype)
+    rows.data[torch.tensor(mask, device=DEV)] = values[torch.tensor(mask, device=DEV)]
+    return rows
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width,n_partials", [(1, 64, 0), (17, 200, 3), (64, 768, 2), (33, 100, 0)])
+def test_layernorm_leaves_packed_rows(K, dtype, rows, width, n_partials):
+    rng = np.random.default_rng(rows + width)
+    gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
+    hidden, total = _pending_rows(K, rng, rows, width, n_partials, n_partials > 0)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    out, summed = K.layernorm(hidden, dev(gamma), dev(beta), 2e-5, out_dtype=dtype, with_sums=True, packed_out=True)
+    assert isinstance(out, K.PackedRows) and out.shape == (rows, width)
+    np.testing.assert_allclose(unpacked(out), P.layernorm(total, gamma, beta, 2e-5), rtol=tol, atol=tol)
+    np.testing.assert_allclose(host(summed), total, rtol=1e-6, atol=1e-6)
+    out = K.layernorm(dev(total), dev(gamma), dev(beta), 2e-5, out_dtype=dtype, packed_out=True)
+    np.testing.assert_allclose(unpacked(out), P.layernorm(total, gamma, beta, 2e-5), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (48, 130, 1000)])
+def test_products_of_few_rows_read_and_write_packed_rows(K, dtype, m, n, k):
+    # x in the packed layout with NaN wherever nothing is defined (rows and columns beyond the
+    # matrix): the product must not use those; the output in the packed layout on request
+    rng = np.random.default_rng(m + n)
+    rounded = bf16_round if dtype == torch.bfloat16 else (lambda a: a.astype(np.float32).astype(np.float64))
+    x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
+    weight = as_weight(K, w, dtype, True)
+    assert K.takes_packed_rows(m, weight, dtype)
+    xp = packed_rows_of(K, rounded(x), dtype)
+    np.testing.assert_allclose(unpacked(xp), rounded(x), rtol=0, atol=0)
+    ref = rounded(x) @ rounded(w).T + b.astype(np.float32)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    out = K.linear(xp, weight, dev(b), out_dtype=torch.float32)
+    np.testing.assert_allclose(host(out), ref, rtol=2e-5, atol=2e-5)
+    out = K.linear(xp, weight, dev(b), activation="gelu_new", packed_out=True)
+    assert isinstance(out, K.PackedRows) and out.dtype == dtype
+    np.testing.assert_allclose(unpacked(out), P.gelu_new(ref), rtol=tol, atol=tol)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    out = K.linear(xp, weight, dev(b), residual=dev(res))
+    np.testing.assert_allclose(host(out), ref + res, rtol=2e-5, atol=2e-5)
+    partials = K.linear_split(xp, weight, 3)
+    np.testing.assert_allclose(host(partials).astype(np.float64).sum(axis=0), rounded(x) @ rounded(w).T, rtol=2e-5, atol=2e-5)
+
+
+def test_packed_rows_are_refused_where_the_kernel_for_few_rows_does_not_run(K):
+    from mini_llm_amd.ops.library import KernelLibraryError
+
+    w = torch.zeros((64, 64), device=DEV)
+    assert not K.takes_packed_rows(65, w, torch.float32) and K.takes_packed_rows(64, w, torch.float32)
+    assert not K.takes_packed_rows(8, torch.zeros((9000, 64), device=DEV, dtype=torch.bfloat16), torch.bfloat16)   # the wide head
+    with pytest.raises(KernelLibraryError, match="few rows"):
+        K.linear(K.empty_packed_rows(65, 64, torch.float32, DEV), w)
+    with pytest.raises(KernelLibraryError, match="few rows"):
+        K.linear(torch.zeros((65, 64), device=DEV), w, packed_out=True)
+    with pytest.raises(KernelLibraryError, match="64 rows"):
+        K.linear_split(K.empty_packed_rows(65, 64, torch.float32, DEV), w, 2)
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 1), (16, 32), (33, 65), (96, 288), (50, 777)])
 @pytest.mark.parametrize("src,dst", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32)])
 @pytest.mark.parametrize("transpose", [False, True])
@@ -128,9 +208,8 @@ def test_linear_f32(K, m, n, k, activation, packed):
 
 @pytest.mark.parametrize("rows", [40, 49, 64])
 def test_few_rows_over_a_large_matrix(K, rows):
-    # more than 48 rows over a bfloat16 matrix of 6 M elements or more take the tiled kernel
-    # (64 x 64 tile) instead of the kernel for few rows: both sides of that border, plain and with
-    # the q/k/v epilogue that writes the cache
+    # 40 to 64 rows over a matrix of 6 M elements (33-48 rows: three row tiles of x where the kernel
+    # holds four), plain and with the q/k/v epilogue that writes the cache
     rng = np.random.default_rng(rows)
     n, k = 2512, 2400
     x, w, b = rng.standard_normal((rows, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n)
@@ -268,6 +347,12 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     )
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
+    if path == "split_keys":  # the same rows in the packed layout, as the output product of few rows takes them
+        packed = K.paged_attention(
+            dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+            n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=1, packed_out=True)
+        assert isinstance(packed, K.PackedRows)
+        np.testing.assert_array_equal(unpacked(packed), host(out.float()))
 
 
 def test_paged_attention_strided_q(K):
@@ -399,6 +484,12 @@ def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_hea
             v_ref[slot // page_size, :, slot % page_size, :] = ref[r, qw + kvw :].reshape(n_kv_heads, head_size)
     np.testing.assert_allclose(host(kp), k_ref, rtol=tol, atol=tol)
     np.testing.assert_allclose(host(vp), v_ref, rtol=tol, atol=tol)
+    if rows <= 64 and packed:  # the same from rows in the packed layout
+        kp.fill_(7.0); vp.fill_(7.0)
+        q2 = K.linear_qkv_cache(packed_rows_of(K, xr, dtype), as_weight(K, w, dtype, packed), dev(b), kp, vp, dev(slots, torch.int32), n_heads, n_kv_heads, head_size)
+        assert torch.equal(q2, q)
+        np.testing.assert_allclose(host(kp), k_ref, rtol=tol, atol=tol)
+        np.testing.assert_allclose(host(vp), v_ref, rtol=tol, atol=tol)
 
 
 @pytest.mark.parametrize("path", ["general", "split_keys", "matrix_cores"])
