@@ -3,6 +3,7 @@ reference's own tests hold, special cases that reduce to a numpy routine, and in
 chosen so that a plausible mistake fails it."""
 
 import math
+import os
 
 import numpy as np
 import pytest
@@ -210,3 +211,43 @@ def test_safetensors_roundtrip(tmp_path):
     # round to nearest even, checked on hand-picked bit patterns
     x = np.array([0x3F808000, 0x3F818000, 0x3F808001], dtype=np.uint32).view(np.float32)
     assert P.f32_to_bf16_rne(x).tolist() == [0x3F80, 0x3F82, 0x3F81]
+
+
+REFERENCE_DUMPS = "/root/reference/engine/tests/reference_data"
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE_DUMPS), reason="the reference's dumped activations are not on this machine")
+def test_dumped_activations_of_the_real_model_follow_the_plain_formulas():
+    # The reference holds what every part of the real GPT-2 put out for the tokens 15496, 11, 995
+    # (scripts/dump_reference.py:76-140: the three gathered embedding rows, per block the outputs of
+    # ln_1, attention, ln_2, the feed-forward and the block, ln_f, all logits), but not the weights.
+    # What they fix without the weights: the embedding is the sum of the two rows; a block is
+    # x + attention + feed-forward; ln_1 reads the block's input, ln_2 the sum after attention, ln_f
+    # the last block (a norm's output is gain * normalised + offset per column, so over the three
+    # rows the points (normalised, output) of a column lie on one line, and only for the right
+    # input); the head is the token table again, without a bias; the next token is the argmax.
+    def dump(name, shape=(3, 768)):
+        return np.fromfile(f"{REFERENCE_DUMPS}/{name}.bin", dtype="<f4").reshape(shape).astype(np.float64)
+
+    def off_the_line(x, y):
+        normalised = P.layernorm(x, np.ones(x.shape[1]), np.zeros(x.shape[1]), 1e-5)
+        gain = (y[1] - y[0]) / (normalised[1] - normalised[0])
+        return np.abs(gain * (normalised[2] - normalised[0]) + y[0] - y[2]).max()
+
+    token_rows, position_rows = dump("wte"), dump("wpe")
+    x = P.embed([0, 1, 2], token_rows, position_rows)
+    for layer in range(12):
+        name = f"block_{layer:02d}"
+        attention, mlp, out = dump(name + "_attn"), dump(name + "_mlp"), dump(name)
+        np.testing.assert_allclose(x + attention + mlp, out, rtol=0, atol=5e-4)
+        assert off_the_line(x, dump(name + "_ln1")) < 1e-4
+        assert off_the_line(x + attention, dump(name + "_ln2")) < 1e-4
+        assert off_the_line(x, dump(name + "_ln2")) > 1.0  # the norm in the wrong place shows
+        x = out
+    final = dump("ln_f")
+    assert off_the_line(x, final) < 1e-3   # outputs up to 180 here
+    logits = dump("logits_full", (3, 50257))
+    np.testing.assert_allclose(P.lm_head(final, token_rows), logits[:, [15496, 11, 995]], rtol=0, atol=1e-4)
+    np.testing.assert_array_equal(dump("logits_last", (50257,)), logits[2])
+    with open(f"{REFERENCE_DUMPS}/expected_next_token.txt") as f:
+        assert int(logits[2].argmax()) == int(f.read()) == 13
