@@ -60,6 +60,17 @@ class StepBatch:
     request_ids: list = field(default_factory=list)
     host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
 
+    def rows_in_order_of(self, request_ids) -> list:
+        """The batch's rows, listed request by request in the given order of the requests (the
+        batch itself may lay the requests out in another order)."""
+        starts = self.host["q_starts"]
+        place = {request_id: i for i, request_id in enumerate(self.request_ids)}
+        rows = []
+        for request_id in request_ids:
+            i = place[request_id]
+            rows.extend(range(int(starts[i]), int(starts[i + 1])))
+        return rows
+
 
 class BatchStaging:
     """Pinned host buffers, used in turn, and the device buffer the batch is copied into. A

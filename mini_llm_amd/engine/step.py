@@ -98,9 +98,11 @@ class ModelRunner:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
 
-    def forward(self, batch, resolve: bool = True):
+    def forward(self, batch, resolve: bool = True, observer=None):
         """Tokens that come from last-token slots are fetched on the device, then the model runs."""
-        return self.model.forward(batch, self.cache, resolve_tokens=resolve)
+        if observer is None:
+            return self.model.forward(batch, self.cache, resolve_tokens=resolve)
+        return self.model.forward(batch, self.cache, resolve_tokens=resolve, observer=observer)
 
     def _graph_for(self, entries):
         if not self.use_graphs or len(entries) > GRAPH_BUCKETS[-1]:
@@ -112,11 +114,13 @@ class ModelRunner:
             self._graphs[capacity] = _DecodeGraph(self, capacity)
         return self._graphs[capacity]
 
-    def step(self, entries: list[StepEntry]):
+    def step(self, entries: list[StepEntry], observer=None):
         """Runs the entries as one batch. Returns float32 logits [wanted places, vocab] on the
         device (None if nothing is wanted), in the order of the entries and of each ``want``;
         they are valid until the next step. Raises StepError / OutOfPages before anything has
-        changed."""
+        changed. ``observer(name, rows)`` is shown the residual stream after the embedding and
+        after each layer, the rows in the order of the entries and of their tokens (such a step
+        is not replayed from a graph)."""
         self.validate(entries)
         reserved = []
         try:
@@ -128,13 +132,17 @@ class ModelRunner:
                 self.cache.rollback(request_id)
             raise
         try:
-            graph = self._graph_for(entries)
+            graph = self._graph_for(entries) if observer is None else None
             if graph is not None:
                 batch, logits = graph.run(entries)
                 self.graph_steps += 1
             else:
                 batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size)
-                logits = self.forward(batch, resolve=any(e.from_slot for e in entries))
+                in_given_order = None
+                if observer is not None:
+                    rows = batch.rows_in_order_of([e.request_id for e in entries])
+                    in_given_order = lambda name, hidden: observer(name, hidden[rows])
+                logits = self.forward(batch, resolve=any(e.from_slot for e in entries), observer=in_given_order)
         except Exception:
             for request_id in reserved:
                 self.cache.rollback(request_id)

@@ -101,18 +101,26 @@ class Model(Part):
                 out[call.cache] = need
         return out
 
-    def forward(self, batch, cache, resolve_tokens: bool = False):
+    def forward(self, batch, cache, resolve_tokens: bool = False, observer=None):
         """The whole step: embeds the batch's tokens, runs the schedule over the cache, and
         returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only. With
-        ``resolve_tokens`` the rows that name a last-token slot take their token from it."""
+        ``resolve_tokens`` the rows that name a last-token slot take their token from it.
+        ``observer(name, rows)``, if given, is shown the residual stream (float32 [tokens, width],
+        rows in the batch's order) after the embedding (name "embedding") and after each entry of
+        the schedule (its index): what the reference's block_outputs are for, finding the layer
+        where a difference starts (engine/include/gpt2_gpu.h:21-25). The step itself runs as without."""
         hidden = self.embedding.forward(batch.tokens, batch.positions, self.position_encoding,
                                         token_sources=batch.token_sources if resolve_tokens else None,
                                         token_slots=cache.last_token if resolve_tokens else None)
-        for call in self.schedule:
+        if observer is not None:
+            observer("embedding", kernels.settle(hidden))
+        for index, call in enumerate(self.schedule):
             block = self.blocks[call.block]
             if not block.takes_pending:
                 hidden = kernels.settle(hidden)
             hidden = block.forward(hidden, cache.layer_context(batch, call))
+            if observer is not None:
+                observer(index, kernels.settle(hidden))
         if batch.n_logit_rows == 0:
             return None
         if not self.final_norm.takes_pending:

@@ -130,9 +130,11 @@ def lm_head(x, wte):
 # --------------------------------------------------------------------------------------------
 # whole model
 # --------------------------------------------------------------------------------------------
-def forward(config: dict, weights: dict, tokens, dtype=np.float64, stored=_keep):
+def forward(config: dict, weights: dict, tokens, dtype=np.float64, stored=_keep, block_outputs=None):
     """Logits [len(tokens), vocab] of one whole sequence (engine/src/gpt2.c:198-262): embed,
-    n_layer blocks, ln_f on every row, tied head. ``stored``: see ``block``."""
+    n_layer blocks, ln_f on every row, tied head. ``stored``: see ``block``. ``block_outputs``: a
+    list that receives the embedding and then every block's output (as the reference can hand out
+    its blocks' outputs: engine/src/gpt2.c:234-237)."""
     w = {name: np.asarray(t, dtype=dtype) for name, t in weights.items()}
     n_layer = config["n_layer"]
     eps = config.get("layer_norm_epsilon", 1e-5)
@@ -140,10 +142,14 @@ def forward(config: dict, weights: dict, tokens, dtype=np.float64, stored=_keep)
     if len(tokens) > config["n_positions"]:
         raise ValueError("sequence longer than n_positions")
     h = embed(tokens, w["wte.weight"], w["wpe.weight"])
+    if block_outputs is not None:
+        block_outputs.append(h)
     for i in range(n_layer):
         prefix = f"h.{i}."
         layer = {k[len(prefix) :]: t for k, t in w.items() if k.startswith(prefix)}
         h = block(h, layer, config["n_head"], eps, activation, stored)
+        if block_outputs is not None:
+            block_outputs.append(h)
     h = stored(layernorm(h, w["ln_f.weight"], w["ln_f.bias"], eps))
     return lm_head(h, w["wte.weight"])
 

@@ -25,13 +25,15 @@ def tolerance(dtype: str) -> dict:
     return F32_TOL if dtype == "float32" else BF16_TOL
 
 
-def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, timeout=600):
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page_size=None, timeout=600, hidden_out=None):
     """Runs bin/trace_run over the steps; returns {step: array [wanted, vocab]}."""
     out_dir = Path(out_dir)
     cmd = [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
            "--out", str(out_dir), "--max-tokens", str(max_tokens)]
     if page_size:
         cmd += ["--page-size", str(page_size)]
+    if hidden_out:
+        cmd += ["--hidden-out", str(hidden_out)]
     text = "".join(json.dumps(s) + "\n" for s in steps)
     done = subprocess.run(cmd, input=text, capture_output=True, text=True, timeout=timeout)
     assert done.returncode == 0, f"trace_run failed ({done.returncode}):\n{done.stderr[-3000:]}"

@@ -65,6 +65,10 @@ def test_short_portions_are_laid_out_first_and_logit_rows_keep_the_given_order()
     slot = {name: cache.requests[name].state_slot for name in "abcde"}
     assert batch.logit_slots.tolist() == [slot["b"], slot["a"], slot["c"], slot["c"], slot["e"]]
     assert batch.state_slots.tolist() == [slot[n] for n in "acebd"]
+    # the rows of the batch, listed in the order of the entries as given
+    given = batch.rows_in_order_of([e.request_id for e in entries])
+    assert given == list(range(10, 30)) + [0] + list(range(30, 39)) + list(range(1, 9)) + [9]
+    assert np.asarray(batch.tokens)[given].tolist() == [t for e in entries for t in e.tokens]
     assert batch.token_sources.tolist() == [-1] * 9 + [slot["e"]] + [-1] * 29
     for i, name in enumerate("acebd"):
         pages = cache.block_table(name, 0)

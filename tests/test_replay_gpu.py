@@ -38,3 +38,36 @@ def test_replay_matches_plain(model_dirs, tmp_path, name, mode, dtype):
     got = collector.gather(outputs)
     ref = replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16"))
     replay.compare(got, ref, **replay.tolerance(dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_hands_out_the_stream_after_every_layer(model_dirs, tmp_path, dtype):
+    # --hidden-out: the residual stream after the embedding and after each layer, the rows in the
+    # order of the entries, in a mixed trace (whose batches are laid out in another order)
+    folder, config, weights = model_dirs["B"]
+    requests = requests_for("B", config)
+    collector = replay.mixed(requests)
+    replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector), hidden_out=tmp_path / "hidden")
+    bf16 = dtype == "bfloat16"
+    plain = {}
+    for name, tokens in requests.items():
+        plain[name] = []
+        plain_gpt2.forward(config, plain_gpt2.bf16_weights(weights) if bf16 else weights, tokens,
+                           stored=plain_gpt2.stored_as_bf16 if bf16 else plain_gpt2._keep, block_outputs=plain[name])
+    width, fed = config["n_embd"], {}
+    names = ["embedding"] + list(range(config["n_layer"]))
+    for step in collector.steps:
+        if not step["entries"]:
+            continue
+        n_rows = sum(len(e["tokens"]) for e in step["entries"])
+        for index, name in enumerate(names):
+            rows = np.fromfile(tmp_path / "hidden" / f"{step['step']}.{name}.f32", dtype="<f4").reshape(n_rows, width)
+            at = 0
+            for e in step["entries"]:
+                start, n = fed.get(e["id"], 0), len(e["tokens"])
+                want = plain[e["id"]][index][start : start + n]
+                tol = dict(atol=1e-5, rtol=1e-5) if not bf16 else dict(atol=3e-2, rtol=2e-2)
+                np.testing.assert_allclose(rows[at : at + n], want, err_msg=f"step {step['step']} after {name}, request {e['id']}", **tol)
+                at += n
+        for e in step["entries"]:
+            fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
