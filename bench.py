@@ -5,7 +5,8 @@
 A step is one decode step: every live sequence gets one new token (greedy, sampled on the
 device and fed back). Sequences start from 512-token uniform-random prompts and decode towards
 1,024 tokens; when they are full they are given back and prefilled again outside the timed
-region, so that exactly K steps are timed. Prints one JSON line. The reference's counterpart is
+region, so that exactly K steps are timed. Before anything is timed, decoding is compared with a
+whole-prompt step on 8 tokens (--no-check skips that). Prints one JSON line. The reference's counterpart is
 engine/bench/bench_batch.c (batched decode at a context) and engine/bench/bench.c."""
 
 from __future__ import annotations
@@ -143,6 +144,50 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
 
 
+def check_before_timing(engine, n_new: int = 8):
+    """The gate before anything is timed, as the reference's bench has one (engine/bench/bench.c:30-31,
+    92-113: its GPU against its CPU path on 8 tokens, scaled difference <= 1e-3 and the same next
+    token). Here two sequences are decoded greedily for 8 tokens the way the timed steps run (single
+    tokens over the cache, replayed from a graph), then each whole sequence runs again as one prompt
+    step, through the other kernels (tiled products, prompt attention): the logits at the decoded
+    places must agree. Returns the largest difference / largest logit."""
+    import numpy as np
+    import torch
+
+    from mini_llm_amd.engine import StepEntry
+
+    rng = np.random.default_rng(SEED + 3)
+    prompts = [rng.integers(0, engine.config.vocab_size, n).tolist() for n in (40, 70)]
+    handles = [engine.try_take_cache() for _ in prompts]
+    logits = engine.runner.step([StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)])
+    stepwise, sequences = [[] for _ in prompts], [list(p) for p in prompts]
+    for _ in range(n_new):
+        rows = logits.float().cpu().numpy()
+        for i, row in enumerate(rows):
+            stepwise[i].append(row)
+            sequences[i].append(int(row.argmax()))
+        logits = engine.runner.step([StepEntry(h, [seq[-1]], [0]) for h, seq in zip(handles, sequences)])
+    for h in handles:
+        engine.release_cache(h)
+    worst = 0.0
+    limit = 1e-3 if engine.options.dtype == "float32" else 5e-2   # bfloat16 rounds every stored activation to 3 digits
+    for i, (prompt, seq) in enumerate(zip(prompts, sequences)):
+        handle = engine.try_take_cache()
+        fed = seq[:-1]
+        whole = engine.runner.step([StepEntry(handle, fed, list(range(len(prompt) - 1, len(fed))))]).float().cpu().numpy()
+        engine.release_cache(handle)
+        for k, (a, b) in enumerate(zip(stepwise[i], whole)):
+            scaled = float(np.abs(a - b).max() / np.abs(b).max())
+            worst = max(worst, scaled)
+            top = np.sort(b)[-2:]
+            clear = (top[1] - top[0]) > 2 * limit * np.abs(b).max()   # a near tie may fall either way
+            if not scaled <= limit or (clear and int(a.argmax()) != int(b.argmax())):
+                raise SystemExit(f"bench.py: decoding and the whole-prompt step disagree at sequence {i}, new token {k}: "
+                                 f"scaled difference {scaled:.3e} (allowed {limit:g}), next token {int(a.argmax())} vs {int(b.argmax())}; nothing was timed")
+    torch.cuda.synchronize()
+    return worst
+
+
 MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
 XL = dict(SMALL, n_layer=48, n_embd=1600, n_head=25, n_inner=6400)
 SHAPES = {"small": (SMALL, SEED), "medium": (MEDIUM, 6), "xl": (XL, 7)}  # the shapes and weight seeds the baseline names
@@ -238,6 +283,7 @@ def main() -> int:
     parser.add_argument("--shape", default="small", choices=("small", "medium", "xl"), help="the GPT-2 shape that is run (the headline is small)")
     parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of each sequence's prompt before decoding is timed")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
+    parser.add_argument("--no-check", action="store_true", help="skip the comparison of decoding with a whole-prompt step before timing")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
@@ -268,6 +314,7 @@ def main() -> int:
     largest = max(args.batch, 1 if args.no_points else 64)
     engine = Engine.from_random(config, seed, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
 
+    checked = None if args.no_check else check_before_timing(engine)
     if args.prefill_only:
         print(json.dumps({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}))
         return 0
@@ -294,6 +341,7 @@ def main() -> int:
             "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": CONTEXT, "page_size": engine.cache.page_size,
             "kv_cache_dtype": args.dtype, "sampling": "greedy", "parallelism": "single-gpu", "seed": seed,
         },
+        "check": None if checked is None else {"decode_vs_whole_prompt_scaled_diff": float(f"{checked:.3g}"), "tokens": 8},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
     }
     if not args.no_points:
