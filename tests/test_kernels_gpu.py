@@ -257,19 +257,47 @@ def test_linear_bf16(K, m, n, k, out_dtype, packed):
         np.testing.assert_allclose(host(out), y + res, rtol=2e-5, atol=2e-5)
 
 
-def test_linear_reads_nothing_past_its_operands(K):
-    # NaN guards right after every operand: an out-of-bounds read would poison the result
-    m, n, k = 5, 37, 20
-    rng = np.random.default_rng(3)
-    xg = torch.full((m * k + 64,), float("nan"), device=DEV)
-    wg = torch.full((n * k + 64,), float("nan"), device=DEV)
-    x, w = rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((n, k)).astype(np.float32)
-    xg[: m * k] = dev(x).flatten()
-    wg[: n * k] = dev(w).flatten()
-    og = torch.full((m * n + 64,), 123.0, device=DEV)
-    K.linear(xg[: m * k].view(m, k), wg[: n * k].view(n, k), out=og[: m * n].view(m, n))
-    np.testing.assert_allclose(host(og[: m * n].view(m, n)), x.astype(np.float64) @ w.T, rtol=1e-5, atol=1e-5)
-    assert (og[m * n :] == 123.0).all()  # and nothing written past the output
+def guarded(values, dtype, fill=float("nan")):
+    """The values on the device with 64 elements of ``fill`` right behind them (the pattern of the
+    reference's kernel tests: engine/tests/test_matvec_batch.cu:21-22): (view of the values, the guard)."""
+    values = np.ascontiguousarray(values)
+    whole = torch.full((values.size + 64,), fill, device=DEV, dtype=dtype)
+    whole[: values.size] = dev(values, dtype).flatten()
+    return whole[: values.size].view(*values.shape), whole[values.size :]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(5, 37, 20), (1, 16, 8), (16, 130, 72), (40, 50, 200), (64, 100, 64), (70, 37, 24), (130, 200, 96),
+                                   (300, 260, 136), (33, 40, 21), (200, 70, 50), (3, 9000, 64)])
+def test_linear_reads_nothing_past_its_operands(K, dtype, m, n, k):
+    # NaN guards right after every operand: an out-of-bounds read would poison the result; a known
+    # value right after the output: nothing is written past it. Every kernel of the product: few
+    # rows, the tiles, an unaligned K, the wide head.
+    rng = np.random.default_rng(m + n + k)
+    rounded = bf16_round if dtype == torch.bfloat16 else (lambda a: a.astype(np.float32).astype(np.float64))
+    x, w, b = rng.standard_normal((m, k)), rng.standard_normal((n, k)) / math.sqrt(k), rng.standard_normal(n).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    xg, _ = guarded(x, dtype)
+    wg, _ = guarded(w, dtype)
+    bg, _ = guarded(b, torch.float32)
+    rg, _ = guarded(res, torch.float32)
+    og, after = guarded(np.zeros((m, n)), torch.float32, fill=123.0)
+    K.linear(xg, wg, bg, residual=rg, out=og)
+    np.testing.assert_allclose(host(og), rounded(x) @ rounded(w).T + b + res, rtol=2e-5, atol=2e-5)
+    assert (after == 123.0).all()
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 64), (7, 100), (5, 768), (3, 1100), (2, 2500)])
+def test_layernorm_reads_nothing_past_its_operands(K, out_dtype, rows, width):
+    rng = np.random.default_rng(rows + width)
+    x, gamma, beta = rng.standard_normal((rows, width)).astype(np.float32), rng.standard_normal(width).astype(np.float32), rng.standard_normal(width).astype(np.float32)
+    xg, _ = guarded(x, torch.float32)
+    gg, _ = guarded(gamma, torch.float32)
+    bg, _ = guarded(beta, torch.float32)
+    out = K.layernorm(xg, gg, bg, 1e-5, out_dtype=out_dtype)
+    tol = 1e-5 if out_dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(out), P.layernorm(x.astype(np.float64), gamma, beta, 1e-5), rtol=tol, atol=tol)
 
 
 def plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window):
