@@ -67,7 +67,6 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     if (row >= n_rows) return;
     int source = row_index ? row_index[row] : row;
     const float* in_row = x + (size_t)source * width;
-    OutT* out_row = out + (size_t)row * width;
     const float n = (float)width;  // divided by, not multiplied with its inverse: a constant row has mean exactly itself
 
     if constexpr (ROW_REGS > 0) {

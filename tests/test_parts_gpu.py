@@ -3,7 +3,6 @@ whole architecture defined in a test (a toy mixer with state of its own, another
 layers) can be registered, built and stepped without a change to the framework's files."""
 
 import json
-import math
 from dataclasses import dataclass
 
 import numpy as np
@@ -92,10 +91,8 @@ def test_dense_mlp_part(activation, dtype):
 def test_dense_mlp_with_a_long_inner_side(dtype, rows):
     # few output columns, a long inner side: the down product comes back cut along K, its sums
     # pending, and the next norm takes them
-    from mini_llm_amd.engine.batch import StepBatch
     from mini_llm_amd.ops import kernels
     from mini_llm_amd.parts import make_part
-    from mini_llm_amd.parts.base import LayerContext
 
     width, inner, eps = 48, 1024, 1e-5
     part = make_part("feed_forward", "dense_mlp", width=width, inner=inner, activation="gelu_new")

@@ -11,7 +11,7 @@ import plain_gpt2
 from conftest import TINY_A, TINY_B, make_plain_model_dir
 from mini_llm_amd.config import config_from_dict, get_architecture
 from mini_llm_amd.precision import Precision
-from mini_llm_amd.weights import SafetensorsFile, WeightsError, load_weights, random_tensors, write_model_dir, write_safetensors
+from mini_llm_amd.weights import SafetensorsFile, WeightsError, load_weights, write_model_dir, write_safetensors
 
 
 def build(config_dict, dtype="float32"):
