@@ -23,6 +23,15 @@ class StepEntry:
     # The (single) token is the one the sampler left in the request's last-token slot on the
     # device in an earlier step; ``tokens`` then holds a placeholder the host never looks at.
     from_slot: bool = False
+    # the tokens as an int32 array, left here by whoever has converted them already (the step
+    # function, when it checks a long portion), so that the batch is not built from the list again
+    checked_tokens: object = field(default=None, repr=False, compare=False)
+
+    def token_array(self) -> np.ndarray:
+        array = self.checked_tokens
+        if array is None or len(array) != len(self.tokens):
+            array = np.asarray(self.tokens, dtype=np.int32)
+        return array
 
 
 @dataclass
@@ -153,7 +162,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     if n_tokens > cap_tokens or n_requests > cap_requests:
         raise ValueError("the batch exceeds the capacity it is laid out for")
 
-    tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    tokens = np.concatenate([e.token_array() for e in entries])
     positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(contexts, q_lens)])
     token_request = np.repeat(np.arange(n_requests, dtype=np.int32), q_lens)
     q_starts = np.full(cap_requests + 1, n_tokens, dtype=np.int32)

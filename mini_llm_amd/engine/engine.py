@@ -50,7 +50,13 @@ class _Executor:
         limit, vocab = self.max_positions(), self._engine.model.vocab_size
         if limit is not None and len(tokens) > limit:
             raise ValueError(f"the prompt has {len(tokens)} tokens; the model holds {limit}")
-        for token in tokens:
+        try:
+            array = np.asarray(tokens)
+            if array.ndim == 1 and array.dtype.kind in "iu" and (array.size == 0 or (0 <= int(array.min()) and int(array.max()) < vocab)):
+                return
+        except (ValueError, TypeError, OverflowError):
+            pass
+        for token in tokens:   # something is wrong: token by token, to name it
             if not 0 <= int(token) < vocab:
                 raise ValueError(f"token {token} is outside the vocabulary [0, {vocab})")
 

@@ -14,6 +14,8 @@ buffer per bucket that is overwritten before each replay."""
 
 from __future__ import annotations
 
+import numpy as np
+
 from ..cache import CacheManager, OutOfPages
 from .batch import BatchStaging, DecodeBatchBuilder, StepBatch, StepEntry, build_step_batch
 
@@ -70,6 +72,26 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs and device is not None and cache.max_length is not None and model.all_graph_safe())
         self._graphs: dict = {}
 
+    @staticmethod
+    def _check_tokens(entry, vocab: int) -> None:
+        """Every token an integer inside the vocabulary: a long portion is looked at as one array, and
+        token by token only to name the one that is wrong."""
+        tokens = entry.tokens
+        entry.checked_tokens = None   # whatever an earlier step left: the list may have changed since
+        if len(tokens) > 16:
+            try:
+                array = np.asarray(tokens)
+            except (ValueError, TypeError, OverflowError):
+                array = None
+            if array is not None and array.ndim == 1 and array.dtype.kind in "iu" and 0 <= int(array.min()) and int(array.max()) < vocab:
+                entry.checked_tokens = array.astype(np.int32, copy=False)
+                return
+        for token in tokens:
+            if not isinstance(token, (int,)) and not hasattr(token, "__index__"):
+                raise StepError(f"request {entry.request_id!r}: token {token!r} is not an integer")
+            if not 0 <= int(token) < vocab:
+                raise StepError(f"request {entry.request_id!r}: token {token} is outside the vocabulary [0, {vocab})")
+
     def validate(self, entries) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
@@ -86,11 +108,8 @@ class ModelRunner:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
             if entry.from_slot and n != 1:
                 raise StepError(f"request {entry.request_id!r}: only a single token can come from the last-token slot")
-            for token in ([] if entry.from_slot else entry.tokens):
-                if not isinstance(token, (int,)) and not hasattr(token, "__index__"):
-                    raise StepError(f"request {entry.request_id!r}: token {token!r} is not an integer")
-                if not 0 <= int(token) < vocab:
-                    raise StepError(f"request {entry.request_id!r}: token {token} is outside the vocabulary [0, {vocab})")
+            if not entry.from_slot:
+                self._check_tokens(entry, vocab)
             length = self.cache.length(entry.request_id)
             if limit is not None and length + n > limit:
                 raise StepError(f"request {entry.request_id!r}: {length} + {n} tokens exceed the model's {limit} positions")
