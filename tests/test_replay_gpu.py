@@ -71,3 +71,58 @@ def test_replay_hands_out_the_stream_after_every_layer(model_dirs, tmp_path, dty
                 at += n
         for e in step["entries"]:
             fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
+
+
+@pytest.fixture(scope="module")
+def small_shape_dir(tmp_path_factory):
+    """Two layers at GPT-2 small's own sizes (width 768, 12 heads of 64, inner 3072, the odd
+    vocabulary of 50,257): the sizes the kernels are tuned for, which the tiny models never reach."""
+    import json
+
+    from conftest import sharpen_attention
+
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 768, "n_head": 12,
+              "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    folder = tmp_path_factory.mktemp("small_shape")
+    weights = plain_gpt2.random_weights(config, 5)
+    sharpen_attention(weights, config, factor=3.0)
+    (folder / "config.json").write_text(json.dumps(config))
+    plain_gpt2.write_safetensors(folder / "model.safetensors", {"transformer." + k: v for k, v in weights.items()})
+    return folder, config, weights
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype):
+    # mixed: portions beside decoded tokens of up to four requests, then the last tokens one by one
+    # (at these sizes the bfloat16 decode steps take the layer kernels, the portions the tiled
+    # products and the prompt attention; the head runs over the whole odd vocabulary)
+    folder, config, weights = small_shape_dir
+    requests = {f"s{i}": random_tokens(200 + i, n, config["vocab_size"]) for i, n in enumerate((40, 70, 130, 23, 65))}
+    collector = replay.mixed(requests, seed=1)
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector))
+    ref = replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16"))
+    replay.compare(collector.gather(outputs), ref, **replay.tolerance(dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype):
+    # two long prompts in one step (the tiled products at hundreds of rows, the prompt attention over
+    # several tiles of keys), logits wanted at a few places; then some tokens one by one
+    folder, config, weights = small_shape_dir
+    requests = {"p": random_tokens(300, 612, config["vocab_size"]), "q": random_tokens(301, 391, config["vocab_size"])}
+    collector = replay.Collector()
+    head = {name: len(tokens) - 6 for name, tokens in requests.items()}
+    collector.add([(name, tokens[: head[name]], sorted({0, 1, 63, 64, 127, 128, 300, head[name] - 1})) for name, tokens in requests.items()])
+    for i in range(6):
+        collector.add([(name, tokens[head[name] + i : head[name] + i + 1], [0]) for name, tokens in requests.items()],
+                      end=list(requests) if i == 5 else [])
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector))
+    got = collector.gather(outputs)
+    ref = replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16"))
+    tol = replay.tolerance(dtype)
+    for name, rows in got.items():
+        assert len(rows) == 8 + 6
+        for position, row in rows.items():
+            want = ref[name][position]
+            err = np.abs(row - want)
+            assert (err <= tol["atol"] + tol["rtol"] * np.abs(want)).all(), f"request {name} position {position}: max error {err.max():.3e}"
