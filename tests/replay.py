@@ -180,3 +180,27 @@ def compare(got, ref, atol, rtol):
                 f"request {name!r} position {position}: {int(bad.sum())} logits differ, max error {err.max():.3e} "
                 f"(allowed {atol:g} + {rtol:g}*|ref|); first wrong position of this request"
             )
+
+
+def compare_within_rounding_noise(got, ref_rounded, ref_exact, max_share=1.0, rms_share=0.6):
+    """For bfloat16 at widths where a fixed bound no longer fits (rounding noise grows with the
+    width and the depth): the engine may differ from the plain implementation that stores the same
+    tensors in bfloat16 by less than that implementation itself differs from exact arithmetic. Per
+    request: at every position the largest difference stays under ``max_share`` of the largest
+    difference between the rounded and the exact plain logits of that request, and the root mean
+    square under ``rms_share`` of theirs. Measured at width 1,600: 0.3 to 0.4 of either (most
+    roundings fall the same way in both); a wrong key, row or page gives differences of the size
+    of the logits, tens of times the noise."""
+    for name, rows in got.items():
+        exact, rounded = ref_exact[name], ref_rounded[name]
+        noise = np.abs(rounded - exact)
+        noise_max, noise_rms = noise.max(), np.sqrt((noise**2).mean())
+        squares, count = 0.0, 0
+        for position, row in sorted(rows.items()):
+            err = np.abs(row.astype(np.float64) - rounded[position])
+            assert err.max() <= max_share * noise_max, (
+                f"request {name!r} position {position}: max error {err.max():.3e}, the rounding noise of this request is {noise_max:.3e}")
+            squares += float((err**2).sum())
+            count += err.size
+        rms = np.sqrt(squares / count)
+        assert rms <= rms_share * noise_rms, f"request {name!r}: rms error {rms:.3e}, the rounding noise has {noise_rms:.3e}"

@@ -73,22 +73,41 @@ def test_replay_hands_out_the_stream_after_every_layer(model_dirs, tmp_path, dty
             fed[e["id"]] = fed.get(e["id"], 0) + len(e["tokens"])
 
 
+REAL_SHAPES = {  # two layers at the sizes of the GPT-2 shapes the benchmarks run
+    "small": dict(n_embd=768, n_head=12, n_inner=3072),
+    "xl": dict(n_embd=1600, n_head=25, n_inner=6400),
+}
+
+
 @pytest.fixture(scope="module")
-def small_shape_dir(tmp_path_factory):
-    """Two layers at GPT-2 small's own sizes (width 768, 12 heads of 64, inner 3072, the odd
-    vocabulary of 50,257): the sizes the kernels are tuned for, which the tiny models never reach."""
+def real_shape_dirs(tmp_path_factory):
+    """Two layers at a GPT-2 shape's own sizes (small: width 768, 12 heads of 64, inner 3072; xl:
+    width 1600, 25 heads, inner 6400; the odd vocabulary of 50,257): the sizes the kernels are tuned
+    for, which the tiny models never reach. Made when first asked for."""
     import json
 
     from conftest import sharpen_attention
 
-    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 768, "n_head": 12,
-              "n_inner": 3072, "vocab_size": 50257, "n_positions": 1024, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
-    folder = tmp_path_factory.mktemp("small_shape")
-    weights = plain_gpt2.random_weights(config, 5)
-    sharpen_attention(weights, config, factor=3.0)
-    (folder / "config.json").write_text(json.dumps(config))
-    plain_gpt2.write_safetensors(folder / "model.safetensors", {"transformer." + k: v for k, v in weights.items()})
-    return folder, config, weights
+    made = {}
+
+    def get(shape):
+        if shape not in made:
+            config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "vocab_size": 50257, "n_positions": 1024,
+                      "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new", **REAL_SHAPES[shape]}
+            folder = tmp_path_factory.mktemp(f"shape_{shape}")
+            weights = plain_gpt2.random_weights(config, 5)
+            sharpen_attention(weights, config, factor=3.0)
+            (folder / "config.json").write_text(json.dumps(config))
+            plain_gpt2.write_safetensors(folder / "model.safetensors", {"transformer." + k: v for k, v in weights.items()})
+            made[shape] = (folder, config, weights)
+        return made[shape]
+
+    return get
+
+
+@pytest.fixture
+def small_shape_dir(real_shape_dirs):
+    return real_shape_dirs("small")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -126,3 +145,59 @@ def test_long_prompts_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype):
             want = ref[name][position]
             err = np.abs(row - want)
             assert (err <= tol["atol"] + tol["rtol"] * np.abs(want)).all(), f"request {name} position {position}: max error {err.max():.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_live", [20, 40, 64])
+def test_many_decoding_requests_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype, n_live):
+    # decode steps of 20, 40 and 64 rows (beyond the layer kernels: the products of few rows at two
+    # and four row tiles, rows handed on in the packed layout, products cut along K), after short
+    # prompts fed eight requests a step
+    folder, config, weights = small_shape_dir
+    requests = {f"d{i}": random_tokens(400 + i, 4 + (7 * i) % 23 + 3, config["vocab_size"]) for i in range(n_live)}
+    collector = replay.Collector()
+    names = list(requests)
+    for at in range(0, n_live, 8):
+        collector.add([(name, requests[name][:-3], [len(requests[name]) - 4]) for name in names[at : at + 8]])
+    for i in range(3, 0, -1):
+        collector.add([(name, requests[name][-i : len(requests[name]) - i + 1], [0]) for name in names], end=names if i == 1 else [])
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector))
+    got = collector.gather(outputs)
+    ref = replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16"))
+    tol = replay.tolerance(dtype)
+    for name, rows in got.items():
+        assert len(rows) == 4
+        for position, row in rows.items():
+            want = ref[name][position]
+            err = np.abs(row - want)
+            assert (err <= tol["atol"] + tol["rtol"] * np.abs(want)).all(), f"request {name} position {position}: max error {err.max():.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_at_gpt2_xl_sizes(real_shape_dirs, tmp_path, dtype):
+    # width 1600 with 25 heads: no layer kernels at this width, other cuts along K, an odd number of heads;
+    # a mixed trace, then 40 requests decoding together
+    folder, config, weights = real_shape_dirs("xl")
+    requests = {f"x{i}": random_tokens(500 + i, n, config["vocab_size"]) for i, n in enumerate((33, 90, 17, 70))}
+    collector = replay.mixed(requests, seed=2)
+    many = {f"m{i}": random_tokens(600 + i, 5 + (5 * i) % 17, config["vocab_size"]) for i in range(40)}
+    names = list(many)
+    for at in range(0, 40, 8):
+        collector.add([(name, many[name][:-2], [len(many[name]) - 3]) for name in names[at : at + 8]])
+    for i in (2, 1):
+        collector.add([(name, many[name][-i : len(many[name]) - i + 1], [0]) for name in names], end=names if i == 1 else [])
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector))
+    got = collector.gather(outputs)
+    assert all(len(rows) == (len(requests[name]) if name in requests else 3) for name, rows in got.items())
+    exact = replay.plain_logits(config, weights, {**requests, **many})
+    if dtype == "float32":
+        tol = replay.tolerance(dtype)
+        for name, rows in got.items():
+            for position, row in rows.items():
+                err = np.abs(row - exact[name][position])
+                assert (err <= tol["atol"] + tol["rtol"] * np.abs(exact[name][position])).all(), f"request {name} position {position}: max error {err.max():.3e}"
+    else:
+        # at this width single logits among millions leave the fixed bound of the tiny models by
+        # rounding alone (largest differences 0.02 to 0.034 against 0.025 + 2 %): the bound here is
+        # the rounding noise itself
+        replay.compare_within_rounding_noise(got, replay.plain_logits(config, weights, {**requests, **many}, bf16=True), exact)
