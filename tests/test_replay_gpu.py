@@ -75,6 +75,7 @@ def test_replay_hands_out_the_stream_after_every_layer(model_dirs, tmp_path, dty
 
 REAL_SHAPES = {  # two layers at the sizes of the GPT-2 shapes the benchmarks run
     "small": dict(n_embd=768, n_head=12, n_inner=3072),
+    "medium": dict(n_embd=1024, n_head=16, n_inner=4096),
     "xl": dict(n_embd=1600, n_head=25, n_inner=6400),
 }
 
@@ -111,11 +112,13 @@ def small_shape_dir(real_shape_dirs):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_replay_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype):
+@pytest.mark.parametrize("shape", ["small", "medium"])
+def test_replay_at_gpt2_small_and_medium_sizes(real_shape_dirs, tmp_path, dtype, shape):
     # mixed: portions beside decoded tokens of up to four requests, then the last tokens one by one
-    # (at these sizes the bfloat16 decode steps take the layer kernels, the portions the tiled
-    # products and the prompt attention; the head runs over the whole odd vocabulary)
-    folder, config, weights = small_shape_dir
+    # (at small's sizes the bfloat16 decode steps take the layer kernels, at medium's the separate
+    # kernels; the portions take the tiled products and the prompt attention; the head runs over the
+    # whole odd vocabulary)
+    folder, config, weights = real_shape_dirs(shape)
     requests = {f"s{i}": random_tokens(200 + i, n, config["vocab_size"]) for i, n in enumerate((40, 70, 130, 23, 65))}
     collector = replay.mixed(requests, seed=1)
     outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector))
