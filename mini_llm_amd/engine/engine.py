@@ -15,7 +15,7 @@ import numpy as np
 
 from ..sampling import SamplingParams
 from .batch import StepEntry
-from .loading import DEFAULT_PAGE_SIZE, load_model, make_cache, random_model
+from .loading import DEFAULT_PAGE_SIZE, load_model, make_cache, random_model, tokens_for_memory
 from .scheduler import Request, Scheduler
 from .step import ModelRunner
 
@@ -28,6 +28,7 @@ class EngineOptions:
     dtype: str = "bfloat16"
     max_sessions: int = 64
     max_tokens: int | None = None        # cache capacity in tokens; None: max_sessions full contexts
+    cache_gib: float | None = None       # or the capacity as memory: GiB of page pools (an MI355X has 288 GB to give)
     page_size: int = DEFAULT_PAGE_SIZE
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
     use_graphs: bool = True              # replay decode steps from captured HIP graphs
@@ -162,7 +163,13 @@ class Engine:
         self.options = options
         self.model = model if model is not None else load_model(model_dir, options.dtype, options.device)
         limit = self.model.max_positions() or 4096
-        max_tokens = options.max_tokens or options.max_sessions * limit
+        if options.max_tokens is not None and options.cache_gib is not None:
+            raise ValueError("give the cache's capacity as max_tokens or as cache_gib, not both")
+        if options.cache_gib is not None:
+            element_size = 2 if options.dtype == "bfloat16" else 4
+            max_tokens = tokens_for_memory(self.model.cache_groups(), element_size, options.cache_gib, options.page_size)
+        else:
+            max_tokens = options.max_tokens or options.max_sessions * limit
         self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
                                 max_requests=options.max_sessions, device=options.device)
         self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs)

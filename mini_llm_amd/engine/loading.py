@@ -39,6 +39,24 @@ def random_model(config, seed: int, dtype, device="cuda:0"):
     return model
 
 
+def cache_bytes_per_token(groups, element_size: int) -> int:
+    """What one token of one request takes in the page pools: a key row and a value row in every
+    cache layer. (Every group's pool holds pages for the same number of tokens; a group with a
+    window gives most of them back, but is sized like the others.)"""
+    return sum(len(g.layers) * 2 * g.n_kv_heads * g.head_size * element_size for g in groups)
+
+
+def tokens_for_memory(groups, element_size: int, gib: float, page_size: int) -> int:
+    """The cache capacity in tokens (whole pages) that ``gib`` GiB of page pools hold."""
+    per_token = cache_bytes_per_token(groups, element_size)
+    if per_token == 0:
+        raise ValueError("this model keeps no keys and values: its cache cannot be sized by memory")
+    tokens = int(gib * (1 << 30)) // per_token // page_size * page_size
+    if tokens < page_size:
+        raise ValueError(f"{gib} GiB hold not even one page of {page_size} tokens ({per_token} bytes a token)")
+    return tokens
+
+
 def make_cache(model, *, max_tokens: int, page_size: int = DEFAULT_PAGE_SIZE, max_requests: int = 256, device="cuda:0"):
     """A cache whose every group holds ``max_tokens`` tokens' worth of pages."""
     num_pages = max(1, -(-max_tokens // page_size))

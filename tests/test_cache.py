@@ -170,3 +170,18 @@ def test_state_slots_exist_even_without_state(tmp_path):
     m.close("a"); m.open("b")
     assert m.requests["b"].state_slot == slot and (m.state[0][slot] == 0).all()
     assert m.k_pages[0].shape == (2, 2, 16, 16) and m.v_pages[1].shape == (2, 2, 16, 16)
+
+
+def test_capacity_from_memory():
+    from mini_llm_amd.engine.loading import cache_bytes_per_token, tokens_for_memory
+
+    small = [CacheGroupSpec("full", tuple(range(12)), 12, 64, None)]
+    assert cache_bytes_per_token(small, 2) == 36864 and cache_bytes_per_token(small, 4) == 73728   # GPT-2 small: 73,728 bytes a token in 32-bit
+    assert tokens_for_memory(small, 4, 4.5, 64) == 65536                     # 64 contexts of 1,024 tokens are 4.5 GiB
+    two = small + [CacheGroupSpec("window", (12, 13), 2, 32, 100)]
+    assert cache_bytes_per_token(two, 2) == 36864 + 2 * 2 * 2 * 32 * 2
+    assert tokens_for_memory(two, 2, 1.0, 128) % 128 == 0
+    with pytest.raises(ValueError):
+        tokens_for_memory(small, 4, 1e-6, 64)
+    with pytest.raises(ValueError):
+        tokens_for_memory([], 4, 1.0, 64)

@@ -383,3 +383,16 @@ def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dt
                 assert after["dropped_tokens"] == 0
     for temperature in (0.0, 0.9):
         assert results[True, temperature] == results[False, temperature]
+
+
+def test_cache_sized_by_memory(model_dirs):
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    folder, config, weights = model_dirs["A"]
+    per_token = config["n_layer"] * 2 * config["n_embd"] * 4
+    engine = Engine(folder, EngineOptions(dtype="float32", cache_gib=300 * 64 * per_token / (1 << 30), page_size=64, max_sessions=4))
+    assert engine.cache.free_pages() == [300]
+    prompt = random_tokens(9, 12, config["vocab_size"])
+    assert engine.generate([prompt], max_new_tokens=6)[0] == plain_gpt2.greedy(config, weights, prompt, 6)
+    with pytest.raises(ValueError):
+        Engine(folder, EngineOptions(dtype="float32", cache_gib=1.0, max_tokens=1024))
