@@ -464,14 +464,15 @@ int skinny_k_blocks(int N, int K) {
 // the compute units idle is cut, while the tiles of the cut product are no more than one and a
 // half to a compute unit and every block keeps eight LDS tiles of K (measured: a product that
 // nearly fills the chip gains less from the cut than adding the partial products up costs). Up to
-// 256 rows of bfloat16 a block may go down to four LDS tiles: the partial products are small then,
-// and a 128 x 768 x 768 product takes 6.1 us in two cuts against 7.9 us whole.
+// 256 rows a block may go down to four LDS tiles: the partial products are small then, and a
+// 128 x 768 x 768 product takes 6.1 us in two cuts against 7.9 us whole (bfloat16; in 32-bit 8.6 us
+// in four cuts against 12.6 us in two).
 template <typename T>
 int tiled_k_blocks(int M, int N, int K) {
     int tiles = ceil_div(M, 128) * ceil_div(N, 64);
     int k_blocks = 1;
     if (tiles > 128) return 1;
-    const int least_tiles = sizeof(T) == 2 && M <= 256 ? 4 : 8;
+    const int least_tiles = M <= 256 ? 4 : 8;
     while (k_blocks < 8 && tiles * k_blocks * 2 <= 384 && K >= least_tiles * Tile<T>::BK * k_blocks * 2) k_blocks *= 2;
     return k_blocks;
 }
@@ -500,7 +501,7 @@ void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const 
         if (M <= 32) tile = 1;
         else if (M <= 64) tile = 2;
         else if (k_blocks == 1 && ceil_div(M, 256) * ceil_div(N, 128) >= (sizeof(T) == 4 ? 256 : 128)) tile = 3;  // 32-bit products are bound by the matrix cores: no compute unit may idle
-        else if (sizeof(T) == 2 && ceil_div(M, 128) * ceil_div(N, 64) * k_blocks <= 128) tile = 2;  // half a block a compute unit or less: twice as many smaller blocks are 10 to 20 % faster (bfloat16, measured from 96 to 1,024 rows)
+        else if (ceil_div(M, 128) * ceil_div(N, 64) * k_blocks <= 128) tile = 2;  // half a block a compute unit or less: twice as many smaller blocks are 10 to 20 % faster in bfloat16 and a third faster in 32-bit (measured from 96 to 1,024 rows)
         else tile = 7;
     }
     switch (tile) {  // other shapes (128x128, 256x128 with eight waves, fewer waves) were measured and lost at every size here
