@@ -273,6 +273,13 @@ def measure_peaks():
     return result
 
 
+def emit(record: dict, path) -> None:
+    line = json.dumps(record)
+    print(line)
+    if path:
+        Path(path).write_text(line + "\n")
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -281,7 +288,9 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--shape", default="small", choices=("small", "medium", "xl"), help="the GPT-2 shape that is run (the headline is small)")
-    parser.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens of each sequence's prompt before decoding is timed")
+    parser.add_argument("--prompt-len", "--prompt-tokens", dest="prompt_len", type=int, default=PROMPT_LEN,
+                        help="tokens of each sequence's prompt before decoding is timed (--prompt-tokens is the reference's name: engine/bench/bench_options.c:25-94)")
+    parser.add_argument("--json", default=None, metavar="PATH", help="also write the printed record to this file (the reference's option)")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-check", action="store_true", help="skip the comparison of decoding with a whole-prompt step before timing")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
@@ -296,11 +305,11 @@ def main() -> int:
         return 2
 
     if args.peaks:
-        print(json.dumps({"measured_peaks": measure_peaks(), "published": {"hbm_GBs": HBM_GBS, "mfma_bf16_TFLOPs": 2500.0, "mfma_fp32_TFLOPs": 157.3}}))
+        emit({"measured_peaks": measure_peaks(), "published": {"hbm_GBs": HBM_GBS, "mfma_bf16_TFLOPs": 2500.0, "mfma_fp32_TFLOPs": 157.3}}, args.json)
         return 0
 
     if args.serving:
-        print(json.dumps({"serving": measure_serving(args.dtype, args.temperature, not args.step_by_step)}))
+        emit({"serving": measure_serving(args.dtype, args.temperature, not args.step_by_step)}, args.json)
         return 0
 
     from mini_llm_amd.config import config_from_dict
@@ -316,7 +325,7 @@ def main() -> int:
 
     checked = None if args.no_check else check_before_timing(engine)
     if args.prefill_only:
-        print(json.dumps({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}))
+        emit({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}, args.json)
         return 0
     seconds, step_bytes = DecodeBench(engine, args.batch, args.prompt_len).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
@@ -351,7 +360,7 @@ def main() -> int:
             s, _ = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
             points[f"decode_b{batch}"] = round(batch * steps / s, 1)
         record["points"] = points
-    print(json.dumps(record))
+    emit(record, args.json)
     return 0
 
 
