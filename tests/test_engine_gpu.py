@@ -396,3 +396,34 @@ def test_cache_sized_by_memory(model_dirs):
     assert engine.generate([prompt], max_new_tokens=6)[0] == plain_gpt2.greedy(config, weights, prompt, 6)
     with pytest.raises(ValueError):
         Engine(folder, EngineOptions(dtype="float32", cache_gib=1.0, max_tokens=1024))
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_workloads_through_the_scheduler_match_plain_greedy(model_dirs, engines, seed):
+    # random prompt lengths and lengths to generate, portions under a small budget, a pool that holds
+    # a few requests (so some wait and some are preempted and recomputed): whatever the scheduler
+    # does, every request gets the plain implementation's greedy tokens
+    name = "AB"[seed]
+    _, config, weights = model_dirs[name]
+    rng = np.random.default_rng(50 + seed)
+    limit = config["n_positions"]
+    prompts, new = [], []
+    for i in range(14):
+        n = int(rng.integers(1, limit // 2))
+        prompts.append(random_tokens(700 + 20 * seed + i, n, config["vocab_size"]))
+        new.append(int(rng.integers(1, min(24, limit - n) + 1)))
+    engine = engines(name, "float32", max_sessions=5, max_tokens=2 * limit, page_size=16, max_tokens_per_step=int(rng.integers(8, 40)))
+    before = engine.stats()["preemptions"]
+    outputs = [engine.generate([prompt], max_new_tokens=n)[0] for prompt, n in zip(prompts[:2], new[:2])]   # alone
+    from mini_llm_amd.engine.scheduler import Request
+
+    together, errors = [[] for _ in prompts], []
+    for i, (prompt, n) in enumerate(zip(prompts, new)):
+        engine.submit(Request(prompt, n, None, lambda token, finish, i=i: together[i].append(token), errors.append))
+    engine.scheduler.run_until_idle()
+    assert not errors
+    assert engine.stats()["preemptions"] > before   # the pool is that small
+    for i, (prompt, n) in enumerate(zip(prompts, new)):
+        assert together[i] == plain_gpt2.greedy(config, weights, prompt, n), f"request {i} ({len(prompt)} prompt tokens, {n} new)"
+    assert outputs == together[:2]
+    assert engine.cache.free_pages() == [engine.cache.pools[0].num_pages] and not engine.cache.requests
