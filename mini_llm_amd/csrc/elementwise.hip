@@ -71,14 +71,20 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
 
     if constexpr (ROW_REGS > 0) {
         // the row, the gains and the offsets are all asked for before anything is reduced, so the
-        // kernel waits for memory once
-        float values[ROW_REGS], gains[ROW_REGS], offsets[ROW_REGS];
+        // kernel waits for memory once; a long row leaves the gains and offsets (which every wave
+        // reads, so they come from the cache) for when they are used: three times its length in
+        // registers would leave too few waves to keep the memory busy
+        constexpr bool EARLY = ROW_REGS <= 16;
+        constexpr int KEPT = EARLY ? ROW_REGS : 1;
+        float values[ROW_REGS], gains[KEPT], offsets[KEPT];
 #pragma unroll
         for (int r = 0; r < ROW_REGS; r++) {
             int i = min(lane + r * WAVE, width - 1);
             values[r] = in_row[i];
-            gains[r] = gamma[i];
-            offsets[r] = beta[i];
+            if constexpr (EARLY) {
+                gains[r] = gamma[i];
+                offsets[r] = beta[i];
+            }
         }
         float sum = 0.0f;
 #pragma unroll
@@ -98,8 +104,10 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
 #pragma unroll
         for (int r = 0; r < ROW_REGS; r++) {
             int i = lane + r * WAVE;
-            if (i < width)
-                out[packed_out ? packed_element<OutT>(row, i, width) : (size_t)row * width + i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gains[r] + offsets[r]);
+            if (i < width) {
+                float gain = EARLY ? gains[EARLY ? r : 0] : gamma[i], offset = EARLY ? offsets[EARLY ? r : 0] : beta[i];
+                out[packed_out ? packed_element<OutT>(row, i, width) : (size_t)row * width + i] = from_float<OutT>((values[r] - mean) * inverse_stddev * gain + offset);
+            }
         }
     } else {
         float sum = 0.0f;
@@ -116,6 +124,70 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int* __restr
     }
 }
 
+// The same for rows whose length is a multiple of four: 16-byte pieces, PIECES of them per lane in
+// registers (PIECES * 256 >= width), so a row of 1,600 is seven loads a lane instead of twenty-five.
+// The gains and offsets are asked for with the row while they fit beside it (PIECES <= 4).
+template <typename OutT, int PIECES>
+__global__ void layernorm_pieces_kernel(const float* __restrict__ x, const int* __restrict__ row_index,
+                                        const float* __restrict__ gamma, const float* __restrict__ beta,
+                                        OutT* __restrict__ out, int n_rows, int width, float eps, int packed_out) {
+    int lane = threadIdx.x % WAVE;
+    int row = blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (row >= n_rows) return;
+    int source = row_index ? row_index[row] : row;
+    const f32x4* in_row = reinterpret_cast<const f32x4*>(x + (size_t)source * width);
+    const f32x4* gain_pieces = reinterpret_cast<const f32x4*>(gamma);
+    const f32x4* offset_pieces = reinterpret_cast<const f32x4*>(beta);
+    const int n_pieces = width / 4;
+    const float n = (float)width;
+    constexpr bool EARLY = PIECES <= 4;
+    constexpr int KEPT = EARLY ? PIECES : 1;
+    f32x4 values[PIECES], gains[KEPT], offsets[KEPT];
+#pragma unroll
+    for (int r = 0; r < PIECES; r++) {
+        int piece = min(lane + r * WAVE, n_pieces - 1);
+        values[r] = in_row[piece];
+        if constexpr (EARLY) {
+            gains[r] = gain_pieces[piece];
+            offsets[r] = offset_pieces[piece];
+        }
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < PIECES; r++) {
+        if (lane + r * WAVE >= n_pieces) values[r] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        sum += (values[r][0] + values[r][1]) + (values[r][2] + values[r][3]);
+    }
+    float mean = wave_sum(sum) / n;
+    float squares = 0.0f;
+#pragma unroll
+    for (int r = 0; r < PIECES; r++) {
+        if (lane + r * WAVE < n_pieces) {
+            f32x4 d = values[r] - mean;
+            squares += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+        }
+    }
+    float inverse_stddev = 1.0f / sqrtf(wave_sum(squares) / n + eps);
+#pragma unroll
+    for (int r = 0; r < PIECES; r++) {
+        int piece = lane + r * WAVE;
+        if (piece < n_pieces) {
+            f32x4 gain = EARLY ? gains[EARLY ? r : 0] : gain_pieces[piece], offset = EARLY ? offsets[EARLY ? r : 0] : offset_pieces[piece];
+            f32x4 y = (values[r] - mean) * inverse_stddev * gain + offset;
+            // four consecutive columns lie together in the packed layout too (inside one 16-byte piece)
+            OutT* at = out + (packed_out ? packed_element<OutT>(row, 4 * piece, width) : (size_t)row * width + 4 * piece);
+            if constexpr (sizeof(OutT) == 2) {
+                bf16x4 rounded;
+#pragma unroll
+                for (int e = 0; e < 4; e++) rounded[e] = from_float<OutT>(y[e]);
+                *reinterpret_cast<bf16x4*>(at) = rounded;
+            } else {
+                *reinterpret_cast<f32x4*>(at) = y;
+            }
+        }
+    }
+}
+
 template <typename OutT>
 static void launch_layernorm(const float* x, const int* row_index, const float* gamma,
                              const float* beta, void* out, int n_rows, int width, float eps,
@@ -123,6 +195,20 @@ static void launch_layernorm(const float* x, const int* row_index, const float* 
     const int waves = 4;
     dim3 grid(ceil_div(n_rows, waves)), block(waves * WAVE);
     OutT* o = (OutT*)out;
+    const bool aligned = (((size_t)x | (size_t)gamma | (size_t)beta | (size_t)out) & 15) == 0;  // 16-byte pieces need it
+    if (aligned && width % 4 == 0 && width <= 16 * 4 * WAVE) {
+        if (width <= 1 * 4 * WAVE)
+            layernorm_pieces_kernel<OutT, 1><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
+        else if (width <= 2 * 4 * WAVE)
+            layernorm_pieces_kernel<OutT, 2><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
+        else if (width <= 4 * 4 * WAVE)
+            layernorm_pieces_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
+        else if (width <= 8 * 4 * WAVE)
+            layernorm_pieces_kernel<OutT, 8><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
+        else
+            layernorm_pieces_kernel<OutT, 16><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
+        return;
+    }
     if (width <= 4 * WAVE)
         layernorm_kernel<OutT, 4><<<grid, block, 0, stream>>>(x, row_index, gamma, beta, o, n_rows, width, eps, packed_out);
     else if (width <= 12 * WAVE)

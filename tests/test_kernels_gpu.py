@@ -50,7 +50,8 @@ def test_embed(K, dtype, rows, width, vocab, npos):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,width,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (9, 768, 1e-5), (3, 1030, 1e-3), (2, 2500, 1e-5)])
+@pytest.mark.parametrize("rows,width,eps", [(1, 64, 1e-5), (5, 96, 1e-6), (9, 768, 1e-5), (3, 1030, 1e-3), (2, 2500, 1e-5),
+                                            (4, 320, 1e-5), (70, 1600, 1e-5), (2, 4096, 1e-5), (2, 4100, 1e-5), (3, 6, 1e-5), (300, 1024, 1e-5)])
 def test_layernorm(K, out_dtype, rows, width, eps):
     rng = np.random.default_rng(1)
     x = (rng.standard_normal((rows, width)) * 2 + 50).astype(np.float32)  # a large mean
@@ -116,7 +117,7 @@ def packed_rows_of(K, x, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,width,n_partials", [(1, 64, 0), (17, 200, 3), (64, 768, 2), (33, 100, 0)])
+@pytest.mark.parametrize("rows,width,n_partials", [(1, 64, 0), (17, 200, 3), (64, 768, 2), (33, 100, 0), (40, 1600, 0), (20, 1024, 2)])
 def test_layernorm_leaves_packed_rows(K, dtype, rows, width, n_partials):
     rng = np.random.default_rng(rows + width)
     gamma, beta = 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)
