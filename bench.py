@@ -320,7 +320,7 @@ def main() -> int:
         parser.error(f"--prompt-len must be in 1..{CONTEXT - 1}")
     layers = args.layers or shape["n_layer"]
     config = config_from_dict(dict(shape, n_layer=layers))
-    largest = max(args.batch, 1 if args.no_points else 64)
+    largest = max(args.batch, 1 if args.no_points else 64, 1 if args.no_check else 2)   # the check before timing runs two sequences
     engine = Engine.from_random(config, seed, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
 
     checked = None if args.no_check else check_before_timing(engine)
