@@ -218,13 +218,26 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     KeySweep<T, HD> sweep;
     sweep.init();
     if (begin < end) {
+        // The query and the pages of the first round are asked for together, the rows of that round
+        // as soon as the pages are known, and only then is the query looked at; the pages of a
+        // round are asked for before the round before it is taken into the softmax. So a wave's
+        // first keys are three trips to memory away (request and position; pages; rows), not five.
+        constexpr int UNROLL = KeySweep<T, HD>::UNROLL;
+        const int spare_key = end - 1;
+        const typename Chunk<T>::Raw raw = *reinterpret_cast<const typename Chunk<T>::Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
+        int page[UNROLL];
+        sweep.look_up(page, table, page_shift, begin, end, spare_key, lane);
+        typename KeySweep<T, HD>::Fetched f;
+        sweep.fetch_rows(f, page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
         float qf[VEC];
-        {
-            typename Chunk<T>::Raw raw = *reinterpret_cast<const typename Chunk<T>::Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
 #pragma unroll
-            for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
+        for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
+        for (int base = begin; base < end; base += KPI) {
+            const int next = base + KPI;
+            if (next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
+            sweep.consume(f, qf, base, end, lane);
+            if (next < end) sweep.fetch_rows(f, page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, next, end, spare_key, lane);
         }
-        sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin, end, lane);
     }
     sweep.merge_groups();
     const float* o = sweep.o;
