@@ -335,6 +335,24 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         x_base[i] = x_packed ? A + (size_t)min(i, (M - 1) / 16) * n_steps * (64 * VEC) : A + (size_t)(x_valid[i] ? t : 0) * K;
     }
 
+    // What the epilogue will want from memory for this thread's outputs (bias, residual, the cache
+    // slot of a key or value row) is asked for now and arrives while the products run: asked for in
+    // the epilogue it would be one more trip to memory at the end of a kernel that is a few long.
+    constexpr int ITEMS = (MT * 4 * WAVE + WAVE * KSPLIT - 1) / (WAVE * KSPLIT);  // outputs a thread finishes
+    float early_bias[ITEMS], early_residual[ITEMS];
+    int early_slot[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++) {
+        int index = threadIdx.x + j * WAVE * KSPLIT;
+        int l = index % WAVE, ir = index / WAVE;
+        int token = (ir / 4) * 16 + l % 16;
+        int col = n0 + 4 * (l / 16) + ir % 4;
+        bool wanted = index < MT * 4 * WAVE && token < M && col < N;
+        early_bias[j] = bias && wanted ? bias[col] : 0.0f;
+        early_residual[j] = residual && wanted && !scatter.enabled ? residual[(size_t)token * N + col] : 0.0f;
+        early_slot[j] = scatter.enabled && wanted && col >= scatter.q_width ? scatter.slots[token] : -1;
+    }
+
     // The block takes the k-steps first_step .. last_step-1: all of them, or, when the launch has
     // several blocks per 16 columns (gridDim.y), its part of K, whose sums then go to matrix
     // blockIdx.y of `out` (partial products; the caller passes no bias, residual or epilogue).
@@ -394,7 +412,10 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
 #pragma unroll
         for (int r = 0; r < 4; r++) sums[wave][i * 4 + r][lane] = acc[i][r];
     __syncthreads();
-    for (int index = threadIdx.x; index < MT * 4 * WAVE; index += WAVE * KSPLIT) {
+#pragma unroll
+    for (int j = 0; j < ITEMS; j++) {
+        int index = threadIdx.x + j * WAVE * KSPLIT;
+        if (index >= MT * 4 * WAVE) continue;
         int l = index % WAVE, ir = index / WAVE;
         int token = (ir / 4) * 16 + l % 16;
         int col = n0 + 4 * (l / 16) + ir % 4;
@@ -402,14 +423,14 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         float value = 0.0f;
 #pragma unroll
         for (int w = 0; w < KSPLIT; w++) value += sums[w][ir][l];  // the same order for every element
-        if (bias) value += bias[col];
+        if (bias) value += early_bias[j];
         if (epilogue == MLLM_EPI_GELU_TANH) value = sizeof(OutT) == 2 ? gelu_tanh_for_bf16(value) : gelu_tanh(value);
         else if (epilogue == MLLM_EPI_GELU_ERF) value = sizeof(OutT) == 2 ? gelu_erf_for_bf16(value) : gelu_erf(value);
         if (scatter.enabled) {
             if (col < scatter.q_width) {
                 out[(size_t)token * scatter.q_width + col] = from_float<OutT>(value);
             } else {
-                int slot = scatter.slots[token];
+                int slot = early_slot[j];
                 if (slot < 0) continue;
                 int c = col - scatter.q_width;
                 OutT* pages = (OutT*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
@@ -421,7 +442,7 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
             continue;
         }
         size_t at = (size_t)token * N + col;
-        if (residual) value = residual[at] + value;
+        if (residual) value = early_residual[j] + value;
         out[out_packed ? packed_element<OutT>(token, col, N) : at] = from_float<OutT>(value);
     }
 }
