@@ -339,6 +339,7 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
     // slot of a key or value row) is asked for now and arrives while the products run: asked for in
     // the epilogue it would be one more trip to memory at the end of a kernel that is a few long.
     constexpr int ITEMS = (MT * 4 * WAVE + WAVE * KSPLIT - 1) / (WAVE * KSPLIT);  // outputs a thread finishes
+    constexpr bool EARLY = MT < 4;  // with four row tiles the registers are better left to the loads of x
     float early_bias[ITEMS], early_residual[ITEMS];
     int early_slot[ITEMS];
 #pragma unroll
@@ -347,7 +348,7 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         int l = index % WAVE, ir = index / WAVE;
         int token = (ir / 4) * 16 + l % 16;
         int col = n0 + 4 * (l / 16) + ir % 4;
-        bool wanted = index < MT * 4 * WAVE && token < M && col < N;
+        bool wanted = EARLY && index < MT * 4 * WAVE && token < M && col < N;
         early_bias[j] = bias && wanted ? bias[col] : 0.0f;
         early_residual[j] = residual && wanted && !scatter.enabled ? residual[(size_t)token * N + col] : 0.0f;
         early_slot[j] = scatter.enabled && wanted && col >= scatter.q_width ? scatter.slots[token] : -1;
@@ -423,14 +424,14 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
         float value = 0.0f;
 #pragma unroll
         for (int w = 0; w < KSPLIT; w++) value += sums[w][ir][l];  // the same order for every element
-        if (bias) value += early_bias[j];
+        if (bias) value += EARLY ? early_bias[j] : bias[col];
         if (epilogue == MLLM_EPI_GELU_TANH) value = sizeof(OutT) == 2 ? gelu_tanh_for_bf16(value) : gelu_tanh(value);
         else if (epilogue == MLLM_EPI_GELU_ERF) value = sizeof(OutT) == 2 ? gelu_erf_for_bf16(value) : gelu_erf(value);
         if (scatter.enabled) {
             if (col < scatter.q_width) {
                 out[(size_t)token * scatter.q_width + col] = from_float<OutT>(value);
             } else {
-                int slot = early_slot[j];
+                int slot = EARLY ? early_slot[j] : scatter.slots[token];
                 if (slot < 0) continue;
                 int c = col - scatter.q_width;
                 OutT* pages = (OutT*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
@@ -442,7 +443,7 @@ __global__ __launch_bounds__(64 * KSPLIT) void gemm_skinny_kernel(
             continue;
         }
         size_t at = (size_t)token * N + col;
-        if (residual) value = early_residual[j] + value;
+        if (residual) value = (EARLY ? early_residual[j] : residual[at]) + value;
         out[out_packed ? packed_element<OutT>(token, col, N) : at] = from_float<OutT>(value);
     }
 }
