@@ -232,10 +232,14 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
         float qf[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
+        // (in 32-bit the pages are asked for after the round: held across it they cost registers,
+        // and over the many rounds of a long context that lost 5 %)
+        constexpr bool PAGES_AHEAD = sizeof(T) == 2;
         for (int base = begin; base < end; base += KPI) {
             const int next = base + KPI;
-            if (next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
+            if (PAGES_AHEAD && next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
             sweep.consume(f, qf, base, end, lane);
+            if (!PAGES_AHEAD && next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
             if (next < end) sweep.fetch_rows(f, page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, next, end, spare_key, lane);
         }
     }
