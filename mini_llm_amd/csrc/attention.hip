@@ -180,7 +180,8 @@ constexpr int DECODE_MAX_SPLITS = 16;
 
 // A block per (token, head); its waves (blockDim.x / 64 of them, a power of two up to 16) split
 // the token's keys evenly among themselves, and their partial results meet in LDS.
-template <typename T, int HD>
+// TOGETHER: how a wave starts (see there); the host chooses.
+template <typename T, int HD, bool TOGETHER>
 __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
@@ -217,7 +218,17 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
 
     KeySweep<T, HD> sweep;
     sweep.init();
-    if (begin < end) {
+    if (begin < end && !TOGETHER) {
+        // the plain order: the query, then round by round the pages, their rows, the softmax
+        float qf[VEC];
+        {
+            typename Chunk<T>::Raw raw = *reinterpret_cast<const typename Chunk<T>::Raw*>(q + (size_t)token * q_stride + head * HD + sub * VEC);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) qf[i] = Chunk<T>::get(raw, i) * scale;
+        }
+        sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin, end, lane);
+    }
+    if (begin < end && TOGETHER) {
         // The query and the pages of the first round are asked for together, the rows of that round
         // as soon as the pages are known, and only then is the query looked at; the pages of a
         // round are asked for before the round before it is taken into the softmax. So a wave's
@@ -274,11 +285,25 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
                     const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
                     int page_shift, int window, float scale, int n_splits, int out_packed, hipStream_t stream) {
     dim3 grid(n_heads, n_tokens), block(WAVE * n_splits);
+    // Measured on MI355X: starting with query and pages together (and, in bfloat16, the pages a
+    // round ahead) is 3 to 15 % faster wherever a wave has few rounds, which is where a kernel's
+    // start counts; in 32-bit it takes twice the registers, and over the many rounds of long
+    // contexts with few waves a token (64 x 25 heads at 900 keys, two waves each) the plain
+    // order is 5 % faster.
+    const int reach = max_blocks << page_shift;
+    const int keys_per_round = (sizeof(T) == 2 ? 4096 : 2048) / head_size;  // KeySweep's KPI
+    const int rounds = ceil_div(ceil_div(window > 0 && window < reach ? window : reach, n_splits), keys_per_round);
+    const bool together = sizeof(T) == 2 || rounds <= 12;
 #define MLLM_DECODE_CASE(HD)                                                                                   \
     case HD:                                                                                                   \
-        attention_decode_kernel<T, HD><<<grid, block, 0, stream>>>(                                            \
-            (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-            positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
+        if (together)                                                                                          \
+            attention_decode_kernel<T, HD, true><<<grid, block, 0, stream>>>(                                  \
+                (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
+        else                                                                                                   \
+            attention_decode_kernel<T, HD, false><<<grid, block, 0, stream>>>(                                 \
+                (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
