@@ -516,10 +516,10 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
 
 // ------------------------------------------------------------------------------------------------
 // norm -> up product -> activation -> this slice's share of the down product.
-// grid (slices of U hidden units, groups of 4, 8 or 16 tokens), 1024 threads. The first pieces of both
-// matrices are asked for at once; while they come, the waves take the pending sums (16 / tokens
-// waves a token, every so-manieth partial row each) and the norm; then all waves run the two
-// products.
+// grid (slices of U hidden units, groups of 1 to 16 tokens), 1024 threads. The partial rows are asked
+// for first and the first pieces of both matrices right behind them; while the matrices come, the
+// waves take the pending sums (16 / tokens waves a token, every so-manieth partial row each) and the
+// norm; then all waves run the two products.
 // ------------------------------------------------------------------------------------------------
 template <int NV, int U>
 __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
