@@ -204,3 +204,33 @@ def test_replay_at_gpt2_xl_sizes(real_shape_dirs, tmp_path, dtype):
         # rounding alone (largest differences 0.02 to 0.034 against 0.025 + 2 %): the bound here is
         # the rounding noise itself
         replay.compare_within_rounding_noise(got, replay.plain_logits(config, weights, {**requests, **many}, bf16=True), exact)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_a_context_of_three_thousand_tokens(tmp_path_factory, tmp_path, dtype, page_size):
+    # n_positions comes from config.json: a tiny model with 3,100 positions, one request fed in
+    # three long portions and then token by token (the prompt attention over dozens of key tiles, the
+    # decode attention with sixteen waves over many rounds, block tables of up to 188 pages)
+    from conftest import make_plain_model_dir
+
+    config = {"architectures": ["GPT2LMHeadModel"], "model_type": "gpt2", "n_layer": 2, "n_embd": 64, "n_head": 2, "n_inner": 96,
+              "vocab_size": 300, "n_positions": 3100, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    folder = tmp_path_factory.mktemp("long_context")
+    weights = make_plain_model_dir(folder, config, 11)
+    tokens = random_tokens(900, 3000, config["vocab_size"])
+    collector = replay.Collector()
+    at = 0
+    for n in (1500, 1000, 492):
+        collector.add([("long", tokens[at : at + n], sorted({0, 1, n // 3, n - 2, n - 1}))])
+        at += n
+    for i in range(at, len(tokens)):
+        collector.add([("long", tokens[i : i + 1], [0])], end=["long"] if i == len(tokens) - 1 else [])
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector), page_size=page_size)
+    got = collector.gather(outputs)["long"]
+    ref = replay.plain_logits(config, weights, {"long": tokens}, bf16=(dtype == "bfloat16"))["long"]
+    tol = replay.tolerance(dtype)
+    assert len(got) == 15 + 8
+    for position, row in got.items():
+        err = np.abs(row - ref[position])
+        assert (err <= tol["atol"] + tol["rtol"] * np.abs(ref[position])).all(), f"position {position}: max error {err.max():.3e}"
