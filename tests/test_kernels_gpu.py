@@ -384,6 +384,48 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
         np.testing.assert_array_equal(unpacked(packed), host(out.float()))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_over_a_block_table_of_more_than_a_thousand_pages(K, dtype):
+    # 17,000 cached keys in pages of 16 (1,066 pages, scrambled): more than the 1,024 table entries
+    # the prompt kernel keeps in LDS. A portion of 40 queries and a single decoded token; one far key
+    # made to stand out for each, in the table's first and last hundred entries. The plain side is
+    # written out for these rows only (softmax over the keys up to each row's position).
+    n_heads, head_size, page_size, total = 2, 32, 16, 17000
+    rng = np.random.default_rng(12)
+    rnd = lambda *s: bf16_round(rng.standard_normal(s)) if dtype == torch.bfloat16 else rng.standard_normal(s).astype(np.float32).astype(np.float64)
+    width = n_heads * head_size
+    n_pages = (total + page_size - 1) // page_size
+    assert n_pages > 1024
+    pages = rng.permutation(n_pages + 7)[:n_pages]
+    k_all, v_all = rnd(total, width), rnd(total, width)
+    for new, path in ((40, "matrix_cores"), (1, "split_keys")):
+        q = rnd(new, width)
+        k_here = k_all.copy()
+        for key in (37, total - new - 50):  # a hot key near each end of the table, for the last query
+            k_here[key] = (bf16_round(q[-1] * 3) if dtype == torch.bfloat16 else q[-1] * 3)
+        kp = torch.full((n_pages + 7, n_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
+        vp = torch.full_like(kp, float("nan"))
+        slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+        K.cache_write(dev(k_here, dtype), dev(v_all, dtype), kp, vp, dev(slots, torch.int32), n_heads, head_size)
+        ref = np.zeros((new, width))
+        for i in range(new):
+            position = total - new + i
+            for h in range(n_heads):
+                cols = slice(h * head_size, (h + 1) * head_size)
+                scores = k_here[: position + 1, cols] @ q[i, cols] / math.sqrt(head_size)
+                weights = np.exp(scores - scores.max())
+                ref[i, cols] = (weights / weights.sum()) @ v_all[: position + 1, cols]
+        extra = {}
+        if path == "matrix_cores":
+            extra = dict(q_starts=dev([0, new], torch.int32), context_lens=dev([total - new], torch.int32))
+        out = K.paged_attention(
+            dev(q, dtype), kp, vp, dev([0] * new, torch.int32), dev(list(range(total - new, total)), torch.int32),
+            dev(pages[None, :].astype(np.int32), torch.int32), n_heads, n_heads, head_size, 1.0 / math.sqrt(head_size),
+            max_q_len=new, **extra)
+        tol = 2e-5 if dtype == torch.float32 else 2e-2
+        np.testing.assert_allclose(host(out), ref, rtol=tol, atol=tol, err_msg=path)
+
+
 def test_paged_attention_strided_q(K):
     # q, k, v as column slices of one fused projection
     rng = np.random.default_rng(5)
