@@ -151,10 +151,11 @@ def test_long_prompts_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_live", [20, 40, 64])
+@pytest.mark.parametrize("n_live", [20, 40, 64, 100])
 def test_many_decoding_requests_at_gpt2_small_sizes(small_shape_dir, tmp_path, dtype, n_live):
-    # decode steps of 20, 40 and 64 rows (beyond the layer kernels: the products of few rows at two
-    # and four row tiles, rows handed on in the packed layout, products cut along K), after short
+    # decode steps of 20, 40, 64 and 100 rows (beyond the layer kernels: the products of few rows at two
+    # and four row tiles, rows handed on in the packed layout, products cut along K; at 100 rows the tiled
+    # product on 64 x 64 tiles with finer cuts), after short
     # prompts fed eight requests a step
     folder, config, weights = small_shape_dir
     requests = {f"d{i}": random_tokens(400 + i, 4 + (7 * i) % 23 + 3, config["vocab_size"]) for i in range(n_live)}
