@@ -235,3 +235,15 @@ def test_a_context_of_three_thousand_tokens(tmp_path_factory, tmp_path, dtype, p
     for position, row in got.items():
         err = np.abs(row - ref[position])
         assert (err <= tol["atol"] + tol["rtol"] * np.abs(ref[position])).all(), f"position {position}: max error {err.max():.3e}"
+
+
+@pytest.mark.parametrize("seed", [3, 4, 5, 6])
+def test_other_random_ways_of_mixing_requests(model_dirs, tmp_path, seed):
+    # the mixed mode again under other seeds (other portion sizes, other steps a request sits out,
+    # other moments at which pages come back and go out again), alternating models and element types
+    name, dtype = ("A", "B", "C", "A")[seed - 3], ("float32", "bfloat16")[seed % 2]
+    folder, config, weights = model_dirs[name]
+    requests = requests_for(name, config)
+    collector = replay.mixed(requests, seed=seed, max_live=3 + seed % 2, tail=5 + seed)
+    outputs = replay.run_trace(folder, dtype, collector.steps, tmp_path / "out", replay.peak_tokens(collector), page_size=(16, 32, 64, 128)[seed - 3])
+    replay.compare(collector.gather(outputs), replay.plain_logits(config, weights, requests, bf16=(dtype == "bfloat16")), **replay.tolerance(dtype))
