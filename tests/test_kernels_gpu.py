@@ -507,6 +507,47 @@ def test_top_p_sampling(K):
     assert (out == int(np.argmax(logits))).all()
 
 
+def test_draws_over_the_whole_vocabulary_are_the_generators(K):
+    # 50,257 logits a row, rows that start at odd addresses, temperature with and without top-p:
+    # every draw is argmax(logit / T + Gumbel noise) over the nucleus, with the noise of the
+    # counter-based generator worked out on the host (vectorised twin of sampling.hip's uniform_open)
+    vocab, rows = 50257, 6
+    rng = np.random.default_rng(8)
+    logits = (rng.standard_normal((rows, vocab)) * 3).astype(np.float32)
+    temperature = np.array([0.7, 1.0, 1.3, 0.9, 0.0, 2.0], dtype=np.float32)
+    top_p = np.array([1.0, 0.9, 0.5, 0.05, 0.3, 1.0], dtype=np.float32)
+    seeds, steps = np.array([1, 2, 3, 4, 5, 2**40 + 17], dtype=np.int64), np.array([0, 7, 7, 300, 1, 9], dtype=np.int32)
+    out = K.sample(dev(logits), dev(temperature), dev(top_p), dev(seeds, torch.int64), dev(steps, torch.int32)).cpu().numpy()
+
+    def uniforms(seed, step):
+        index = np.arange(vocab, dtype=np.uint64)
+        with np.errstate(over="ignore"):
+            z = np.uint64(seed) + np.uint64(0x9E3779B97F4A7C15) * np.uint64(step + 1) + np.uint64(0xD1B54A32D192ED03) * (index + np.uint64(1))
+            z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+            z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+            z = z ^ (z >> np.uint64(31))
+        return ((z >> np.uint64(40)).astype(np.float64) + 0.5) / 16777216.0
+
+    for r in range(rows):
+        row = logits[r].astype(np.float64)
+        if temperature[r] == 0:
+            assert out[r] == int(np.argmax(row))
+            continue
+        p = P.softmax(row / temperature[r])
+        # the mass of all strictly more likely tokens (the logits are all different): kept if it is
+        # below top_p (P.top_p_keep's rule, here by one sort); a token whose mass is within 1e-4 of
+        # top_p is at the nucleus' edge and may fall either way by rounding
+        order = np.argsort(-p)
+        above = np.empty(vocab)
+        above[order] = np.cumsum(p[order]) - p[order]
+        keep = above < top_p[r] if top_p[r] < 1 else np.ones(vocab, dtype=bool)
+        edge = np.abs(above - top_p[r]) < 1e-4 if top_p[r] < 1 else np.zeros(vocab, dtype=bool)
+        noisy = (row - row.max()) / temperature[r] - np.log(-np.log(uniforms(int(seeds[r]), int(steps[r]))))
+        sure = keep & ~edge
+        best_sure = noisy[sure].max()
+        assert (sure[out[r]] and noisy[out[r]] >= best_sure - 1e-3) or (edge[out[r]] and noisy[out[r]] >= best_sure - 1e-3), f"row {r}: token {out[r]}"
+
+
 def test_add(K):
     rng = np.random.default_rng(2)
     a, b = rng.standard_normal((7, 33)).astype(np.float32), rng.standard_normal((7, 33)).astype(np.float32)
