@@ -216,7 +216,8 @@ def measure_serving(dtype: str, temperature: float, step_ahead: bool = True):
         for i, prompt in enumerate(prompts):
             def emit(token, finish, i=i):
                 counts[i] += 1
-            engine.submit(Request(prompt, 256, None, emit, lambda message: None, SamplingParams(temperature=temperature, seed=i)))
+            engine.submit(Request(prompt, on_token=emit, on_error=lambda message: None, max_new_tokens=256,
+                                  sampling=SamplingParams(temperature=temperature, seed=i)))
         torch.cuda.synchronize()
         begin = time.perf_counter()
         engine.scheduler.run_until_idle()

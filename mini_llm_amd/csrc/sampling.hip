@@ -60,7 +60,9 @@ __device__ __forceinline__ float uniform_open(uint64_t seed, uint32_t step, uint
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
     z = z ^ (z >> 31);
-    return ((float)(z >> 40) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+    // 23 bits: (v + 0.5) / 2^23 with v < 2^23 is exact in 32-bit (24 significant bits hold 2v + 1) and
+    // lies in [2^-24, 1 - 2^-24]: never 0 or 1, so -log(-log(u)) is finite
+    return ((float)(z >> 41) + 0.5f) * (1.0f / 8388608.0f);
 }
 
 // One block per row. With token_slots the chosen token is also left in token_slots[slot_of_row[row]]

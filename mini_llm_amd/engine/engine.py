@@ -196,8 +196,8 @@ class Engine:
         self.close()
 
     def close(self) -> None:
-        if self.scheduler.is_running():
-            self.scheduler.stop()
+        """Whatever is still live or waiting ends with an error; its pages go back."""
+        self.scheduler.shutdown()
 
     # --- one sequence at a time (native.py) ---------------------------------------------------------
     def forward_last(self, token_ids) -> np.ndarray:
@@ -304,8 +304,8 @@ class Engine:
             def fail(message, i=i):
                 errors[i] = message
 
-            self.submit(Request(tokens, max_new_tokens, eos_token_id, emit, fail,
-                                SamplingParams(temperature=temperature, top_p=top_p, seed=seed + i)))
+            self.submit(Request(tokens, on_token=emit, on_error=fail, max_new_tokens=max_new_tokens, eos_token_id=eos_token_id,
+                                sampling=SamplingParams(temperature=temperature, top_p=top_p, seed=seed + i)))
         self.scheduler.run_until_idle()
         failed = [f"prompt {i}: {e}" for i, e in enumerate(errors) if e is not None]
         if failed:

@@ -1,26 +1,30 @@
 """Continuous batching over the step function.
 
-The reference's scheduler (pytorch/src/mini_llm/scheduler.py) admits a waiting request when a
-cache is free, prefills its whole prompt in a call of its own, and decodes all running requests
-in one batched step. This one keeps its queues, its finish reasons and their order, its error
-scopes and its statistics, and differs where the engine below differs: prompts are cut into
-portions under a token budget and run in the same step as the decodes, the currency of
-admission is pages, and a decision is made for the case that pages run out.
+What is kept of the reference's scheduler (pytorch/src/mini_llm/scheduler.py) is its behaviour:
+first come, first served; a request that finds no room keeps its place; the three reasons to
+finish and the order in which they are looked at (:185-196); the finishing token is delivered;
+an error of the engine ends every live request, a bad prompt or a failing consumer only its own
+(:131-141, :170-177, :202-211); the counters of ``stats`` (:93-102). What differs follows from the
+engine below: prompts are cut into portions under a token budget and run in the same step as the
+decodes, admission is paid in pages, and there is a decision for the case that pages run out.
+The scheduler is single-threaded: whoever calls ``step`` owns it (``engine.background`` has a
+thread for callers that want one).
 
-Every iteration (`step`):
+One iteration (``step``):
 1. cancelled requests leave;
-2. plan: running requests past their prompt bring one token each; what is left of the token
-   budget goes to prompts, first those already running, then newly admitted ones in arrival
+2. plan: live requests past their prompt bring one token each; what is left of the token
+   budget goes to prompts, first those already live, then newly admitted ones in arrival
    order (no request overtakes the head of the queue; a request is admitted when the pages for
    its whole prompt are free, though it is fed in portions);
-3. when pages run out for a running request, the request admitted last is preempted: it gives
+3. when pages run out for a live request, the request admitted last is preempted: it gives
    everything back and returns to the FRONT of the queue with its prompt extended by what it has
    generated, to be recomputed when there is room. A request that does not fit an empty pool
    fails;
 4. one step of the engine; each request whose prompt is complete gets one new token, sampled
-   on the device; `emit(token, finish)`; a finished request leaves at once and frees its pages.
+   on the device, and hears of it through ``on_token(token, finish)``; a finished request leaves
+   at once and frees its pages.
 
-One step ahead (an executor with `launch` / `collect`): the step planned in 2 is launched before
+One step ahead (an executor with ``launch`` / ``collect``): the step planned in 2 is launched before
 the tokens of the step before it have been read. A request that was sampled in the step in
 flight brings "the token in my slot" (the sampler leaves it there on the device), so planning,
 batch layout and launch of step n+1 take place while the device still runs step n, and the device
@@ -36,16 +40,15 @@ from __future__ import annotations
 
 import collections
 import logging
-import threading
-from dataclasses import dataclass, field
-from typing import Callable, Literal, Protocol
+from typing import Protocol
 
 from ..sampling import SamplingParams
 from .batch import StepEntry
 
-logger = logging.getLogger(__name__)
+log = logging.getLogger(__name__)
 
-FinishReason = Literal["stop", "length", "context"]
+# Why a request ended, in the order the checks are made.
+STOP, CONTEXT, LENGTH = "stop", "context", "length"
 
 
 class StepExecutor(Protocol):
@@ -69,36 +72,51 @@ class StepExecutor(Protocol):
     # def collect(self, handle) -> list[int]: ...
 
 
-@dataclass(eq=False)
 class Request:
-    """The reference's Request (scheduler.py:41-53) plus how to sample."""
+    """A prompt to continue and where its tokens go.
 
-    tokens: list
-    max_new_tokens: int | None
-    eos_token_id: int | None
-    # emit(token, finish): finish is None for every token but the last one.
-    emit: Callable[[int, FinishReason | None], None]
-    fail: Callable[[str], None]
-    sampling: SamplingParams = field(default_factory=SamplingParams)
-    cancelled: bool = field(default=False, init=False)
+    ``on_token(token, finish)`` is called once per generated token; ``finish`` is None except
+    with the last one, where it is "stop" (the end token came, and is delivered), "context" (the
+    model's positions are used up) or "length" (``max_new_tokens`` reached). ``on_error(message)``
+    is called instead if the request cannot run or the engine fails under it. ``max_new_tokens``
+    None: until one of the other two reasons ends it."""
+
+    __slots__ = ("prompt", "on_token", "on_error", "max_new_tokens", "eos_token_id", "sampling", "_cancelled")
+
+    def __init__(self, prompt, *, on_token, on_error, max_new_tokens=None, eos_token_id=None, sampling: SamplingParams | None = None):
+        self.prompt = prompt
+        self.on_token, self.on_error = on_token, on_error
+        self.max_new_tokens, self.eos_token_id = max_new_tokens, eos_token_id
+        self.sampling = SamplingParams() if sampling is None else sampling
+        self._cancelled = False
 
     def cancel(self) -> None:
-        self.cancelled = True
+        """May be called from any thread; the scheduler looks at it before its next step."""
+        self._cancelled = True
+
+    @property
+    def cancelled(self) -> bool:
+        return self._cancelled
 
 
-@dataclass(eq=False)  # compared by identity: membership tests must not walk every field
-class _Running:
-    request: Request
-    request_id: int
-    pending: list              # tokens not yet fed: the rest of the prompt, or the last sampled token
-    history: list = field(default_factory=list)   # tokens fed since it was (re)admitted: what its pages hold
-    generated: int = 0         # tokens delivered
-    launched: int = 0          # tokens whose sampling has been launched (= generated, or one more)
-    awaiting: bool = False     # its next token is the output of the step in flight
-    fed_ahead: bool = False    # the step in flight takes the token of the step before it from the slot
-    prompt_len: int = 0        # of the original prompt (a preempted request's recompute does not count)
-    order: int = 0             # admission order; the largest is preempted first
-    finished: bool = False
+class _Live:
+    """A request that holds pages. Compared by identity."""
+
+    __slots__ = ("request", "request_id", "pending", "history", "generated", "launched", "awaiting", "fed_ahead",
+                 "prompt_len", "order", "finished")
+
+    def __init__(self, request: Request, prompt: list):
+        self.request = request
+        self.request_id = -1
+        self.pending = prompt        # tokens not yet fed: the rest of the prompt, or the last sampled token
+        self.history = []            # tokens fed since it was (re)admitted: what its pages hold
+        self.generated = 0           # tokens delivered
+        self.launched = 0            # tokens whose sampling has been launched (= generated, or one more)
+        self.awaiting = False        # its next token is the output of the step in flight
+        self.fed_ahead = False       # the step in flight takes the token of the step before it from the slot
+        self.prompt_len = len(prompt)  # of the original prompt (a preempted request's recompute does not count)
+        self.order = 0               # admission order; the largest is preempted first
+        self.finished = False
 
 
 class _PagePlan:
@@ -115,92 +133,88 @@ class _PagePlan:
         self.taken = [t + n for t, n in zip(self.taken, need)]
 
 
-@dataclass
 class _Flight:
     """A step that has been launched and whose tokens have not been read."""
 
-    handle: object
-    sampled: list              # the _Running of each token, in the step's order
+    __slots__ = ("handle", "sampled")
+
+    def __init__(self, handle, sampled):
+        self.handle, self.sampled = handle, sampled   # sampled: the _Live of each token, in the step's order
 
 
 class _SettleFirst(Exception):
     """The plan has to preempt: the step in flight is collected first."""
 
 
+class _Tally:
+    """Running totals behind ``stats``."""
+
+    def __init__(self):
+        self.steps = self.step_tokens = 0              # every step, and the tokens it was fed
+        self.decode_steps = self.decode_rows = 0       # steps with at least one decoded token, and those tokens
+        self.delivered = self.first_tokens = 0         # tokens handed out; requests that got their first one
+        self.preemptions = self.dropped = 0
+
+
 class Scheduler:
+    NO_ROOM = "the request needs more cache pages than the pool has"
+
     def __init__(self, executor: StepExecutor, max_batch: int = 16, max_tokens_per_step: int = 2048,
                  max_prefills_per_step: int | None = None, step_ahead: bool = True):
-        if max_batch < 1 or max_tokens_per_step < 1:
-            raise ValueError("max_batch and max_tokens_per_step must be at least 1")
+        for name, value in (("max_batch", max_batch), ("max_tokens_per_step", max_tokens_per_step)):
+            if value < 1:
+                raise ValueError(f"{name} must be at least 1, not {value}")
         if max_prefills_per_step is not None and max_prefills_per_step < 1:
-            raise ValueError("max_prefills_per_step must be at least 1")
+            raise ValueError(f"max_prefills_per_step must be at least 1, not {max_prefills_per_step}")
         self._executor = executor
         self._max_batch, self._budget, self._max_prefills = max_batch, max_tokens_per_step, max_prefills_per_step
-        self._step_ahead = step_ahead and hasattr(executor, "launch") and hasattr(executor, "collect")
+        self._step_ahead = step_ahead and all(hasattr(executor, name) for name in ("launch", "collect"))
         self._in_flight: _Flight | None = None
-        self._waiting: collections.deque = collections.deque()   # Request, or _Running that was preempted
-        self._running: list[_Running] = []
-        self._wake = threading.Condition()
-        self._stopping = False
-        self._thread: threading.Thread | None = None
-        self._next_id = 0
-        self._order = 0
-        self._steps = self._decode_steps = self._tokens = self._prefills = 0
-        self._batch_sizes = self._step_tokens = self._preemptions = self._dropped_tokens = 0
+        # Request, or a _Live that was preempted. deque.append / popleft / appendleft are atomic: another
+        # thread may submit while this one steps.
+        self._queue: collections.deque = collections.deque()
+        self._live: list[_Live] = []
+        self._ids = self._admissions = 0
+        self._tally = _Tally()
+        self._closed_with: str | None = None
 
-    # --- called from other threads -------------------------------------------------------------
+    # --- the caller's side -----------------------------------------------------------------------
     def submit(self, request: Request) -> None:
-        with self._wake:
-            self._waiting.append(request)
-            self._wake.notify()
-
-    def stats(self) -> dict:
-        steps = self._decode_steps
-        return {
-            "decode_steps": steps,
-            "tokens": self._tokens,
-            "prefills": self._prefills,
-            "mean_batch_size": self._batch_sizes / steps if steps else 0.0,
-            "running": len(self._running),
-            "waiting": len(self._waiting),
-            "steps": self._steps,
-            "tokens_per_step": self._step_tokens / self._steps if self._steps else 0.0,
-            "preemptions": self._preemptions,
-            "dropped_tokens": self._dropped_tokens,   # computed past an end token nobody had seen yet
-        }
-
-    def start(self) -> None:
-        self._thread = threading.Thread(target=self._loop, name="scheduler", daemon=True)
-        self._thread.start()
-
-    def stop(self) -> None:
-        with self._wake:
-            self._stopping = True
-            self._wake.notify()
-        if self._thread is not None:
-            self._thread.join()
-        self._fail_everything("the engine is shutting down")
-
-    def is_running(self) -> bool:
-        return self._thread is not None and self._thread.is_alive()
+        if self._closed_with is not None:
+            request.on_error(self._closed_with)
+            return
+        self._queue.append(request)
 
     def has_work(self) -> bool:
-        with self._wake:
-            return bool(self._running) or bool(self._waiting) or self._in_flight is not None
+        return bool(self._live or self._queue or self._in_flight is not None)
 
     def run_until_idle(self) -> None:
         while self.step():
             pass
 
-    # --- the scheduler thread ------------------------------------------------------------------
-    def _loop(self) -> None:
-        while True:
-            with self._wake:
-                while not self._stopping and not self._running and not self._waiting and self._in_flight is None:
-                    self._wake.wait()
-                if self._stopping:
-                    return
-            self.step()
+    def shutdown(self, message: str = "the engine is shutting down") -> None:
+        """Every live and waiting request hears ``message`` as its error and gives its pages back; a
+        step in flight is forgotten; what is submitted afterwards fails at once."""
+        self._closed_with = message
+        self._abandon_live(message)
+        while self._queue:
+            item = self._queue.popleft()
+            (item.request if isinstance(item, _Live) else item).on_error(message)
+
+    def stats(self) -> dict:
+        t = self._tally
+        return {
+            "decode_steps": t.decode_steps,
+            "tokens": t.delivered,
+            "prefills": t.first_tokens,
+            "mean_batch_size": t.decode_rows / max(1, t.decode_steps),
+            "running": len(self._live),
+            "waiting": len(self._queue),
+            "steps": t.steps,
+            "tokens_per_step": t.step_tokens / max(1, t.steps),
+            "preemptions": t.preemptions,
+            "dropped_tokens": t.dropped,   # computed past an end token nobody had seen yet
+        }
 
     def step(self) -> bool:
         """One iteration. Returns False if there was nothing to do."""
@@ -216,169 +230,160 @@ class Scheduler:
             self._in_flight = launched
             if not self._step_ahead:
                 self._collect()
-        except Exception as error:  # the engine is shared: every running request is affected
-            logger.exception("engine error")
-            self._fail_running(str(error))
+        except Exception as error:
+            # the step function serves all live requests at once: none of them can go on
+            log.exception("the step failed; every live request ends with its message")
+            self._abandon_live(str(error))
             return True
         return bool(entries) or self.has_work()
 
     # --- planning ------------------------------------------------------------------------------
     def _drop_cancelled(self) -> None:
-        for running in [r for r in self._running if r.request.cancelled]:
-            self._executor.close(running.request_id)
-            self._running.remove(running)
-            running.finished = True   # a token of its that is still in flight is dropped
+        for live in [r for r in self._live if r.request.cancelled]:
+            self._executor.close(live.request_id)
+            self._live.remove(live)
+            live.finished = True   # a token of its that is still in flight is dropped
 
-    def _portion_that_fits(self, running: _Running, plan: "_PagePlan", most: int):
+    def _portion_that_fits(self, live: _Live, plan: _PagePlan, most: int):
         """(n, pages): the largest portion n <= most whose pages can be had beside what is planned
         already, and those pages per group; n = 0 if not even one token fits."""
         n = most
         while n >= 1:
-            need = self._executor.pages_needed(running.request_id, n)
+            need = self._executor.pages_needed(live.request_id, n)
             if plan.fits(need):
                 return n, need
             # shrink to the end of the page before the last one the portion touches
-            length = self._executor.length(running.request_id)
+            length = self._executor.length(live.request_id)
             page = self._executor.page_size
             n = min(n - 1, ((length + n - 1) // page) * page - length)
         return 0, None
 
-    def _preempt(self, victim: _Running) -> None:
+    def _preempt(self, victim: _Live) -> None:
         """The victim gives everything back and waits at the front of the queue; what it has been
         fed so far becomes prompt again, so that it is recomputed and goes on where it was."""
         assert not victim.awaiting, "a victim's tokens are all known"
         self._executor.close(victim.request_id)
-        self._running.remove(victim)
+        self._live.remove(victim)
         victim.pending = victim.history + victim.pending
         victim.history = []
-        self._preemptions += 1
-        with self._wake:
-            self._waiting.appendleft(victim)
+        self._tally.preemptions += 1
+        self._queue.appendleft(victim)
 
     def _plan(self):
         entries, owners = [], []
         plan = _PagePlan(self._executor.free_pages())
         budget = self._budget
         preempted = False
-        # Running requests first, in admission order: decodes bring one token, prompts a portion.
+        # Live requests first, in admission order: decodes bring one token, prompts a portion.
         # Requests are planned oldest first and preempted youngest first, so a victim never has
         # an entry in the plan yet.
-        for running in sorted(self._running, key=lambda r: r.order):
-            if running not in self._running:
+        for live in sorted(self._live, key=lambda r: r.order):
+            if live not in self._live:
                 continue  # preempted while an older request was planned
             if budget < 1:
                 break
-            if self._ends_in_flight(running):
+            if self._ends_in_flight(live):
                 continue
-            most = min(self._to_feed(running), budget)
-            n, need = self._portion_that_fits(running, plan, most)
+            most = min(self._to_feed(live), budget)
+            n, need = self._portion_that_fits(live, plan, most)
             while n == 0:
                 if self._in_flight is not None:
                     raise _SettleFirst()   # nothing has been changed so far
-                victim = max(self._running, key=lambda r: r.order)
+                victim = max(self._live, key=lambda r: r.order)
                 preempted = True
-                if victim is running:
-                    if len(self._running) == 1:
+                if victim is live:
+                    if len(self._live) == 1:
                         # alone, with every other page free, and still no room
-                        self._executor.close(running.request_id)
-                        self._running.remove(running)
-                        running.request.fail("the request needs more cache pages than the pool has")
+                        self._executor.close(live.request_id)
+                        self._live.remove(live)
+                        live.request.on_error(self.NO_ROOM)
                     else:
-                        self._preempt(running)
+                        self._preempt(live)
                     break
                 self._preempt(victim)
                 plan.free = self._executor.free_pages()
-                n, need = self._portion_that_fits(running, plan, most)
+                n, need = self._portion_that_fits(live, plan, most)
             if n == 0:
                 continue
-            self._add_entry(entries, owners, plan, running, n, need)
+            self._add_entry(entries, owners, plan, live, n, need)
             budget -= n
         # Then admissions, in arrival order; the head of the queue is never overtaken. None in a
         # step that had to preempt: the preempted request would come straight back.
         admitted = 0
-        while not preempted and budget >= 1 and len(self._running) < self._max_batch:
+        while not preempted and budget >= 1 and len(self._live) < self._max_batch and self._queue:
             if self._max_prefills is not None and admitted >= self._max_prefills:
                 break
-            item = self._pop_waiting()
-            if item is None:
-                break
-            running = self._admit(item, plan, bool(entries))
-            if running is None:
+            item = self._queue.popleft()
+            live = self._admit(item, plan, bool(entries))
+            if live is None:
                 continue          # cancelled or failed: the next one gets its turn
-            if running is False:
-                self._push_front(item)
-                break             # no room yet: wait for a running request to end
-            n, need = self._portion_that_fits(running, plan, min(len(running.pending), budget))
-            self._add_entry(entries, owners, plan, running, n, need)
+            if live is False:
+                self._queue.appendleft(item)
+                break             # no room yet: wait for a live request to end
+            n, need = self._portion_that_fits(live, plan, min(len(live.pending), budget))
+            self._add_entry(entries, owners, plan, live, n, need)
             budget -= n
             admitted += 1
         return entries, owners
 
     @staticmethod
-    def _to_feed(running: _Running) -> int:
-        return 1 if running.awaiting else len(running.pending)
+    def _to_feed(live: _Live) -> int:
+        return 1 if live.awaiting else len(live.pending)
 
-    def _ends_in_flight(self, running: _Running) -> bool:
+    def _ends_in_flight(self, live: _Live) -> bool:
         """The token being sampled in the step in flight is this request's last, whatever it is."""
-        if not running.awaiting:
+        if not live.awaiting:
             return False
-        request, limit = running.request, self._executor.max_positions()
-        return ((limit is not None and running.prompt_len + running.launched >= limit)
-                or (request.max_new_tokens is not None and running.launched >= request.max_new_tokens))
+        request, limit = live.request, self._executor.max_positions()
+        return ((limit is not None and live.prompt_len + live.launched >= limit)
+                or (request.max_new_tokens is not None and live.launched >= request.max_new_tokens))
 
-    def _add_entry(self, entries, owners, plan, running, n, need) -> None:
-        if running.awaiting:
-            entry = StepEntry(running.request_id, [0], [0], from_slot=True)
+    def _add_entry(self, entries, owners, plan, live, n, need) -> None:
+        if live.awaiting:
+            entry = StepEntry(live.request_id, [0], [0], from_slot=True)
         else:
-            completes = n == len(running.pending)
-            entry = StepEntry(running.request_id, list(running.pending[:n]), [n - 1] if completes else [])
+            completes = n == len(live.pending)
+            entry = StepEntry(live.request_id, list(live.pending[:n]), [n - 1] if completes else [])
         entries.append(entry)
-        owners.append(running)
+        owners.append(live)
         plan.take(need)
 
     def _admit(self, item, plan, others_planned: bool):
-        """None: the request is gone (cancelled / failed). False: no room now. Else the _Running."""
-        request = item.request if isinstance(item, _Running) else item
+        """None: the request is gone (cancelled / failed). False: no room now. Else the _Live."""
+        request = item.request if isinstance(item, _Live) else item
         if request.cancelled:
             return None
-        if isinstance(item, _Running):
-            running = item
+        if isinstance(item, _Live):
+            live = item
         else:
             try:
-                if not request.tokens:
+                prompt = list(request.prompt)
+                if not prompt:
                     raise ValueError("the prompt has no tokens")
-                self._executor.check_prompt(list(request.tokens))
-            except Exception as error:  # a bad prompt is the problem of this request only
-                logger.warning("request refused: %s", error)
-                request.fail(str(error))
+                self._executor.check_prompt(prompt)
+            except Exception as error:
+                log.warning("a request was refused at admission: %s", error)
+                request.on_error(str(error))   # nobody else is touched by a prompt that cannot run
                 return None
-            running = _Running(request, -1, list(request.tokens), prompt_len=len(request.tokens))
+            live = _Live(request, prompt)
         if not self._executor.can_open():
             return False
-        request_id = self._next_id
+        request_id = self._ids
         self._executor.open(request_id)
         # Admitted only if its whole prompt has room beside what is planned: a request that could
         # take a first portion and then stall would only be preempted again.
-        if not plan.fits(self._executor.pages_needed(request_id, len(running.pending))):
+        if not plan.fits(self._executor.pages_needed(request_id, len(live.pending))):
             self._executor.close(request_id)
-            if not self._running and not others_planned:
-                request.fail("the request needs more cache pages than the pool has")
+            if not self._live and not others_planned:
+                request.on_error(self.NO_ROOM)
                 return None
             return False
-        self._next_id += 1
-        running.request_id = request_id
-        running.order = self._order
-        self._order += 1
-        self._running.append(running)
-        return running
-
-    def _pop_waiting(self):
-        with self._wake:
-            return self._waiting.popleft() if self._waiting else None
-
-    def _push_front(self, item) -> None:
-        with self._wake:
-            self._waiting.appendleft(item)
+        self._ids += 1
+        live.request_id = request_id
+        live.order = self._admissions
+        self._admissions += 1
+        self._live.append(live)
+        return live
 
     # --- running and delivering ----------------------------------------------------------------
     def _launch(self, entries, owners) -> _Flight:
@@ -389,12 +394,13 @@ class Scheduler:
             handle = self._executor.launch(entries, sampling, steps)
         else:
             handle = self._executor.run(entries, sampling, steps)
-        self._steps += 1
-        self._step_tokens += sum(len(e.tokens) for e in entries)
+        tally = self._tally
+        tally.steps += 1
+        tally.step_tokens += sum(len(e.tokens) for e in entries)
         decodes = sum(1 for o, e in zip(owners, entries) if o.launched > 0 and len(e.tokens) == 1)
         if decodes:
-            self._decode_steps += 1
-            self._batch_sizes += decodes
+            tally.decode_steps += 1
+            tally.decode_rows += decodes
         for owner, entry in zip(owners, entries):
             if entry.from_slot:
                 owner.fed_ahead = True     # the token joins its history when it is known
@@ -414,11 +420,10 @@ class Scheduler:
         tokens = self._executor.collect(flight.handle) if self._step_ahead else flight.handle
         for owner, token in zip(flight.sampled, tokens):
             if owner.finished:
-                self._dropped_tokens += 1
+                self._tally.dropped += 1
                 continue
             token = int(token)
-            if owner.generated == 0:
-                self._prefills += 1
+            self._tally.first_tokens += owner.generated == 0
             owner.generated += 1
             if owner.fed_ahead:            # the step launched after this one has been fed it already
                 owner.history.append(token)
@@ -426,47 +431,40 @@ class Scheduler:
             else:
                 owner.awaiting = False
                 owner.pending = [token]
-            self._deliver(owner, token)
-        self._running = [r for r in self._running if not r.finished]
+            self._hand_over(owner, token)
+        self._live = [r for r in self._live if not r.finished]
 
-    def _finish_reason(self, running: _Running, token: int) -> FinishReason | None:
-        # the order of the reference's checks (scheduler.py:185-196)
-        request = running.request
-        if request.eos_token_id is not None and token == request.eos_token_id:
-            return "stop"
-        limit = self._executor.max_positions()
-        if limit is not None and running.prompt_len + running.generated >= limit:
-            return "context"
-        if request.max_new_tokens is not None and running.generated >= request.max_new_tokens:
-            return "length"
-        return None
+    def _ending(self, live: _Live, token: int):
+        """The reason this token ends its request, or None. First match wins:
+        end token, then positions used up, then the request's own limit."""
+        request, positions = live.request, self._executor.max_positions()
+        checks = (
+            (STOP, request.eos_token_id is not None and token == request.eos_token_id),
+            (CONTEXT, positions is not None and live.prompt_len + live.generated >= positions),
+            (LENGTH, request.max_new_tokens is not None and live.generated >= request.max_new_tokens),
+        )
+        return next((reason for reason, holds in checks if holds), None)
 
-    def _deliver(self, running: _Running, token: int) -> None:
-        """Hands one token to its request. If that ends the request, its pages are given back."""
-        reason = self._finish_reason(running, token)
-        self._tokens += 1
+    def _hand_over(self, live: _Live, token: int) -> None:
+        """One token to its request; if it is the last one, the pages go back now."""
+        ending = self._ending(live, token)
+        self._tally.delivered += 1
         try:
-            running.request.emit(token, reason)
+            live.request.on_token(token, ending)
         except Exception:
-            # The consumer is gone. That is the problem of this request only.
-            logger.exception("emit failed, dropping the request")
-            reason = "stop"
-        if reason is not None:
-            self._executor.close(running.request_id)
-            running.finished = True
+            log.exception("on_token raised: this request alone is dropped")
+            ending = ending or STOP
+        if ending is not None:
+            live.finished = True
+            self._executor.close(live.request_id)
 
-    def _fail_running(self, message: str) -> None:
-        running, self._running = self._running, []
-        self._in_flight = None
-        for item in running:
-            item.finished = True
+    def _abandon_live(self, message: str) -> None:
+        """Every live request ends with ``message``; the step in flight is forgotten."""
+        abandoned, self._live, self._in_flight = self._live, [], None
+        for live in abandoned:
+            live.finished = True
             try:
-                self._executor.close(item.request_id)
+                self._executor.close(live.request_id)
             except Exception:
-                logger.exception("closing a request after an engine error failed")
-            item.request.fail(message)
-
-    def _fail_everything(self, message: str) -> None:
-        self._fail_running(message)
-        while (item := self._pop_waiting()) is not None:
-            (item.request if isinstance(item, _Running) else item).fail(message)
+                log.exception("a request's pages could not be given back after the step failed")
+            live.request.on_error(message)

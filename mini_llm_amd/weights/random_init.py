@@ -8,24 +8,21 @@ from pathlib import Path
 
 import torch
 
+from .counter_rng import normal_tensor
 from .safetensors_io import write_safetensors
 from .spec import INT_TABLE
 
 
 def random_tensors(model, seed: int, dtype: torch.dtype = torch.float32) -> dict:
-    """name -> CPU tensor in the stored layout. One generator, tensors in sorted-name order, so
-    the result depends on the seed and the configuration alone."""
-    generator = torch.Generator(device="cpu")
-    generator.manual_seed(int(seed))
+    """name -> CPU tensor in the stored layout. Every element is a function of (seed, the tensor's
+    name, its index in the tensor) alone (``counter_rng``): the same seed gives the same model
+    whatever the order of the tensors, the installed libraries or the language of whoever draws it."""
     out = {}
-    specs = model.named_tensor_specs()
-    for name in sorted(specs):
-        spec = specs[name]
+    for name, spec in model.named_tensor_specs().items():
         if spec.role == INT_TABLE:
             raise ValueError(f"{name}: no random recipe for integer tables")
-        values = torch.empty(spec.shape, dtype=torch.float32)
-        values.normal_(spec.init.mean, spec.init.std, generator=generator)
-        out[name] = values.to(dtype)
+        values = normal_tensor(int(seed), name, tuple(spec.shape), spec.init.mean, spec.init.std)
+        out[name] = torch.from_numpy(values).to(dtype)
     return out
 
 

@@ -306,3 +306,46 @@ def random_weights(config: dict, seed: int) -> dict:
     w["ln_f.weight"] = n((d,), 0.05, 1.0)
     w["ln_f.bias"] = n((d,), 0.02)
     return w
+
+
+# --- the framework's documented random-weights generator, written out a second time -----------------
+# (its definition: mini_llm_amd/weights/counter_rng.py's docstring; integers here are Python's own)
+def counter_normal(seed: int, name: str, count: int) -> np.ndarray:
+    """n(0) .. n(count - 1) of tensor ``name`` under ``seed``, float64."""
+    m = (1 << 64) - 1
+
+    def mix(z):
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+        return z ^ (z >> 31)
+
+    h = 0xCBF29CE484222325
+    for byte in name.encode("utf-8"):
+        h = ((h ^ byte) * 0x100000001B3) & m
+    key = mix(mix(seed & m) ^ h)
+    g = 0x9E3779B97F4A7C15
+    a = np.array([mix((key + (2 * i + 1) * g) & m) >> 12 for i in range(count)], dtype=np.float64)
+    b = np.array([mix((key + (2 * i + 2) * g) & m) >> 12 for i in range(count)], dtype=np.float64)
+    u1, u2 = (a + 0.5) / 2.0**52, (b + 0.5) / 2.0**52
+    return np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+
+
+def counter_random_weights(config: dict, seed: int) -> dict:
+    """The tensors the framework's random-weights mode writes for this configuration and seed."""
+    d, L, V, P = config["n_embd"], config["n_layer"], config["vocab_size"], config["n_positions"]
+    ff = config.get("n_inner") or 4 * d
+    proj_std = 0.02 / math.sqrt(2 * L)
+    recipe = {"wte.weight": ((V, d), 0.0, 0.02), "wpe.weight": ((P, d), 0.0, 0.02),
+              "ln_f.weight": ((d,), 1.0, 0.05), "ln_f.bias": ((d,), 0.0, 0.02)}
+    for i in range(L):
+        p = f"h.{i}."
+        recipe.update({
+            p + "ln_1.weight": ((d,), 1.0, 0.05), p + "ln_1.bias": ((d,), 0.0, 0.02),
+            p + "attn.c_attn.weight": ((d, 3 * d), 0.0, 0.02), p + "attn.c_attn.bias": ((3 * d,), 0.0, 0.01),
+            p + "attn.c_proj.weight": ((d, d), 0.0, proj_std), p + "attn.c_proj.bias": ((d,), 0.0, 0.01),
+            p + "ln_2.weight": ((d,), 1.0, 0.05), p + "ln_2.bias": ((d,), 0.0, 0.02),
+            p + "mlp.c_fc.weight": ((d, ff), 0.0, 0.02), p + "mlp.c_fc.bias": ((ff,), 0.0, 0.01),
+            p + "mlp.c_proj.weight": ((ff, d), 0.0, proj_std), p + "mlp.c_proj.bias": ((d,), 0.0, 0.01),
+        })
+    return {name: (mean + std * counter_normal(seed, name, int(np.prod(shape)))).astype(np.float32).reshape(shape)
+            for name, (shape, mean, std) in recipe.items()}

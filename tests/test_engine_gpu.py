@@ -64,7 +64,7 @@ def host_uniform(seed, step, index):
     z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
     z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
     z = z ^ (z >> 31)
-    return ((z >> 40) + 0.5) / 16777216.0
+    return float((np.float32(z >> 41) + np.float32(0.5)) * np.float32(1.0 / 8388608.0))   # 23 bits, in 32-bit like the kernel
 
 
 def test_temperature_sampling_in_chunks_beside_decodes(model_dirs, engines):
@@ -367,8 +367,8 @@ def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dt
             for i, prompt in enumerate(prompts):
                 def emit(token, finish, i=i):
                     outputs[i].append((token, finish))
-                engine.submit(Request(prompt, 24, ends[i], emit, errors.append,
-                                      SamplingParams(temperature=temperature, seed=31 + i)))
+                engine.submit(Request(prompt, on_token=emit, on_error=errors.append, max_new_tokens=24, eos_token_id=ends[i],
+                                      sampling=SamplingParams(temperature=temperature, seed=31 + i)))
             before = engine.stats()
             engine.scheduler.run_until_idle()
             after = engine.stats()
@@ -419,7 +419,8 @@ def test_random_workloads_through_the_scheduler_match_plain_greedy(model_dirs, e
 
     together, errors = [[] for _ in prompts], []
     for i, (prompt, n) in enumerate(zip(prompts, new)):
-        engine.submit(Request(prompt, n, None, lambda token, finish, i=i: together[i].append(token), errors.append))
+        engine.submit(Request(prompt, on_token=lambda token, finish, i=i: together[i].append(token), on_error=errors.append,
+                              max_new_tokens=n))
     engine.scheduler.run_until_idle()
     assert not errors
     assert engine.stats()["preemptions"] > before   # the pool is that small

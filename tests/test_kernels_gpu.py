@@ -526,7 +526,7 @@ def test_draws_over_the_whole_vocabulary_are_the_generators(K):
             z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
             z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
             z = z ^ (z >> np.uint64(31))
-        return ((z >> np.uint64(40)).astype(np.float64) + 0.5) / 16777216.0
+        return (((z >> np.uint64(41)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 8388608.0)).astype(np.float64)   # in 32-bit like the kernel
 
     for r in range(rows):
         row = logits[r].astype(np.float64)

@@ -8,6 +8,7 @@ import time
 import pytest
 
 from mini_llm_amd.cache import CacheManager
+from mini_llm_amd.engine.background import SchedulerThread
 from mini_llm_amd.engine.scheduler import Request, Scheduler
 from mini_llm_amd.models.base import CacheGroupSpec
 from mini_llm_amd.sampling import SamplingParams
@@ -94,7 +95,7 @@ class Sink:
 
 def submit(scheduler, prompt, max_new=4, eos=None, **kw):
     sink = Sink()
-    request = Request(list(prompt), max_new, eos, sink.emit, sink.fail, **kw)
+    request = Request(list(prompt), on_token=sink.emit, on_error=sink.fail, max_new_tokens=max_new, eos_token_id=eos, **kw)
     scheduler.submit(request)
     return sink, request
 
@@ -271,7 +272,7 @@ def test_a_raising_callback_drops_only_its_request():
     good, _ = submit(s, [100], max_new=3)
     def boom(token, finish):
         raise RuntimeError("consumer gone")
-    s.submit(Request([200], 3, None, boom, lambda m: None))
+    s.submit(Request([200], on_token=boom, on_error=lambda m: None, max_new_tokens=3))
     s.run_until_idle()
     assert good.tokens == [101, 102, 103] and ex.all_free()
     assert sum(1 for step in ex.steps for r, _, _ in step if r == 1) == 1
@@ -305,19 +306,31 @@ def test_stats():
 
 def test_thread_idles_processes_and_stops():
     ex = FakeExecutor()
-    s = Scheduler(ex, max_batch=1)
+    s = SchedulerThread(Scheduler(ex, max_batch=1))
     s.start()
     assert s.is_running()
+    with pytest.raises(RuntimeError):
+        s.start()
     sink, _ = submit(s, [100], max_new=3)
     deadline = time.time() + 5
     while sink.finish is None and time.time() < deadline:
         time.sleep(0.01)
     assert sink.tokens == [101, 102, 103]
     s.stop()
-    assert not s.is_running()
-    late, _ = submit(s, [200])
-    s.stop()
+    assert not s.is_running() and ex.all_free()
+    late, _ = submit(s, [200])                     # after the end: refused at once
     assert late.error is not None and "shutting down" in late.error
+
+
+def test_shutdown_fails_what_is_live_and_what_waits():
+    ex = FakeExecutor()
+    s = Scheduler(ex, max_batch=1)
+    live, _ = submit(s, [100], max_new=5)
+    waiting, _ = submit(s, [200], max_new=5)
+    s.step()
+    s.shutdown("closing")
+    assert live.tokens == [101] and live.error == "closing" and waiting.error == "closing" and waiting.tokens == []
+    assert ex.all_free() and not s.has_work() and s.step() is False
 
 
 def test_options_are_checked():
@@ -473,7 +486,8 @@ def test_step_ahead_can_be_switched_off():
 
 def test_thread_runs_one_step_ahead_and_stops_with_a_step_in_flight():
     ex = AheadExecutor()
-    s = Scheduler(ex, max_batch=2)
+    scheduler = Scheduler(ex, max_batch=2)
+    s = SchedulerThread(scheduler)
     s.start()
     sinks = [submit(s, [100 * (i + 1)], max_new=5, eos=(203 if i == 1 else None))[0] for i in range(3)]
     deadline = time.time() + 5
@@ -482,9 +496,9 @@ def test_thread_runs_one_step_ahead_and_stops_with_a_step_in_flight():
     assert [x.tokens for x in sinks] == [[101, 102, 103, 104, 105], [201, 202, 203], [301, 302, 303, 304, 305]]
     assert [x.finish for x in sinks] == ["length", "stop", "length"]
     deadline = time.time() + 5
-    while s.has_work() and time.time() < deadline:   # the token past the end token is collected and dropped
+    while scheduler.has_work() and time.time() < deadline:   # the token past the end token is collected and dropped
         time.sleep(0.01)
-    assert ex.all_free() and ex.launched_ahead > 0 and s.stats()["dropped_tokens"] == 1
+    assert ex.all_free() and ex.launched_ahead > 0 and scheduler.stats()["dropped_tokens"] == 1
     slow_collect = ex.collect
     ex.collect = lambda handle: (time.sleep(0.01), slow_collect(handle))[1]
     endless, _ = submit(s, [400], max_new=None)                       # 63 tokens at 10 ms each

@@ -147,3 +147,46 @@ def test_random_weights_mode_writes_a_folder_the_loader_reads(tmp_path):
     write_model_dir(config, 7, tmp_path / "bf", dtype="bfloat16")
     f = SafetensorsFile(tmp_path / "bf" / "model.safetensors")
     assert f.dtype("wte.weight") == torch.bfloat16 and f.shape("wte.weight") == (1000, 96)
+
+
+def test_random_weights_are_the_documented_counter_based_draws(tmp_path):
+    """Every element is a function of (seed, tensor name, element index): the framework's folder
+    equals, bit for bit, what the plain implementation's own copy of the generator draws; a
+    tensor's numbers do not depend on its shape's split, and a few values are pinned."""
+    from mini_llm_amd.weights.counter_rng import normal_tensor, tensor_key
+
+    for raw, seed in ((TINY_A, 0), (TINY_B, 7)):
+        folder = tmp_path / f"m{seed}"
+        write_model_dir(config_from_dict(raw), seed, folder)
+        _, written = plain_gpt2.load_model_dir(folder)
+        twin = plain_gpt2.counter_random_weights(raw, seed)
+        assert sorted(written) == sorted(twin)
+        for name in twin:
+            assert written[name].dtype == np.float32
+            np.testing.assert_array_equal(written[name], twin[name], err_msg=name)
+    # element i is the same whether asked for alone, in a longer tensor, or across a chunk border
+    long = normal_tensor(3, "t", (300_000,))
+    np.testing.assert_array_equal(long[:7], normal_tensor(3, "t", (7,)))
+    np.testing.assert_array_equal(long.reshape(3, 100_000)[2], long[200_000:])
+    np.testing.assert_array_equal(long[131_070:131_075], plain_gpt2.counter_normal(3, "t", 131_075)[131_070:].astype(np.float32))
+    # name and seed both decide
+    assert not np.array_equal(long[:7], normal_tensor(3, "u", (7,))) and not np.array_equal(long[:7], normal_tensor(4, "t", (7,)))
+    # pinned: the integer part exactly, the values to the last bit of float32
+    assert tensor_key(5, "wte.weight") == plain_key(5, "wte.weight") == 0xF103BFA14EA3A977
+    bits = lambda *a: [int(v) for v in normal_tensor(*a).view(np.uint32)]
+    assert bits(5, "wte.weight", (4,), 0.0, 0.02) == [0xBC4D3DD8, 0x3C783C2F, 0x3CBA8C95, 0xBBFEB98D]   # -0.0125269, 0.0151511, 0.0227721, -0.0077736
+    assert bits(0, "ln_f.bias", (4,), 1.0, 0.05) == [0x3F70A79D, 0x3F866C6B, 0x3F82D16B, 0x3F89BB6E]    # 0.9400576, 1.0501837, 1.0220159, 1.0760324
+    draws = normal_tensor(11, "h.0.mlp.c_fc.weight", (1000, 1000))
+    assert abs(draws.mean()) < 3e-3 and abs(draws.std() - 1.0) < 3e-3 and abs((draws**4).mean() - 3.0) < 0.05   # normal, not merely centred
+
+
+def plain_key(seed, name):
+    m = (1 << 64) - 1
+    h = 0xCBF29CE484222325
+    for byte in name.encode():
+        h = ((h ^ byte) * 0x100000001B3) & m
+    def mix(z):
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+        return z ^ (z >> 31)
+    return mix(mix(seed & m) ^ h)
