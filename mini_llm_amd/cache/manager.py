@@ -30,6 +30,7 @@ class RequestCache:
     tables: list = field(default_factory=list)        # per group: page of each block (NO_PAGE once given back)
     state_slot: int = NO_PAGE
     reserved: int = 0                                 # tokens beyond ``length`` that have pages
+    token_in_slot: bool = False                       # a sampler has left a token in the last-token slot since admission
 
 
 class CacheManager:
@@ -98,6 +99,15 @@ class CacheManager:
 
     def length(self, request_id) -> int:
         return self._entry(request_id).length
+
+    def note_sampled(self, request_id) -> None:
+        """A sampler has been launched that leaves this request's token in its last-token slot."""
+        self._entry(request_id).token_in_slot = True
+
+    def has_sampled_token(self, request_id) -> bool:
+        """Whether the request's last-token slot holds a token of its own (a slot keeps what its
+        previous owner left until the new owner is sampled for the first time)."""
+        return self._entry(request_id).token_in_slot
 
     def _entry(self, request_id) -> RequestCache:
         try:

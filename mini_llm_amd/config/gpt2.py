@@ -10,6 +10,7 @@ from dataclasses import dataclass
 
 from .base import ConfigError, ModelConfig, take_float, take_int
 
+MAX_HEAD_SIZE = 256  # the widest head the attention kernels take (parts.attention.MAX_HEAD_SIZE)
 ACTIVATIONS = ("gelu_new", "gelu")  # tanh form / exact erf form (engine/src/gelu.c:5-20)
 
 
@@ -35,6 +36,9 @@ class GPT2Config(ModelConfig):
         n_head = take_int(raw, "n_head", 12)
         if n_embd % n_head:
             raise ConfigError(f"n_embd={n_embd} is not divisible by n_head={n_head}")
+        if n_embd // n_head > MAX_HEAD_SIZE:
+            raise ConfigError(f"heads of {n_embd // n_head} (n_embd={n_embd} / n_head={n_head}) are wider than the attention kernels take: "
+                              f"any size from 1 to {MAX_HEAD_SIZE} runs")
         # n_inner null or absent means four times the width (scripts/dump_reference.py:57)
         n_inner = raw.get("n_inner")
         n_inner = 4 * n_embd if n_inner is None else take_int(raw, "n_inner")

@@ -30,6 +30,7 @@ class EngineOptions:
     max_tokens: int | None = None        # cache capacity in tokens; None: max_sessions full contexts
     cache_gib: float | None = None       # or the capacity as memory: GiB of page pools (an MI355X has 288 GB to give)
     page_size: int = DEFAULT_PAGE_SIZE
+    max_length: int | None = None        # longest sequence, for a model without a position limit of its own
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
     use_graphs: bool = True              # replay decode steps from captured HIP graphs
     step_ahead: bool = True              # the scheduler launches a step before it has read the one before
@@ -45,7 +46,8 @@ class _Executor:
         self._hosts, self._turn = [], 0
 
     def max_positions(self):
-        return self._engine.model.max_positions()
+        """The model's own limit, else the longest sequence the cache was made for."""
+        return self._engine.model.max_positions() or self._engine.cache.max_length
 
     def check_prompt(self, tokens):
         limit, vocab = self.max_positions(), self._engine.model.vocab_size
@@ -98,6 +100,9 @@ class _Executor:
         n = logits.shape[0]
         tokens = engine.sampler.sample(logits, sampling, steps, token_slots=engine.cache.last_token,
                                        slot_of_row=engine.runner.last_batch.logit_slots)
+        for entry in entries:
+            if entry.want:
+                engine.cache.note_sampled(entry.request_id)
         if not self._hosts or self._hosts[0].shape[0] < n:
             size = max(n, engine.options.max_sessions)
             self._hosts = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
@@ -156,22 +161,32 @@ class Engine:
     def __init__(self, model_dir=None, options: EngineOptions = EngineOptions(), *, model=None):
         """model_dir: folder with config.json and model.safetensors. ``model``: an already
         loaded model instead (see ``from_random``)."""
+        import torch
+
         from ..ops import library
         from ..sampling import Sampler
 
         library()  # fails loudly here if the kernels are missing
         self.options = options
         self.model = model if model is not None else load_model(model_dir, options.dtype, options.device)
-        limit = self.model.max_positions() or 4096
+        # the longest sequence a request may reach: the model's own limit, else the caller's
+        limit = self.model.max_positions() or options.max_length
         if options.max_tokens is not None and options.cache_gib is not None:
             raise ValueError("give the cache's capacity as max_tokens or as cache_gib, not both")
         if options.cache_gib is not None:
-            element_size = 2 if options.dtype == "bfloat16" else 4
+            element_size = torch.empty((), dtype=self.model.precision.compute).element_size()
             max_tokens = tokens_for_memory(self.model.cache_groups(), element_size, options.cache_gib, options.page_size)
+        elif options.max_tokens is not None:
+            max_tokens = options.max_tokens
+        elif limit is not None:
+            max_tokens = options.max_sessions * limit
         else:
-            max_tokens = options.max_tokens or options.max_sessions * limit
+            raise ValueError("this model has no position limit of its own: size the cache with max_tokens or cache_gib, "
+                             "or give max_length")
+        if limit is None:
+            limit = max_tokens   # one request may fill the whole cache, never more
         self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
-                                max_requests=options.max_sessions, device=options.device)
+                                max_requests=options.max_sessions, device=options.device, max_length=limit)
         self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs)
         self.sampler = Sampler(self.runner.staging)
         self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step,
@@ -224,23 +239,27 @@ class Engine:
     def release_cache(self, handle) -> None:
         self.cache.close(handle)
 
-    def _greedy(self, logits, n: int):
+    def _greedy(self, logits, handles):
         """argmax per row on the device; each token is also left in its request's last-token slot."""
-        return self.sampler.sample(logits, [SamplingParams()] * n, [0] * n, token_slots=self.cache.last_token,
-                                   slot_of_row=self.runner.last_batch.state_slots)
+        n = len(handles)
+        tokens = self.sampler.sample(logits, [SamplingParams()] * n, [0] * n, token_slots=self.cache.last_token,
+                                     slot_of_row=self.runner.last_batch.state_slots)
+        for handle in handles:
+            self.cache.note_sampled(handle)
+        return tokens
 
     def prefill_greedy(self, handle, token_ids) -> int:
         tokens = [int(t) for t in token_ids]
         if not tokens:
             raise RuntimeError("the prompt has no tokens")
         logits = self.runner.step([StepEntry(handle, tokens, [len(tokens) - 1])])
-        return int(self._greedy(logits, 1).cpu()[0])
+        return int(self._greedy(logits, [handle]).cpu()[0])
 
     def decode_batch(self, handles, tokens) -> list[int]:
         if len(handles) != len(tokens) or not handles:
             raise RuntimeError("a batch has one token per sequence and at least one sequence")
         logits = self.runner.step([StepEntry(h, [int(t)], [0]) for h, t in zip(handles, tokens)])
-        return self._greedy(logits, len(handles)).cpu().tolist()
+        return self._greedy(logits, list(handles)).cpu().tolist()
 
     # --- queued decoding: step n+1 is launched before the host has read token n ------------------------
     # (the reference's enqueue / take: engine/src/gpt2_gpu_greedy.cu:80-123, native.py:123-155)
@@ -257,7 +276,7 @@ class Engine:
         if len(self._queued) >= self.MAX_QUEUED:
             raise RuntimeError(f"{self.MAX_QUEUED} steps are queued already: take one first")
         logits = self.runner.step([StepEntry(h, [0], [0], from_slot=True) for h in handles])
-        tokens = self._greedy(logits, len(handles))
+        tokens = self._greedy(logits, list(handles))
         if len(self._token_buffers) < self.MAX_QUEUED:
             self._token_buffers.append(torch.empty(self.options.max_sessions, dtype=torch.int32, pin_memory=True))
         host = self._token_buffers[self._queue_turn % self.MAX_QUEUED]

@@ -57,10 +57,13 @@ def tokens_for_memory(groups, element_size: int, gib: float, page_size: int) -> 
     return tokens
 
 
-def make_cache(model, *, max_tokens: int, page_size: int = DEFAULT_PAGE_SIZE, max_requests: int = 256, device="cuda:0"):
-    """A cache whose every group holds ``max_tokens`` tokens' worth of pages."""
+def make_cache(model, *, max_tokens: int, page_size: int = DEFAULT_PAGE_SIZE, max_requests: int = 256, device="cuda:0",
+               max_length: int | None = None):
+    """A cache whose every group holds ``max_tokens`` tokens' worth of pages. ``max_length``: the
+    longest sequence of one request (it sets the width of the block tables); by default the
+    model's own position limit."""
     num_pages = max(1, -(-max_tokens // page_size))
     return CacheManager(
         model.cache_groups(), model.state_needs(), num_pages=num_pages, page_size=page_size, max_requests=max_requests,
-        dtype=model.precision.compute, device=device, max_length=model.max_positions(),
+        dtype=model.precision.compute, device=device, max_length=max_length if max_length is not None else model.max_positions(),
     )

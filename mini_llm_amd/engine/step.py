@@ -108,6 +108,8 @@ class ModelRunner:
                 raise StepError(f"request {entry.request_id!r} brings no tokens")
             if entry.from_slot and n != 1:
                 raise StepError(f"request {entry.request_id!r}: only a single token can come from the last-token slot")
+            if entry.from_slot and not self.cache.has_sampled_token(entry.request_id):
+                raise StepError(f"request {entry.request_id!r}: no token has been sampled into its last-token slot yet")
             if not entry.from_slot:
                 self._check_tokens(entry, vocab)
             length = self.cache.length(entry.request_id)

@@ -17,6 +17,13 @@ from .linear import Linear
 from .norms import LayerNorm
 
 
+# The widest head any attention kernel takes (the general kernel keeps a head's output in four
+# registers a lane). Heads of 16 to 128 in steps of 16 take the matrix-core kernel in prompt
+# portions and powers of two the split-key kernel in decoding; every other size runs through the
+# general kernel, a wave per (token, head).
+MAX_HEAD_SIZE = 256
+
+
 class CausalSelfAttention(Mixer):
     graph_safe = True
 
@@ -27,8 +34,8 @@ class CausalSelfAttention(Mixer):
         self.head_size = width // n_heads if head_size is None else head_size
         if self.n_heads % self.n_kv_heads:
             raise ValueError(f"{n_heads} heads do not divide into {self.n_kv_heads} key/value heads")
-        if self.head_size % 16 or not 16 <= self.head_size <= 256:
-            raise ValueError(f"head size {self.head_size} is not a multiple of 16 in 16..256")
+        if not 1 <= self.head_size <= MAX_HEAD_SIZE:
+            raise ValueError(f"head size {self.head_size} is not in 1..{MAX_HEAD_SIZE}")
         self.window = window
         self.scale = 1.0 / math.sqrt(self.head_size)
         self.q_width = self.n_heads * self.head_size

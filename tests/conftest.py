@@ -59,7 +59,37 @@ TINY_C = {
     "activation_function": "gelu_new",
     "tie_word_embeddings": True,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 8)}
+# Sizes no kernel's fast path takes: heads of 14 (no multiple of 16), a width and hidden units that
+# are no multiple of four, an odd vocabulary.
+TINY_D = {
+    "architectures": ["GPT2LMHeadModel"],
+    "model_type": "gpt2",
+    "n_layer": 2,
+    "n_embd": 42,
+    "n_head": 3,
+    "n_inner": 75,
+    "vocab_size": 301,
+    "n_positions": 96,
+    "layer_norm_epsilon": 2e-5,
+    "activation_function": "gelu",
+    "tie_word_embeddings": True,
+}
+# Heads of 24 and hidden units that are a multiple of four but not of eight: the down product's K is
+# a whole number of 16-byte pieces in 32-bit and not in bfloat16.
+TINY_E = {
+    "architectures": ["GPT2LMHeadModel"],
+    "model_type": "gpt2",
+    "n_layer": 3,
+    "n_embd": 72,
+    "n_head": 3,
+    "n_inner": 100,
+    "vocab_size": 409,
+    "n_positions": 160,
+    "layer_norm_epsilon": 1e-5,
+    "activation_function": "gelu_new",
+    "tie_word_embeddings": True,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 8), "D": (TINY_D, 11), "E": (TINY_E, 12)}
 
 
 def sharpen_attention(weights: dict, config: dict, factor: float = 8.0) -> None:

@@ -185,3 +185,18 @@ def test_capacity_from_memory():
         tokens_for_memory(small, 4, 1e-6, 64)
     with pytest.raises(ValueError):
         tokens_for_memory([], 4, 1.0, 64)
+
+
+def test_a_slot_says_whether_its_own_request_has_been_sampled():
+    # the last-token slot keeps what its previous owner left: a new owner has no token there until a sampler says so
+    from mini_llm_amd.cache import CacheManager
+    from mini_llm_amd.models.base import CacheGroupSpec
+
+    cache = CacheManager([CacheGroupSpec("full", (0,), 1, 16, None)], {}, num_pages=4, page_size=4, max_requests=1)
+    cache.open("a")
+    assert not cache.has_sampled_token("a")
+    cache.note_sampled("a")
+    assert cache.has_sampled_token("a")
+    cache.close("a")
+    cache.open("b")                      # the same slot
+    assert not cache.has_sampled_token("b")

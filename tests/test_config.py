@@ -90,3 +90,13 @@ def test_another_architecture_can_be_registered():
     register_architecture("ToyForTests", GPT2Config, lambda config, precision: calls.append(config) or "model")
     config = config_from_dict(dict(TINY_A, architectures=["ToyForTests"]))
     assert get_architecture(config.architecture).build(config, None) == "model" and calls == [config]
+
+
+def test_any_head_size_the_kernels_take_is_a_valid_configuration():
+    # the reference takes every width that its heads divide (pytorch/src/mini_llm/vector_addition_extension.cpp:180)
+    for n_embd, n_head in ((40, 4), (42, 3), (72, 3), (256, 1), (7, 7)):
+        assert config_from_dict(dict(TINY_A, n_embd=n_embd, n_head=n_head)).head_size == n_embd // n_head
+    with pytest.raises(ConfigError, match="wider than the attention kernels take"):
+        config_from_dict(dict(TINY_A, n_embd=514, n_head=2))
+    with pytest.raises(ConfigError, match="not divisible"):
+        config_from_dict(dict(TINY_A, n_embd=42, n_head=4))

@@ -340,6 +340,22 @@ def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
     engine.release_cache(h)
     while engine._queued:
         engine.take()
+    # a request that was never sampled has no token in its slot (the slot still holds its previous
+    # owner's): queueing a step for it is refused, and nothing has changed
+    from mini_llm_amd.engine import StepError
+
+    fresh = engine.try_take_cache()
+    with pytest.raises(StepError, match="no token has been sampled"):
+        engine.decode_batch_enqueue([fresh])
+    with engine.open_session() as session:
+        session.prefill(prompts[0])                                  # logits to the host, nothing sampled
+        with pytest.raises(StepError, match="no token has been sampled"):
+            engine.decode_batch_enqueue([session._handle])
+        assert session.length() == len(prompts[0])
+    assert engine.prefill_greedy(fresh, prompts[0]) == got[0][0]
+    engine.decode_batch_enqueue([fresh])
+    assert engine.take() == [got[0][1]]
+    engine.release_cache(fresh)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -213,10 +213,12 @@ def test_safetensors_roundtrip(tmp_path):
     assert P.f32_to_bf16_rne(x).tolist() == [0x3F80, 0x3F82, 0x3F81]
 
 
-REFERENCE_DUMPS = "/root/reference/engine/tests/reference_data"
+# The reference repository's root, where a checkout of it is at hand (MINI_LLM_REFERENCE=/path/to/mini_llm).
+REFERENCE_DUMPS = os.path.join(os.environ.get("MINI_LLM_REFERENCE", ""), "engine", "tests", "reference_data")
 
 
-@pytest.mark.skipif(not os.path.isdir(REFERENCE_DUMPS), reason="the reference's dumped activations are not on this machine")
+@pytest.mark.skipif(not os.environ.get("MINI_LLM_REFERENCE") or not os.path.isdir(REFERENCE_DUMPS),
+                    reason="MINI_LLM_REFERENCE does not name a checkout of the reference with its dumped activations")
 def test_dumped_activations_of_the_real_model_follow_the_plain_formulas():
     # The reference holds what every part of the real GPT-2 put out for the tokens 15496, 11, 995
     # (scripts/dump_reference.py:76-140: the three gathered embedding rows, per block the outputs of

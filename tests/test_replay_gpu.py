@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 def requests_for(name, config):
     vocab, limit = config["vocab_size"], config["n_positions"]
-    lengths = {"A": [5, 17, 33, 100, 128, 64, 65], "B": [1, 9, 40, 64, 63, 33], "C": [130, 257, 600, 40, 191]}[name]
+    lengths = {"A": [5, 17, 33, 100, 128, 64, 65], "B": [1, 9, 40, 64, 63, 33], "C": [130, 257, 600, 40, 191],
+               "D": [3, 96, 40, 65, 70], "E": [160, 33, 70, 129, 2]}[name]
     return {f"r{i}": random_tokens(100 + i, min(n, limit), vocab) for i, n in enumerate(lengths)}
 
 
@@ -28,7 +29,7 @@ MODES = {
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mode", list(MODES))
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_replay_matches_plain(model_dirs, tmp_path, name, mode, dtype):
     folder, config, weights = model_dirs[name]
     requests = requests_for(name, config)
