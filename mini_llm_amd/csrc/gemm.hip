@@ -7,6 +7,9 @@
 // linear.cu:9-18) and its epilogue order sum -> +bias -> activation -> residual + that
 // (engine/include/matvec_common.h:40-54).
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 namespace {
 
@@ -654,4 +657,77 @@ MLLM_API int mllm_gemm_qkv_cache(const void* A, const void* W, int w_packed, con
     if (dtype == MLLM_F32) { MLLM_QKV_CASE(float) } else { MLLM_QKV_CASE(bf16_t) }
 #undef MLLM_QKV_CASE
     return mllm_check_launch("gemm_qkv_cache");
+}
+
+// ------------------------------------------------------------------------------------------------
+// The product cut along K without an allocation (no_alloc.h): the partial products go to a fixed
+// array of the library instead of memory the caller brings.
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)1 << 20;  // 4 MiB
+// Each GPU holds its own copy of this array at its own address. In host code the name is only a
+// handle for hipGetSymbolAddress: kernels get the address that call returns, never the name.
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+
+constexpr int MAX_DEVICES = 64;
+float* g_scratch_at[MAX_DEVICES];  // per device: the array's address there, null until looked up
+std::mutex g_scratch_lock;
+
+// The current device's array. The lookup runs once per device, with that device current.
+int static_scratch(float** at) {
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    MLLM_REQUIRE(status == hipSuccess, "static scratch: no current device: %s", hipGetErrorString(status));
+    MLLM_REQUIRE(device >= 0 && device < MAX_DEVICES, "static scratch: device %d is beyond the %d this library keeps track of", device, MAX_DEVICES);
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if (g_scratch_at[device] == nullptr) {
+        void* address = nullptr;
+        status = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        MLLM_REQUIRE(status == hipSuccess && address != nullptr, "static scratch: the array's address on device %d is not known: %s", device,
+                     hipGetErrorString(status));
+        g_scratch_at[device] = static_cast<float*>(address);
+    }
+    *at = g_scratch_at[device];
+    return 0;
+}
+
+// out = residual + bias + partials[0] + partials[1] + ..., in that order (the order of
+// pending_sum_kernel, so that both give the same numbers). grid (column groups of 256, rows).
+__global__ __launch_bounds__(256) void static_sum_kernel(const float* __restrict__ partials, const float* __restrict__ bias,
+                                                         const float* __restrict__ residual, float* __restrict__ out, int M, int N,
+                                                         int k_blocks) {
+    const int col = blockIdx.x * 256 + threadIdx.x, row = blockIdx.y;
+    if (col >= N) return;
+    const size_t at = (size_t)row * N + col;
+    float value = residual ? residual[at] : 0.0f;
+    if (bias) value += bias[col];
+    for (int s = 0; s < k_blocks; s++) value += partials[(size_t)s * M * N + at];
+    out[at] = value;
+}
+
+}  // namespace
+
+MLLM_API long long mllm_static_scratch_bytes(void) { return (long long)(STATIC_SCRATCH_FLOATS * sizeof(float)); }
+
+MLLM_API int mllm_static_scratch_prepare(void) {
+    float* at = nullptr;
+    return static_scratch(&at);
+}
+
+MLLM_API int mllm_linear_split_static(const void* A, const void* W, int w_packed, const float* bias, const float* residual,
+                                      float* out, int M, int N, int K, int in_dtype, int k_blocks, hipStream_t stream) {
+    MLLM_REQUIRE(A != nullptr && W != nullptr && out != nullptr, "linear_split_static: an operand is missing");
+    MLLM_REQUIRE(M >= 0 && N > 0 && K > 0 && M <= 65535, "linear_split_static: bad sizes M=%d N=%d K=%d", M, N, K);
+    MLLM_REQUIRE(k_blocks >= 1 && k_blocks <= 16, "linear_split_static: %d partial products is not in 1..16", k_blocks);
+    MLLM_REQUIRE((size_t)k_blocks * (size_t)M * (size_t)N <= STATIC_SCRATCH_FLOATS,
+                 "linear_split_static: %d partial products of %d x %d floats do not fit the library's %lld bytes of scratch memory", k_blocks, M, N,
+                 mllm_static_scratch_bytes());
+    if (M == 0) return 0;
+    float* partials = nullptr;
+    if (static_scratch(&partials)) return 1;
+    if (mllm_gemm_split(A, W, w_packed, partials, M, N, K, in_dtype, k_blocks, 0, stream)) return 1;
+    dim3 grid(ceil_div(N, 256), M);
+    static_sum_kernel<<<grid, 256, 0, stream>>>(partials, bias, residual, out, M, N, k_blocks);
+    return mllm_check_launch("linear_split_static");
 }

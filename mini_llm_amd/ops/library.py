@@ -40,6 +40,8 @@ _SIGNATURES = {
                                    c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_decode_mlp_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_pending_sum": [P, P, P, c_int, P, c_int, c_int, P],
+    "mllm_linear_split_static": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
+    "mllm_static_scratch_prepare": [],
     "mllm_pending_layernorm": [P, P, P, c_int, c_int, P, P, P, P, P, c_int, c_int, c_float, c_int, c_int, P],
 }
 
@@ -68,6 +70,8 @@ def library() -> ctypes.CDLL:
             fn.argtypes = argtypes
             fn.restype = c_int
         lib.mllm_packed_elements.restype = c_longlong
+        lib.mllm_static_scratch_bytes.restype = c_longlong
+        lib.mllm_static_scratch_bytes.argtypes = []
         lib.mllm_last_error.restype = ctypes.c_char_p
         lib.mllm_last_error.argtypes = []
         lib.path = path
