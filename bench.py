@@ -5,9 +5,11 @@
 A step is one decode step: every live sequence gets one new token (greedy, sampled on the
 device and fed back). Sequences start from 512-token uniform-random prompts and decode towards
 1,024 tokens; when they are full they are given back and prefilled again outside the timed
-region, so that exactly K steps are timed. Before anything is timed, decoding is compared with a
-whole-prompt step on 8 tokens (--no-check skips that). Prints one JSON line. The reference's counterpart is
-engine/bench/bench_batch.c (batched decode at a context) and engine/bench/bench.c."""
+region, so that exactly K steps are timed. Before anything is timed, 8 decoded tokens are compared
+with a whole-prompt step and with the plain implementation under tests/ (--no-check skips that).
+Prints one JSON line: the headline in bfloat16, the same figures in 32-bit under "points_fp32", and
+under "kernels" what the kernels a step's time goes to reach of their own roofline. The reference's
+counterpart is engine/bench/bench_batch.c (batched decode at a context) and engine/bench/bench.c."""
 
 from __future__ import annotations
 
@@ -144,13 +146,132 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
 
 
-def check_before_timing(engine, n_new: int = 8):
+def measure_kernels(engine, batch: int = 8, context: int = 768, reps: int = 7):
+    """What the kernels that a step's time goes to reach of their own roofline, each timed alone
+    between two events over all layers' weights in turn (as a step walks them), median of ``reps``:
+    for a 2,048-token prompt step the four products of a layer and the prompt attention (flops /
+    time / the matrix cores' peak), for a decode step of ``batch`` sequences at ``context`` tokens the
+    two halves of a layer and the head (the bytes each has to read / time / the memory's peak). The
+    reference prices its kernels the same way, against a pure read of the same bytes
+    (docs/kernels/010_matvec_batch.md:20,108-117)."""
+    import numpy as np
+    import torch
+
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.batch import build_step_batch
+    from mini_llm_amd.ops import kernels
+
+    model, cache, runner = engine.model, engine.cache, engine.runner
+    config, dtype = engine.config, engine.options.dtype
+    e = element_size(dtype)
+    compute = model.precision.compute
+    d, ff, n_layer, vocab = config.n_embd, config.n_inner, config.n_layer, config.vocab_size
+    rng = np.random.default_rng(SEED + 4)
+    calls = [(model.blocks[call.block], cache.layer_context, call) for call in model.schedule]
+
+    def timed(per_layer) -> float:
+        """Seconds of one call of per_layer(block, ctx), averaged over the layers."""
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        samples = []
+        for rep in range(reps + 2):
+            start.record()
+            for block, context_of, call in calls:
+                per_layer(block, context_of(batch_of_step, call))
+            stop.record()
+            torch.cuda.synchronize()
+            samples.append(start.elapsed_time(stop) / 1e3 / len(calls))
+        return float(np.median(samples[2:]))
+
+    def staged(entries):
+        """The batch of a step whose pages are reserved but which is never committed."""
+        for entry in entries:
+            cache.reserve(entry.request_id, len(entry.tokens))
+        return build_step_batch(entries, cache, runner.staging, vocab_size=vocab, short_portion=model.short_portion())
+
+    out = {}
+
+    def note(name, seconds, work, peak, unit):
+        out[name] = {"us": round(seconds * 1e6, 2), "frac": round(work / seconds / peak, 4), "of": unit}
+
+    # --- a prompt step of two 1,024-token prompts
+    lengths = [CONTEXT, CONTEXT]
+    handles = [engine.try_take_cache() for _ in lengths]
+    entries = [StepEntry(h, rng.integers(0, vocab, n).tolist(), [n - 1]) for h, n in zip(handles, lengths)]
+    batch_of_step = staged(entries)
+    rows = sum(lengths)
+    hidden = model.embedding.forward(batch_of_step.tokens, batch_of_step.positions, model.position_encoding)
+    block0 = model.blocks[0]
+    mixer, feed = block0.mixer_part(), block0.feed_forward
+    x = block0.norm_1.forward(hidden, compute)
+    peak, unit = PEAK_FLOPS[dtype], f"{'bf16' if dtype == 'bfloat16' else 'fp32'} matrix peak"
+    kept = {}
+
+    def qkv(block, ctx):
+        m = block.mixer_part()
+        kept["q"] = kernels.linear_qkv_cache(x, m.qkv.weight, m.qkv.bias, ctx.k_pages, ctx.v_pages, ctx.group.slots, m.n_heads, m.n_kv_heads, m.head_size)
+
+    note("prefill_qkv_product", timed(qkv), 2.0 * rows * d * 3 * d, peak, unit)
+
+    def attention(block, ctx):
+        m, b = block.mixer_part(), ctx.batch
+        kept["mixed"] = kernels.paged_attention(kept["q"], ctx.k_pages, ctx.v_pages, b.token_request, b.positions, ctx.group.block_tables, m.n_heads,
+                                                m.n_kv_heads, m.head_size, m.scale, max_q_len=b.max_q_len, max_len=b.max_total_len,
+                                                q_starts=b.q_starts, context_lens=b.context_lens)
+
+    note("prefill_attention", timed(attention), sum(4.0 * (n * (n + 1) / 2) * d for n in lengths), peak, unit)
+    note("prefill_out_product", timed(lambda block, ctx: block.mixer_part().out.forward_pending(kept["mixed"], hidden)), 2.0 * rows * d * d, peak, unit)
+
+    def up(block, ctx):
+        kept["u"] = block.feed_forward.up.forward(x, activation=block.feed_forward.activation)
+
+    note("prefill_up_product", timed(up), 2.0 * rows * d * ff, peak, unit)
+    note("prefill_down_product", timed(lambda block, ctx: block.feed_forward.down.forward_pending(kept["u"], hidden)), 2.0 * rows * d * ff, peak, unit)
+    kept.clear()
+    for h in handles:
+        cache.rollback(h)
+        engine.release_cache(h)
+
+    # --- a decode step: ``batch`` sequences that hold ``context`` tokens each
+    handles = [engine.try_take_cache() for _ in range(batch)]
+    for i in range(0, batch, 4):
+        runner.step([StepEntry(h, rng.integers(0, vocab, context - 1).tolist(), []) for h in handles[i : i + 4]])
+    entries = [StepEntry(h, [int(rng.integers(0, vocab))], [0]) for h in handles]
+    batch_of_step = staged(entries)
+    hidden = model.embedding.forward(batch_of_step.tokens, batch_of_step.positions, model.position_encoding)
+    hbm = HBM_GBS * 1e9
+    # each half takes the stream as the other half leaves it (with its last sums pending, where the parts do that)
+    context_0 = cache.layer_context(batch_of_step, model.schedule[0])
+    after_mlp = feed.forward_normed(hidden, block0.norm_2, compute, context_0)
+    after_attention = mixer.forward_normed(after_mlp, block0.norm_1, compute, context_0)
+    note("decode_attention_half", timed(lambda block, ctx: block.mixer_part().forward_normed(after_mlp, block.norm_1, compute, ctx)),
+         (4.0 * d * d + batch * context * 2.0 * d) * e, hbm, "HBM peak")
+    note("decode_mlp_half", timed(lambda block, ctx: block.feed_forward.forward_normed(after_attention, block.norm_2, compute, ctx)),
+         2.0 * d * ff * e, hbm, "HBM peak")
+    normed = model.final_norm.forward(kernels.settle(hidden), compute, row_index=batch_of_step.logit_rows)
+    logits = {}
+
+    def head(block, ctx):
+        logits["rows"] = model.head.forward(normed)
+
+    note("decode_head", timed(head), float(vocab) * d * e, hbm, "HBM peak")
+    note("decode_sampler", timed(lambda block, ctx: kernels.sample(logits["rows"])), batch * vocab * 4.0, hbm, "HBM peak")
+    for h in handles:
+        cache.rollback(h)
+        engine.release_cache(h)
+    torch.cuda.synchronize()
+    return out
+
+
+def check_before_timing(engine, host_weights=None, n_new: int = 8):
     """The gate before anything is timed, as the reference's bench has one (engine/bench/bench.c:30-31,
     92-113: its GPU against its CPU path on 8 tokens, scaled difference <= 1e-3 and the same next
-    token). Here two sequences are decoded greedily for 8 tokens the way the timed steps run (single
-    tokens over the cache, replayed from a graph), then each whole sequence runs again as one prompt
-    step, through the other kernels (tiled products, prompt attention): the logits at the decoded
-    places must agree. Returns the largest difference / largest logit."""
+    token). Two sequences are decoded greedily for 8 tokens the way the timed steps run (single
+    tokens over the cache, replayed from a graph). Then (1) each whole sequence runs again as one
+    prompt step, through the other kernels (tiled products, prompt attention), and (2) with
+    ``host_weights`` (the model's tensors as numpy arrays) the first sequence runs through the plain
+    implementation under tests/ (numpy, float64, no cache; storing in bfloat16 what a bfloat16 run
+    stores): the logits at the decoded places must agree with both. Returns the largest
+    difference / largest logit of (1) and of (2)."""
     import numpy as np
     import torch
 
@@ -169,23 +290,41 @@ def check_before_timing(engine, n_new: int = 8):
         logits = engine.runner.step([StepEntry(h, [seq[-1]], [0]) for h, seq in zip(handles, sequences)])
     for h in handles:
         engine.release_cache(h)
-    worst = 0.0
-    limit = 1e-3 if engine.options.dtype == "float32" else 5e-2   # bfloat16 rounds every stored activation to 3 digits
-    for i, (prompt, seq) in enumerate(zip(prompts, sequences)):
-        handle = engine.try_take_cache()
-        fed = seq[:-1]
-        whole = engine.runner.step([StepEntry(handle, fed, list(range(len(prompt) - 1, len(fed))))]).float().cpu().numpy()
-        engine.release_cache(handle)
-        for k, (a, b) in enumerate(zip(stepwise[i], whole)):
+    bf16 = engine.options.dtype == "bfloat16"
+
+    def compare(what, got_rows, want_rows, limit, sequence):
+        worst = 0.0
+        for k, (a, b) in enumerate(zip(got_rows, want_rows)):
             scaled = float(np.abs(a - b).max() / np.abs(b).max())
             worst = max(worst, scaled)
             top = np.sort(b)[-2:]
             clear = (top[1] - top[0]) > 2 * limit * np.abs(b).max()   # a near tie may fall either way
             if not scaled <= limit or (clear and int(a.argmax()) != int(b.argmax())):
-                raise SystemExit(f"bench.py: decoding and the whole-prompt step disagree at sequence {i}, new token {k}: "
-                                 f"scaled difference {scaled:.3e} (allowed {limit:g}), next token {int(a.argmax())} vs {int(b.argmax())}; nothing was timed")
+                raise SystemExit(f"bench.py: decoding and {what} disagree at sequence {sequence}, new token {k}: scaled difference "
+                                 f"{scaled:.3e} (allowed {limit:g}), next token {int(a.argmax())} vs {int(b.argmax())}; nothing was timed")
+        return worst
+
+    worst_whole = 0.0
+    limit = 5e-2 if bf16 else 1e-3   # bfloat16 rounds every stored activation to 3 digits, and the two paths round at different places
+    for i, (prompt, seq) in enumerate(zip(prompts, sequences)):
+        handle = engine.try_take_cache()
+        fed = seq[:-1]
+        whole = engine.runner.step([StepEntry(handle, fed, list(range(len(prompt) - 1, len(fed))))]).float().cpu().numpy()
+        engine.release_cache(handle)
+        worst_whole = max(worst_whole, compare("the whole-prompt step", stepwise[i], whole, limit, i))
     torch.cuda.synchronize()
-    return worst
+    worst_plain = None
+    if host_weights is not None:
+        sys.path.insert(0, str(Path(__file__).resolve().parent / "tests"))
+        import plain_gpt2
+
+        raw = engine.config.to_dict()
+        weights = plain_gpt2.bf16_weights(host_weights) if bf16 else host_weights
+        fed = sequences[0][:-1]
+        plain = plain_gpt2.forward(raw, weights, fed, stored=plain_gpt2.stored_as_bf16 if bf16 else plain_gpt2._keep)
+        # against exact arithmetic over the same stored numbers: 2e-2 of the largest logit in bfloat16 (observed: a few 1e-3)
+        worst_plain = compare("the plain implementation", stepwise[0], plain[len(prompts[0]) - 1 :], 2e-2 if bf16 else 1e-3, 0)
+    return worst_whole, worst_plain
 
 
 MEDIUM = dict(SMALL, n_layer=24, n_embd=1024, n_head=16, n_inner=4096)
@@ -294,7 +433,8 @@ def main() -> int:
     parser.add_argument("--json", default=None, metavar="PATH", help="also write the printed record to this file (the reference's option)")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-check", action="store_true", help="skip the comparison of decoding with a whole-prompt step before timing")
-    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points and the prefill")
+    parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points, the prefill, the kernels and the other precision")
+    parser.add_argument("--one-dtype", action="store_true", help="skip the figures in the other precision")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
@@ -315,6 +455,8 @@ def main() -> int:
 
     from mini_llm_amd.config import config_from_dict
     from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.loading import build_model, require_gpu
+    from mini_llm_amd.weights import bind_tensors, random_tensors
 
     shape, seed = SHAPES[args.shape]
     if not 1 <= args.prompt_len < CONTEXT:
@@ -322,15 +464,36 @@ def main() -> int:
     layers = args.layers or shape["n_layer"]
     config = config_from_dict(dict(shape, n_layer=layers))
     largest = max(args.batch, 1 if args.no_points else 64, 1 if args.no_check else 2)   # the check before timing runs two sequences
-    engine = Engine.from_random(config, seed, EngineOptions(dtype=args.dtype, max_sessions=largest, max_tokens=largest * CONTEXT))
+    tensors = {}
 
-    checked = None if args.no_check else check_before_timing(engine)
+    def make_engine(dtype):
+        """An engine over the seed's random weights (drawn once, on the host, and kept there for the check)."""
+        model = build_model(config, dtype)
+        if not tensors:
+            tensors.update(random_tensors(model, seed))
+        bind_tensors(model, tensors, require_gpu())
+        return Engine(options=EngineOptions(dtype=dtype, max_sessions=largest, max_tokens=largest * CONTEXT), model=model)
+
+    def host_weights():
+        return {name: tensor.numpy() for name, tensor in tensors.items()}
+
+    engine = make_engine(args.dtype)
+    checked = None if args.no_check else check_before_timing(engine, host_weights())
     if args.prefill_only:
         emit({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}, args.json)
         return 0
     seconds, step_bytes = DecodeBench(engine, args.batch, args.prompt_len).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
     achieved = step_bytes / (seconds / args.steps) / 1e9
+    short = {"bfloat16": "bf16", "float32": "fp32"}
+
+    def check_record(values):
+        if values is None:
+            return None
+        whole, plain = values
+        return {"decode_vs_whole_prompt_scaled_diff": float(f"{whole:.3g}"), "decode_vs_plain_scaled_diff": None if plain is None else float(f"{plain:.3g}"),
+                "tokens": 8}
+
     record = {
         "metric": f"decode tokens/s at batch {args.batch}, GPT-2 {args.shape}, {args.prompt_len}-token prompts decoding towards 1024",
         "value": round(args.batch * args.steps / seconds, 1),
@@ -342,7 +505,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "dtype": short[args.dtype],
         "data": "synthetic: seeded random weights, uniform-random token ids",
         "config": {
             "model": f"gpt2-{args.shape}", "n_layer": shape["n_layer"], "layers_run": layers, "n_embd": config.n_embd,
@@ -351,7 +514,7 @@ def main() -> int:
             "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": CONTEXT, "page_size": engine.cache.page_size,
             "kv_cache_dtype": args.dtype, "sampling": "greedy", "parallelism": "single-gpu", "seed": seed,
         },
-        "check": None if checked is None else {"decode_vs_whole_prompt_scaled_diff": float(f"{checked:.3g}"), "tokens": 8},
+        "check": check_record(checked),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
     }
     if not args.no_points:
@@ -361,6 +524,28 @@ def main() -> int:
             s, _ = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
             points[f"decode_b{batch}"] = round(batch * steps / s, 1)
         record["points"] = points
+        record["kernels"] = measure_kernels(engine)
+        if not args.one_dtype:
+            # the same figures in the other precision (the headline names both): one record for the two
+            other = "float32" if args.dtype == "bfloat16" else "bfloat16"
+            del engine
+            import torch
+
+            torch.cuda.empty_cache()
+            engine = make_engine(other)
+            other_check = None if args.no_check else check_before_timing(engine, host_weights())
+            figures = {}
+            for batch, steps in ((1, 64), (args.batch, 64), (64, 32)):
+                s, step_bytes = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
+                figures[f"decode_b{batch}"] = round(batch * steps / s, 1)
+                if batch == args.batch:
+                    figures["ms_per_step"] = round(s / steps * 1e3, 4)
+                    figures["roofline_frac"] = round(step_bytes / (s / steps) / 1e9 / HBM_GBS, 4)
+            prefill = measure_prefill(engine)
+            figures.update({"prefill": prefill["value"], "prefill_ms": prefill["ms"], "prefill_frac": prefill["frac"]})
+            if other_check is not None:
+                figures["check_vs_plain_scaled_diff"] = None if other_check[1] is None else float(f"{other_check[1]:.3g}")
+            record[f"points_{short[other]}"] = figures
     emit(record, args.json)
     return 0
 

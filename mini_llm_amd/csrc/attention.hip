@@ -687,8 +687,6 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
         }
 }
 
-int g_prefill_shape = 0;  // 0: chosen by size; set by mllm_attention_prefill_force_shape for tuning runs
-
 template <typename T, int HD_PAD>
 void launch_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride,
                     const int* q_starts, const int* context_lens, const int* block_tables, int max_blocks,
@@ -699,8 +697,7 @@ void launch_prefill(const void* q, int q_stride, const void* k_pages, const void
     constexpr bool ROOMY = PrefillLds<T, HD_PAD, 1, 4>::TILE_BYTES <= 80 * 1024;
     // Measured on MI355X (two 1,024-token prompts, 12 heads of 64): 128 queries per block run 2.5
     // times faster than 32, because every block reads its keys and values again from the cache.
-    int shape = g_prefill_shape;
-    if (shape == 0) shape = max_q_len > 64 ? 3 : (max_q_len > 32 ? 5 : (ROOMY ? 1 : 4));
+    const int shape = max_q_len > 64 ? 3 : (max_q_len > 32 ? 5 : (ROOMY ? 1 : 4));
 #define MLLM_PREFILL_LAUNCH(QG, KS)                                                                                   \
     {                                                                                                                  \
         dim3 grid(ceil_div(max_q_len, 32 * QG), n_heads, n_requests);                                                  \
@@ -723,9 +720,6 @@ void launch_prefill(const void* q, int q_stride, const void* k_pages, const void
 }
 
 }  // namespace
-
-// Tuning aid: forces one block shape of the prefill kernel (0 gives the choice back to the sizes).
-MLLM_API void mllm_attention_prefill_force_shape(int shape) { g_prefill_shape = shape; }
 
 // 1 if the matrix-core prefill kernel takes this head size and page size.
 MLLM_API int mllm_attention_prefill_supported(int head_size, int page_size) {

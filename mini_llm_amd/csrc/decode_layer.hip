@@ -29,19 +29,6 @@ constexpr int DL_MAX_WIDTH = 2048;  // a row's 4-column pieces: at most 2 per th
 constexpr int DL_KSPLIT = 4;        // waves that share the k range of one 16-row tile
 constexpr int DL_TOKENS = 16;       // tokens a feed-forward block takes: the matrix core's other 16
 
-// Tuning aid, compiled in with -DMLLM_PHASE_STAMPS only: block (1, 1) notes the 100 MHz clock at
-// the numbered places of a kernel (places 20.. by the first lane of wave 8, the others by thread
-// 0); mllm_phase_stamps() copies the notes out.
-#ifdef MLLM_PHASE_STAMPS
-__device__ long long dl_stamps[32];
-#define DL_STAMP(i)                                                                         \
-    do {                                                                                    \
-        if (blockIdx.x == 1 && blockIdx.y == (gridDim.y > 1) && threadIdx.x == ((i) >= 20 ? 512 : 0)) dl_stamps[i] = wall_clock64(); \
-    } while (0)
-#else
-#define DL_STAMP(i)
-#endif
-
 struct PendingSum {
     const float* base;      // [rows, width]
     const float* partials;  // [n_partials, rows, width]
@@ -208,7 +195,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
     const int role_wave = attends ? wave - DL_PROJECT_WAVES : wave;
     const int head = blockIdx.x, token = blockIdx.y;
     const int n_pieces = width / 4;
-    DL_STAMP(0);
     float* out_row = partial_out + ((size_t)head * n_tokens + token) * width;
     const int request = token_request[token];
     const int position = positions[token];
@@ -299,10 +285,8 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         keep_order();
         typename Sweep::Fetched fetched;
         sweep.fetch_rows(fetched, key_page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
-        DL_STAMP(20);
         lds_barrier();  // 4
         lds_barrier();  // 5: q, k, v of this token are in LDS
-        DL_STAMP(21);
         float qf[VEC];
 #pragma unroll
         for (int i = 0; i < VEC; i++) qf[i] = qkv_row[0][sub * VEC + i] * scale;
@@ -323,7 +307,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
                 merged[entry][HD + 1] = sweep.running_sum;
             }
         }
-        DL_STAMP(22);
         lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
         lds_barrier();  // 7
         return;
@@ -351,9 +334,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         return;
     }
     share_of_keys();
-    DL_STAMP(1);
     lds_barrier();  // 1: the eight sums of the partial rows are in LDS
-    DL_STAMP(8);
     // width / 4 <= 512: the threads of these waves cover the row
     row += pending_bias * (in.bias ? 1.0f : 0.0f);
     if (owns) {
@@ -363,9 +344,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         row = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     row_lds[tid] = row;
-    DL_STAMP(9);
     lds_barrier();  // 2: the row with its sums taken is in LDS
-    DL_STAMP(16);
 
     // the norm, centred, in 32-bit: every wave takes the statistics of the whole row for itself (no
     // further meeting of the waves), then norms the four columns it owns
@@ -391,9 +370,7 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         if (!owns) y = f32x4{0.0f, 0.0f, 0.0f, 0.0f};  // beyond the width: zeros, the products read whole 32-column steps
         store_bf16x4(x_hat + 4 * tid, y);
     }
-    DL_STAMP(17);
     lds_barrier();  // 3: the normed row is in LDS
-    DL_STAMP(2);
     int far_page[Sweep::UNROLL];  // the pages of this wave's share of the far keys (of the spare key, if there are none)
     sweep.look_up(far_page, table, page_shift, begin, end, spare_key, lane);
 
@@ -415,7 +392,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
             }
         }
     };
-    DL_STAMP(3);
     if (n_far > 0) {  // a long context (the same for the whole block): these waves attend to their shares of the far keys
         typename Sweep::Fetched fetched;
         sweep.fetch_rows(fetched, far_page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, begin, end, spare_key, lane);
@@ -436,7 +412,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         lds_barrier();  // 5
         sweep.init();
     }
-    DL_STAMP(4);
     {
         const int entry = wave * MERGE_ENTRIES + lane / MERGE_SPAN;
         if (lane % MERGE_SPAN < LPR) {
@@ -463,7 +438,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
             out_piece[g][s] = load16<Vec16>(w_out + packed_offset<bf16_t>(out_tile, out_step0 + s, out_k_steps, 0), lane * 16);
     }
     lds_barrier();  // 6: every wave's (max, sum, output) is in LDS
-    DL_STAMP(5);
     if (wave < (HD_PAD + WAVE - 1) / WAVE) {  // whole waves (the wave sums below need every lane); the mixed row lies where its columns lie in the chunks of w_out, zeros around it
         // out = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M) over the triples s (one without keys has
         // m = -inf, l = 0). Each wave works the weights out once, a lane a triple, and keeps them in
@@ -485,7 +459,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         if (tid < HD_PAD) mixed[tid] = static_cast<bf16_t>(value);
     }
     lds_barrier();  // 7: the mixed row of this head is in LDS
-    DL_STAMP(6);
 
     // this head's share of the output product: rows of w_out in tiles of 16, columns head*HD ..
     for (int tile0 = wave; tile0 < out_tiles; tile0 += DL_PROJECT_WAVES * OUT_GROUP) {
@@ -511,7 +484,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
             if (row16 == 0 && out_col < width) *reinterpret_cast<f32x4*>(out_row + out_col) = acc;
         }
     }
-    DL_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -548,7 +520,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
     const int row16 = lane % 16, quad = lane / 16;
     const int n_steps = (width + 31) / 32;
     const int steps_per_unit = (n_steps + DL_KSPLIT - 1) / DL_KSPLIT;
-    DL_STAMP(10);
 
     // ---- the pending sums and the norm. With T tokens in this block (rounded up to a power of
     // two), wave w works for token w % T and takes the partial rows w / T, w / T + 16 / T, ...
@@ -665,7 +636,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
                 }
             }
         }
-        DL_STAMP(11);
         bf16_t* x_row = x_hat + wave * x_stride;  // wave w < t2 is token w's first wave; the others clear the rows from t2 on
         if (sub == 0 && live) {
             float sum = 0.0f;
@@ -696,7 +666,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
         }
     }
     lds_barrier();
-    DL_STAMP(12);
 
     // ---- up product for this slice's U hidden units: TILES tiles of 16 rows, DL_KSPLIT waves a tile
     {
@@ -728,7 +697,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
                 for (int r = 0; r < 4; r++) up_part[((up_part_of[u] * TILES + up_tile[u]) * 4 + r) * WAVE + lane] = acc[u][r];
             }
     }
-    DL_STAMP(13);
     lds_barrier();
     // acc[r] of lane l in tile t is (token l % 16, hidden unit 16 t + 4 (l / 16) + r)
 #pragma unroll
@@ -750,7 +718,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
         hidden[(l % 16) * H_STRIDE + unit] = static_cast<bf16_t>(value);
     }
     lds_barrier();
-    DL_STAMP(14);
 
     // ---- this slice's share of the down product: rows of w_down in tiles of 16, columns slice*U ..
     {
@@ -780,7 +747,6 @@ __global__ __launch_bounds__(DL_THREADS) void decode_mlp_half_kernel(
             }
         }
     }
-    DL_STAMP(15);
 }
 
 // Four columns of a pending row with their sums taken: eight partial rows asked for at a time.
@@ -894,6 +860,17 @@ MLLM_API int mllm_decode_layer_supported(int width, int head_size, int page_size
     return 1;
 }
 
+// Up to how many rows the two layer kernels beat the kernels run one by one, for a layer of this
+// width (0: never). A property of the kernels, measured on MI355X: every (token, head) block pulls
+// its own copy of the partial rows and of its head's matrices through one compute unit, which grows
+// with the width, while what the fusion saves (five kernel boundaries a layer) does not. Up to 768
+// columns the fused kernels win up to 16 rows (by 2 % at 1 row, 11 % at 8, 12 % at 16, and lose by
+// 4 % at 32); at 1,024 columns they lose at every row count (1.10 against 0.96 ms a step at 1 row).
+MLLM_API int mllm_decode_layer_rows(int width) {
+    if (!mllm_decode_layer_supported(width, 0, 0, 0)) return 0;
+    return width <= 768 ? 16 : 0;
+}
+
 MLLM_API int mllm_decode_attention_half(
     const float* base, const float* partials, const float* pending_bias, int n_partials, float* summed,
     const float* gamma, const float* beta, float eps, const void* w_qkv, const float* b_qkv, const void* w_out,
@@ -994,7 +971,3 @@ MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, co
         MLLM_REQUIRE(false, "pending_layernorm: unknown output dtype %d", out_dtype);
     return mllm_check_launch("pending_layernorm");
 }
-
-#ifdef MLLM_PHASE_STAMPS
-MLLM_API int mllm_phase_stamps(long long* out) { return hipMemcpyFromSymbol(out, HIP_SYMBOL(dl_stamps), sizeof(long long) * 32) == hipSuccess ? 0 : 1; }
-#endif

@@ -502,8 +502,6 @@ int tiled_k_blocks(int M, int N, int K) {
     return k_blocks;
 }
 
-int g_forced_tile = 0;  // 0: chosen by size; set by mllm_gemm_force_tile for tuning runs
-
 template <typename T, typename OutT, bool ALIGNED, int BM, int BN, int WAVES_M, int WAVES_N>
 void launch_tile(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
                  int K, int epilogue, hipStream_t stream, CacheScatter scatter, int k_blocks) {
@@ -517,8 +515,8 @@ void launch_tile(const T* a, const T* w, bool packed, const float* bias, const f
 template <typename T, typename OutT, bool ALIGNED>
 void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
                   int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
-    int tile = g_forced_tile;
-    if (tile == 0) {
+    int tile = 0;
+    {
         // measured on MI355X at GPT-2 sizes: many waves per block hide latency best; the large tile
         // (sixteen waves, half the traffic from the cache of the chip for the same product) from
         // about half a block a compute unit on, where it wins by 5 % (2,048 x 2,304 x 768) to 25 %
@@ -546,7 +544,7 @@ bool takes_few_row_kernel(int M, int N, int K) {
     const bool aligned = K % Tile<T>::VEC == 0;
     const bool wide = N >= 8192;
     const int skinny_rows = !wide ? 64 : 0;  // over 50,257 columns the 32-row tile takes 40 us in 32-bit at 1 to 12 rows, this kernel 50 us
-    return g_forced_tile == 0 && aligned && M <= skinny_rows;
+    return aligned && M <= skinny_rows;
 }
 
 template <typename T, typename OutT>
@@ -567,9 +565,6 @@ void launch_gemm(const void* A, const void* W, bool packed, const float* bias, c
 }
 
 }  // namespace
-
-// Tuning aid: forces one tile shape of the tiled kernel (1: 32x128, 2: 64x64, 3: 256x128, another number: 128x64; 0 gives the choice back to the sizes).
-MLLM_API void mllm_gemm_force_tile(int tile) { g_forced_tile = tile; }
 
 // 1 if a product of M rows with an [N, K] matrix takes rows in the packed layout (x_packed, out_packed).
 MLLM_API int mllm_gemm_takes_packed_rows(int M, int N, int K, int in_dtype) {

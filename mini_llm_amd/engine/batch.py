@@ -40,9 +40,11 @@ class GroupStepData:
     slots: object          # int32 [n_tokens]: cache row each token's key/value is written to
 
 
-# Portions up to this long are laid out before the longer ones, whatever the order of the
+# Portions up to so many tokens are laid out before the longer ones, whatever the order of the
 # entries, so that a mixer can treat the two kinds apart (single decoded tokens over long
-# contexts beside long portions want different kernels) by cutting the batch at one row.
+# contexts beside long portions want different kernels) by cutting the batch at one row. How many
+# is the model's to say (Model.short_portion: what its mixers' kernels for short portions take);
+# this is what a batch built without a model gets.
 SHORT_PORTION = 8
 
 
@@ -54,7 +56,7 @@ class StepBatch:
     max_q_len: int          # the longest portion in the batch
     short_requests: int     # the first so many requests bring portions of at most SHORT_PORTION tokens,
     short_rows: int         # which are the first so many rows; the requests after them bring longer ones
-    short_portion: int = field(default=SHORT_PORTION, init=False)
+    short_portion: int = field(default=SHORT_PORTION, kw_only=True)   # the length that cut was made at
     max_total_len: int      # the longest sequence after this step
     tokens: object          # int32 [n_tokens]
     positions: object       # int32 [n_tokens]
@@ -134,7 +136,7 @@ def _pad(array: np.ndarray, length: int, fill: int) -> np.ndarray:
 
 
 def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int, capacity: int | None = None,
-                     device_buffer=None) -> StepBatch:
+                     device_buffer=None, short_portion: int = SHORT_PORTION) -> StepBatch:
     """Lays out the batch on the host and uploads it in one copy. The entries have been checked
     and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests).
 
@@ -142,16 +144,16 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     -1, request -1, slot -1), so that the layout depends on the capacity alone; ``device_buffer``
     then is the fixed device buffer the batch is copied into (a captured graph reads it).
 
-    The requests are laid out short portions first (SHORT_PORTION); the logit rows keep the order
-    of the entries as given."""
+    The requests are laid out short portions first (up to ``short_portion`` tokens); the logit rows
+    keep the order of the entries as given."""
     n_requests = len(entries)
     given = entries
-    layout = sorted(range(n_requests), key=lambda i: len(given[i].tokens) > SHORT_PORTION)  # stable
+    layout = sorted(range(n_requests), key=lambda i: len(given[i].tokens) > short_portion)  # stable
     place = {i: at for at, i in enumerate(layout)}   # entry as given -> its place in the layout
     entries = [given[i] for i in layout]
     q_lens = [len(e.tokens) for e in entries]
-    short_requests = sum(1 for q in q_lens if q <= SHORT_PORTION)
-    short_rows = sum(q for q in q_lens if q <= SHORT_PORTION)
+    short_requests = sum(1 for q in q_lens if q <= short_portion)
+    short_rows = sum(q for q in q_lens if q <= short_portion)
     n_tokens = sum(q_lens)
     contexts = [cache.length(e.request_id) for e in entries]
     n_groups = len(cache.groups)
@@ -223,7 +225,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
-        request_ids=[e.request_id for e in entries], host=host,
+        request_ids=[e.request_id for e in entries], host=host, short_portion=short_portion,
     )
 
 

@@ -158,7 +158,7 @@ class ModelRunner:
                 batch, logits = graph.run(entries)
                 self.graph_steps += 1
             else:
-                batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size)
+                batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size, short_portion=self.model.short_portion())
                 in_given_order = None
                 if observer is not None:
                     rows = batch.rows_in_order_of([e.request_id for e in entries])

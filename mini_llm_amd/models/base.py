@@ -76,6 +76,12 @@ class Model(Part):
             return self.position_encoding.max_positions()
         return None
 
+    def short_portion(self) -> int:
+        """The longest portion that the batch lays out among the short ones: what every mixer's
+        kernel for short portions takes (a mixer without such a kernel does not care)."""
+        limits = [limit for limit in (block.mixer_part().short_portion for block in self.blocks) if limit is not None]
+        return min(limits) if limits else 1
+
     def cache_groups(self) -> list[CacheGroupSpec]:
         groups: dict = {}
         for call in self.schedule:

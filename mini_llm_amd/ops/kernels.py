@@ -479,13 +479,20 @@ MLP_SLICE_UNITS = 64         # hidden units a block of the feed-forward kernel t
 LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kernels
 
 
+_layer_kernel_rows: dict = {}
+
+
 def layer_kernel_rows(width: int) -> int:
-    """Rows up to which the layer kernels for decoding beat the separate kernels (measured on
-    MI355X: at GPT-2 small's width up to 16 rows; at GPT-2 medium's the separate kernels, with
-    their products cut along K, win at every batch size: every (token, head) block reading its
-    own copy of the partial rows and of the matrices costs more than the launches and round trips
-    the fusion saves)."""
-    return min(16, LAYER_KERNEL_MAX_ROWS) if width <= 768 else 0
+    """Rows up to which the layer kernels for decoding beat the separate kernels at this width: the
+    library's own answer (mllm_decode_layer_rows, where the measurements behind it are written
+    down), or MINI_LLM_LAYER_KERNEL_ROWS from the environment, for measuring the crossover again."""
+    if width not in _layer_kernel_rows:
+        import os
+
+        forced = os.environ.get("MINI_LLM_LAYER_KERNEL_ROWS")
+        rows = int(forced) if forced is not None else int(library().mllm_decode_layer_rows(int(width)))
+        _layer_kernel_rows[width] = max(0, min(rows, LAYER_KERNEL_MAX_ROWS))
+    return _layer_kernel_rows[width]
 
 
 def _pending(hidden):

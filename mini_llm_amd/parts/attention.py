@@ -26,6 +26,7 @@ MAX_HEAD_SIZE = 256
 
 class CausalSelfAttention(Mixer):
     graph_safe = True
+    short_portion = kernels.DECODE_MAX_Q_LEN   # what the split-key kernel takes
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int | None = None, head_size: int | None = None,
                  window: int | None = None, out_std: float = 0.02, qkv_name: str = "c_attn.", out_name: str = "c_proj."):

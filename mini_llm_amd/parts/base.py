@@ -105,6 +105,9 @@ class Mixer(Part):
     """Mixes information between the positions of a sequence (attention here)."""
 
     graph_safe = False  # a mixer says so itself
+    # Portions up to so many tokens this mixer runs through a kernel of their own, apart from longer
+    # ones (None: it makes no difference): the batch lays such portions out first.
+    short_portion: int | None = None
 
     def kv_need(self) -> KVNeed | None:
         return None
