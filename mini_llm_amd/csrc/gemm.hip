@@ -38,6 +38,12 @@ struct Tile<bf16_t> {
     static constexpr int PAD = 8;
 };
 
+}  // namespace
+
+#include "gemm_stream.h"
+
+namespace {
+
 // One 16-byte piece of a row. With ALIGNED (K a multiple of VEC, so every row starts on a
 // 16-byte boundary and a piece is whole or absent) the load is unconditional from a clamped
 // address; whether the piece lies inside the matrix is returned in `valid` and applied later,
@@ -515,6 +521,12 @@ void launch_tile(const T* a, const T* w, bool packed, const float* bias, const f
 template <typename T, typename OutT, bool ALIGNED>
 void launch_tiled(const T* a, const T* w, bool packed, const float* bias, const float* residual, OutT* o, int M, int N,
                   int K, int epilogue, hipStream_t stream, CacheScatter scatter = CacheScatter{}, int k_blocks = 1) {
+    if constexpr (sizeof(T) == 2) {  // bfloat16 with many rows and a packed W: the kernel that streams its operands straight into LDS
+        if (ALIGNED && stream::takes(M, N, K, packed, scatter, sizeof(OutT))) {
+            stream::dispatch<OutT>(a, w, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks);
+            return;
+        }
+    }
     int tile = 0;
     {
         // measured on MI355X at GPT-2 sizes: many waves per block hide latency best; the large tile

@@ -185,7 +185,10 @@ def test_pack_matrix(K, rows, cols, src, dst, transpose):
 
 GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
                (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20),
-               (2100, 2010, 104), (4100, 2010, 40)]  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
+               (2100, 2010, 104), (4100, 2010, 40),  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
+               # K in whole tiles of 64, columns in whole pieces, 192 rows or more: in bfloat16 with a packed matrix the kernel that
+               # streams its operands into LDS (128 x 64 tiles with two and, from a K of 1,536, three stages; 128 x 128 from 256 tiles on)
+               (300, 136, 192), (193, 2008, 128), (2100, 264, 64), (700, 776, 320), (300, 72, 1600), (2100, 2008, 128), (192, 8, 64)]
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -269,7 +272,8 @@ def guarded(values, dtype, fill=float("nan")):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k", [(5, 37, 20), (1, 16, 8), (16, 130, 72), (40, 50, 200), (64, 100, 64), (70, 37, 24), (130, 200, 96),
-                                   (300, 260, 136), (33, 40, 21), (200, 70, 50), (3, 9000, 64)])
+                                   (300, 260, 136), (33, 40, 21), (200, 70, 50), (3, 9000, 64), (300, 264, 128), (200, 72, 64), (1000, 2056, 64),
+                                   (2050, 2056, 192)])
 def test_linear_reads_nothing_past_its_operands(K, dtype, m, n, k):
     # NaN guards right after every operand: an out-of-bounds read would poison the result; a known
     # value right after the output: nothing is written past it. Every kernel of the product: few
@@ -286,6 +290,16 @@ def test_linear_reads_nothing_past_its_operands(K, dtype, m, n, k):
     K.linear(xg, wg, bg, residual=rg, out=og)
     np.testing.assert_allclose(host(og), rounded(x) @ rounded(w).T + b + res, rtol=2e-5, atol=2e-5)
     assert (after == 123.0).all()
+    # the same with the matrix in the packed layout (its chunks hold zeros beyond the matrix, the rows of x do not)
+    og, after = guarded(np.zeros((m, n)), torch.float32, fill=123.0)
+    K.linear(xg, as_weight(K, w, dtype, True), bg, residual=rg, out=og)
+    np.testing.assert_allclose(host(og), rounded(x) @ rounded(w).T + b + res, rtol=2e-5, atol=2e-5)
+    assert (after == 123.0).all()
+    if dtype == torch.bfloat16:
+        ob, after = guarded(np.zeros((m, n)), torch.bfloat16, fill=123.0)
+        K.linear(xg, as_weight(K, w, dtype, True), bg, out=ob)
+        np.testing.assert_allclose(host(ob), rounded(x) @ rounded(w).T + b, rtol=1e-2, atol=1e-2)
+        assert (after == 123.0).all()
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
@@ -570,12 +584,15 @@ def test_operands_are_checked_on_the_host(K):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size", [(1, 4, 4, 16, 16), (9, 3, 3, 32, 64), (33, 6, 2, 48, 32), (64, 2, 1, 80, 16), (65, 3, 3, 32, 16), (300, 5, 5, 48, 64),
-                                                                         (2100, 14, 14, 48, 64)])  # enough rows and columns for the large tile
+@pytest.mark.parametrize("rows,n_heads,n_kv_heads,head_size,page_size,width", [
+    (1, 4, 4, 16, 16, 72), (9, 3, 3, 32, 64, 72), (33, 6, 2, 48, 32, 72), (64, 2, 1, 80, 16, 72), (65, 3, 3, 32, 16, 72), (300, 5, 5, 48, 64, 72),
+    (2100, 14, 14, 48, 64, 72),  # enough rows and columns for the large tile
+    # a width in whole tiles of 64: in bfloat16 with a packed matrix the kernel that streams its operands into LDS; heads of 40
+    # and 24 (a 16-byte piece of columns stays inside a head), grouped heads, and heads of 20 (it does not: the other kernel)
+    (300, 5, 5, 48, 64, 128), (700, 6, 2, 40, 32, 192), (2100, 14, 14, 24, 16, 64), (250, 3, 3, 20, 64, 64)])
 @pytest.mark.parametrize("packed", [False, True])
-def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, packed):
+def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, width, packed):
     rng = np.random.default_rng(rows)
-    width = 72
     qw, kvw = n_heads * head_size, n_kv_heads * head_size
     x, w, b = rng.standard_normal((rows, width)), rng.standard_normal((qw + 2 * kvw, width)) / 8, rng.standard_normal(qw + 2 * kvw)
     num_pages = max(8, rows // page_size + 2)
@@ -836,7 +853,8 @@ def test_layernorm_gives_the_summed_rows_too(K, out_dtype, with_bias):
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k,k_blocks", [(1, 40, 2048, 8), (20, 100, 1000, 3), (64, 1024, 1104, 4), (48, 200, 520, 2), (33, 16, 64, 16), (7, 50, 96, 1),
-                                            (65, 40, 2048, 4), (300, 130, 1000, 3), (129, 64, 520, 8), (200, 70, 96, 2)])
+                                            (65, 40, 2048, 4), (300, 130, 1000, 3), (129, 64, 520, 8), (200, 70, 96, 2),
+                                            (300, 136, 1024, 3), (513, 72, 640, 8), (2100, 776, 3072, 2)])
 def test_linear_split_leaves_partial_products(K, m, n, k, k_blocks, dtype, packed):
     # the product cut along K: the partial products add up to it, whatever the cut (also one that
     # leaves the last blocks without any k); up to 64 rows in the kernel for few rows, more in the tiled one
