@@ -721,6 +721,8 @@ void launch_prefill(const void* q, int q_stride, const void* k_pages, const void
 
 }  // namespace
 
+#include "attention_stream.h"
+
 // 1 if the matrix-core prefill kernel takes this head size and page size.
 MLLM_API int mllm_attention_prefill_supported(int head_size, int page_size) {
     bool page_ok = page_size > 0 && (page_size & (page_size - 1)) == 0;
@@ -746,6 +748,17 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
 #define MLLM_PREFILL_CASE(T, PAD)                                                                                      \
     launch_prefill<T, PAD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,      \
                            max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_shift, window, scale, stream)
+    if (dtype == MLLM_BF16 && prefill_stream::takes(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+        // long portions in bfloat16, heads of 32 / 64 / 128, pages of 32 keys or more: keys and values stream from the pages straight into LDS
+#define MLLM_STREAM_CASE(HD)                                                                                            \
+    prefill_stream::launch<HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
+                               max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
+        if (head_size == 32) MLLM_STREAM_CASE(32);
+        else if (head_size == 64) MLLM_STREAM_CASE(64);
+        else MLLM_STREAM_CASE(128);
+#undef MLLM_STREAM_CASE
+        return mllm_check_launch("attention_prefill");
+    }
     if (dtype == MLLM_F32) {
         if (padded == 32) MLLM_PREFILL_CASE(float, 32);
         else if (padded == 64) MLLM_PREFILL_CASE(float, 64);

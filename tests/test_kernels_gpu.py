@@ -399,6 +399,59 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
+    "n_heads,n_kv_heads,head_size,page_size,window",
+    [(3, 3, 32, 16, 0), (2, 2, 64, 64, 0), (4, 2, 64, 16, 150), (2, 1, 128, 8, 0), (2, 2, 128, 256, 0), (3, 3, 32, 32, 70),
+     (2, 2, 48, 32, 0), (5, 5, 64, 4, 0)],
+)
+def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head_size, page_size, window):
+    # portions of several query tiles over several key tiles, requests of different lengths in one call (one
+    # with a single token, one that starts at position 0, one whose portion ends one past a tile), pages
+    # scrambled and unwritten places holding NaN. In the longest request some queries look hard at one far
+    # key each (the first key, keys at the two sides of tile and page edges), so that a tile that is
+    # skipped, read twice or read from a wrong page shows in those rows.
+    rng = np.random.default_rng(head_size * 10 + page_size)
+    shapes = [(0, 300), (200, 129), (500, 1), (70, 65), (0, 2)]
+    need = sum((c + n + page_size - 1) // page_size for c, n in shapes)
+    num_pages = need + 5
+    order = rng.permutation(num_pages).tolist()
+    kp = torch.full((num_pages, n_kv_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
+    vp = torch.full_like(kp, float("nan"))
+    max_blocks = max((c + n + page_size - 1) // page_size for c, n in shapes)
+    tables = np.zeros((len(shapes), max_blocks), dtype=np.int32)
+    q_rows, treq, tpos, refs = [], [], [], []
+    rnd = lambda *s: bf16_round(rng.standard_normal(s)) if dtype == torch.bfloat16 else rng.standard_normal(s).astype(np.float32).astype(np.float64)
+    group = n_heads // n_kv_heads
+    for r, (ctx, new) in enumerate(shapes):
+        total = ctx + new
+        k_all, v_all = rnd(total, n_kv_heads * head_size), rnd(total, n_kv_heads * head_size)
+        q = rnd(new, n_heads * head_size)
+        if (ctx, new) == (0, 300):
+            for query, key in ((299, 0), (290, 63), (280, 64), (270, 127), (260, 128), (250, 191), (240, 192), (230, page_size - 1),
+                               (220, page_size), (131, 129), (128, 128), (127, 1), (200, 200 - 69), (210, 255), (211, 256)):
+                if window and query - key >= window:
+                    continue
+                far = q[query].reshape(n_heads, head_size)[::group].reshape(-1) * 4
+                k_all[key] = bf16_round(far) if dtype == torch.bfloat16 else far
+        n_blocks = (total + page_size - 1) // page_size
+        pages = [order.pop() for _ in range(n_blocks)]
+        tables[r, :n_blocks] = pages
+        slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+        K.cache_write(dev(k_all, dtype), dev(v_all, dtype), kp, vp, dev(slots, torch.int32), n_kv_heads, head_size)
+        q_rows.append(q)
+        treq += [r] * new
+        tpos += list(range(ctx, total))
+        refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window or None))
+    starts = np.cumsum([0] + [new for _, new in shapes])
+    out = K.paged_attention(
+        dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+        n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=300,
+        q_starts=dev(starts, torch.int32), context_lens=dev([c for c, _ in shapes], torch.int32))
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_over_a_block_table_of_more_than_a_thousand_pages(K, dtype):
     # 17,000 cached keys in pages of 16 (1,066 pages, scrambled): more than the 1,024 table entries
     # the prompt kernel keeps in LDS. A portion of 40 queries and a single decoded token; one far key
