@@ -151,7 +151,8 @@ def measure_kernels(engine, batch: int = 8, context: int = 768, reps: int = 7):
     between two events over all layers' weights in turn (as a step walks them), median of ``reps``:
     for a 2,048-token prompt step the four products of a layer and the prompt attention (flops /
     time / the matrix cores' peak), for a decode step of ``batch`` sequences at ``context`` tokens the
-    two halves of a layer and the head (the bytes each has to read / time / the memory's peak). The
+    two halves of a layer and the head (the bytes each has to read / time / the memory's peak); a time
+    holds the gap to the next kernel, as in a step. The
     reference prices its kernels the same way, against a pure read of the same bytes
     (docs/kernels/010_matvec_batch.md:20,108-117)."""
     import numpy as np
@@ -170,13 +171,22 @@ def measure_kernels(engine, batch: int = 8, context: int = 768, reps: int = 7):
     calls = [(model.blocks[call.block], cache.layer_context, call) for call in model.schedule]
 
     def timed(per_layer) -> float:
-        """Seconds of one call of per_layer(block, ctx), averaged over the layers."""
+        """Seconds of one call of per_layer(block, ctx), averaged over the layers. The calls over the layers are captured into
+        a graph and the replay is timed, as a step runs them: launched one by one the host's path through Python would count."""
+        def over_the_layers():
+            for block, context_of, call in calls:
+                per_layer(block, context_of(batch_of_step, call))
+
+        over_the_layers()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            over_the_layers()
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         samples = []
         for rep in range(reps + 2):
             start.record()
-            for block, context_of, call in calls:
-                per_layer(block, context_of(batch_of_step, call))
+            graph.replay()
             stop.record()
             torch.cuda.synchronize()
             samples.append(start.elapsed_time(stop) / 1e3 / len(calls))

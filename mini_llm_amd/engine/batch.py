@@ -123,6 +123,24 @@ class BatchStaging:
         return target
 
 
+class FixedBuffer:
+    """The device buffer that a captured step reads its batch from: made when the first batch is laid out into it,
+    and of that length from then on (a graph is replayed only for batches whose layout has the same length)."""
+
+    def __init__(self, device):
+        self.device = device
+        self.tensor = None
+
+    def take(self, n_ints: int):
+        import torch
+
+        if self.tensor is None:
+            self.tensor = torch.zeros(n_ints, dtype=torch.int32, device=self.device)
+        if n_ints != len(self.tensor):
+            raise ValueError(f"a batch of {n_ints} numbers does not fit the {len(self.tensor)} this buffer was made for")
+        return self.tensor
+
+
 def _aligned(n: int) -> int:
     return (n + 3) & ~3  # sections start on 16-byte boundaries
 
@@ -136,13 +154,16 @@ def _pad(array: np.ndarray, length: int, fill: int) -> np.ndarray:
 
 
 def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int, capacity: int | None = None,
-                     device_buffer=None, short_portion: int = SHORT_PORTION) -> StepBatch:
+                     device_buffer=None, short_portion: int = SHORT_PORTION, fixed_reach: bool = False) -> StepBatch:
     """Lays out the batch on the host and uploads it in one copy. The entries have been checked
     and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests).
 
     ``capacity`` pads the batch to that many tokens and requests with rows that do nothing (token
     -1, request -1, slot -1), so that the layout depends on the capacity alone; ``device_buffer``
-    then is the fixed device buffer the batch is copied into (a captured graph reads it).
+    then is the fixed device buffer the batch is copied into (a captured graph reads it); a
+    ``FixedBuffer`` is made to the batch's length at its first use. ``fixed_reach`` names the longest
+    sequence the cache can hold as the longest of this batch, as a padded batch does, so that nothing
+    a kernel launch is sized by depends on how far the requests have come.
 
     The requests are laid out short portions first (up to ``short_portion`` tokens); the logit rows
     keep the order of the entries as given."""
@@ -213,6 +234,8 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         flat = np.zeros(max(total, 4), dtype=np.int32)
         for offset, section in zip(offsets, sections):
             flat[offset : offset + len(section)] = section
+        if isinstance(device_buffer, FixedBuffer):
+            device_buffer = device_buffer.take(len(flat))
         device = staging.upload(flat, into=device_buffer)
         views = [device[o : o + len(s)] for o, s in zip(offsets, sections)]
     groups = [
@@ -222,7 +245,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     return StepBatch(
         n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
         short_requests=short_requests, short_rows=short_rows,
-        max_total_len=max_total if capacity is None else (cache.max_length or table_width * cache.page_size),
+        max_total_len=max_total if capacity is None and not fixed_reach else (cache.max_length or table_width * cache.page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
         request_ids=[e.request_id for e in entries], host=host, short_portion=short_portion,

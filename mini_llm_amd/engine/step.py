@@ -10,16 +10,26 @@ after the step has been launched (engine/src/gpt2_gpu.cu:364).
 A step in which every request brings one token and wants its logits (a decode step) is
 launch-bound, as the reference found (docs/kernels/007_fewer_launches.md): it is captured once
 per batch-size bucket in a HIP graph and replayed; the batch's metadata lies in a fixed device
-buffer per bucket that is overwritten before each replay."""
+buffer per bucket that is overwritten before each replay. Steps with portions of prompts are
+captured too, per shape of batch, once a shape has come twice: up to a few thousand tokens of a
+small model the host needs longer to launch the kernels than the GPU to run them."""
 
 from __future__ import annotations
+
+from collections import OrderedDict
 
 import numpy as np
 
 from ..cache import CacheManager, OutOfPages
-from .batch import BatchStaging, DecodeBatchBuilder, StepBatch, StepEntry, build_step_batch
+from .batch import BatchStaging, DecodeBatchBuilder, FixedBuffer, StepBatch, StepEntry, build_step_batch
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+# Steps with portions of prompts: a step of a few thousand tokens of a small model is over on the GPU before the host has
+# launched its kernels one by one, so a shape of batch that comes again is captured too. Larger steps are bound by the GPU
+# and would only hold their activations' memory; so many shapes are kept, the least recently used one going first.
+PORTION_GRAPH_MAX_TOKENS = 8192
+PORTION_GRAPHS_KEPT = 8
+PORTION_SHAPES_COUNTED = 4096
 
 
 class StepError(ValueError):
@@ -40,26 +50,60 @@ class _DecodeGraph:
         self.logits = None
 
     def run(self, entries):
-        import torch
-
         runner = self.runner
         runner.staging.upload(self.builder.fill(entries), into=self.buffer)
         batch = self.static_batch
         batch.request_ids = [e.request_id for e in entries]
         if self.graph is None:
-            # once eagerly (on a side stream, as capture needs), then the capture itself
-            side = torch.cuda.Stream(device=runner.device)
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                runner.forward(batch)
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize(runner.device)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = runner.forward(batch)
-            self.graph = graph
+            self.graph, self.logits = _capture(runner, batch)
         self.graph.replay()
         return batch, self.logits[: len(entries)]
+
+
+def _capture(runner, batch):
+    """Runs the batch once eagerly (on a side stream, as capture needs), then captures the same."""
+    import torch
+
+    side = torch.cuda.Stream(device=runner.device)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        runner.forward(batch)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize(runner.device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        logits = runner.forward(batch)
+    return graph, logits
+
+
+class _PortionGraph:
+    """One captured step for batches of one shape: so many tokens, requests and wanted places, the same longest portion and
+    the same cut between short and long portions. Everything else about a batch (tokens, positions, pages, which rows are
+    wanted) lies in the device buffer that the kernels read, and is overwritten before each replay."""
+
+    def __init__(self, runner: "ModelRunner"):
+        self.runner = runner
+        self.buffer = FixedBuffer(runner.device)
+        self.graph = None
+        self.logits = None
+        self.batch = None
+
+    def run(self, entries):
+        runner = self.runner
+        batch = build_step_batch(entries, runner.cache, runner.staging, vocab_size=runner.model.vocab_size, device_buffer=self.buffer,
+                                 short_portion=runner.model.short_portion(), fixed_reach=True)
+        if self.graph is None:
+            self.graph, self.logits = _capture(runner, batch)
+            self.batch = batch
+        else:  # the captured kernels read the first batch's views of the buffer, which now holds this batch
+            captured = self.batch
+            same = (captured.n_tokens, captured.n_requests, captured.n_logit_rows, captured.max_q_len, captured.short_requests,
+                    captured.short_rows, captured.max_total_len) == (batch.n_tokens, batch.n_requests, batch.n_logit_rows,
+                                                                      batch.max_q_len, batch.short_requests, batch.short_rows, batch.max_total_len)
+            if not same:
+                raise RuntimeError("a captured step was asked to run a batch of another shape")
+        self.graph.replay()
+        return batch, self.logits
 
 
 class ModelRunner:
@@ -71,6 +115,9 @@ class ModelRunner:
         self.last_batch: StepBatch | None = None
         self.use_graphs = bool(use_graphs and device is not None and cache.max_length is not None and model.all_graph_safe())
         self._graphs: dict = {}
+        self._portion_graphs: OrderedDict = OrderedDict()   # shape of batch -> _PortionGraph, least recently used first
+        self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
+        self.portion_graph_steps = 0
 
     @staticmethod
     def _check_tokens(entry, vocab: int) -> None:
@@ -126,14 +173,39 @@ class ModelRunner:
         return self.model.forward(batch, self.cache, resolve_tokens=resolve, observer=observer)
 
     def _graph_for(self, entries):
-        if not self.use_graphs or len(entries) > GRAPH_BUCKETS[-1]:
+        if not self.use_graphs:
             return None
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return self._portion_graph_for(entries)
+        if len(entries) > GRAPH_BUCKETS[-1]:
             return None
         capacity = next(b for b in GRAPH_BUCKETS if b >= len(entries))
         if capacity not in self._graphs:
             self._graphs[capacity] = _DecodeGraph(self, capacity)
         return self._graphs[capacity]
+
+    def _portion_graph_for(self, entries):
+        """The captured step for batches of this shape, once the shape has come a second time."""
+        short = self.model.short_portion()
+        lengths = [len(e.tokens) for e in entries]
+        n_tokens = sum(lengths)
+        if n_tokens > PORTION_GRAPH_MAX_TOKENS:
+            return None
+        shape = (n_tokens, len(entries), sum(len(e.want) for e in entries), max(lengths),
+                 sum(1 for n in lengths if n <= short), sum(n for n in lengths if n <= short))
+        graph = self._portion_graphs.get(shape)
+        if graph is not None:
+            self._portion_graphs.move_to_end(shape)
+            return graph
+        if len(self._shapes_seen) >= PORTION_SHAPES_COUNTED:
+            self._shapes_seen.clear()
+        self._shapes_seen[shape] = self._shapes_seen.get(shape, 0) + 1
+        if self._shapes_seen[shape] < 2:
+            return None
+        while len(self._portion_graphs) >= PORTION_GRAPHS_KEPT:
+            self._portion_graphs.popitem(last=False)
+        graph = self._portion_graphs[shape] = _PortionGraph(self)
+        return graph
 
     def step(self, entries: list[StepEntry], observer=None):
         """Runs the entries as one batch. Returns float32 logits [wanted places, vocab] on the
@@ -156,7 +228,10 @@ class ModelRunner:
             graph = self._graph_for(entries) if observer is None else None
             if graph is not None:
                 batch, logits = graph.run(entries)
-                self.graph_steps += 1
+                if isinstance(graph, _PortionGraph):
+                    self.portion_graph_steps += 1
+                else:
+                    self.graph_steps += 1
             else:
                 batch = build_step_batch(entries, self.cache, self.staging, vocab_size=self.model.vocab_size, short_portion=self.model.short_portion())
                 in_given_order = None

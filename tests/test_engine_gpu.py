@@ -295,6 +295,58 @@ def test_graph_replays_match_eager_steps(model_dirs, dtype):
         assert results[True][name].keys() == results[False][name].keys()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
+    # steps with portions of prompts whose shape of batch comes again (so many tokens, requests and wanted places) are
+    # captured at the second time and replayed from the third: here the same shapes come with other requests, at other
+    # depths of the cache and with other places wanted, with decode replays, eager steps of other shapes and
+    # synchronisations between them; every step is checked against the plain implementation, with and without graphs
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    folder, config, weights = model_dirs["C"]
+    vocab = config["vocab_size"]
+    seqs = {name: random_tokens(80 + i, 190, vocab) for i, name in enumerate("abcdef")}
+    import replay
+
+    ref = replay.plain_logits(config, weights, seqs, bf16=(dtype == "bfloat16"))
+    tol = replay.tolerance(dtype)
+    for use_graphs in (True, False):
+        engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=8, max_tokens=2048, use_graphs=use_graphs))
+        handles = {name: engine.try_take_cache() for name in seqs}
+        fed = {name: 0 for name in seqs}
+        checked = 0
+
+        def run(step):
+            nonlocal checked
+            entries = [StepEntry(handles[name], seqs[name][fed[name] : fed[name] + n], list(want)) for name, n, want in step]
+            logits = engine.runner.step(entries).cpu().numpy()
+            row = 0
+            for name, n, want in step:
+                for w in want:
+                    np.testing.assert_allclose(logits[row], ref[name][fed[name] + w], err_msg=f"{name} {fed[name] + w} graphs={use_graphs}", **tol)
+                    row += 1
+                    checked += 1
+                fed[name] += n
+
+        # shape X: 30 + 1 tokens, two requests, two places wanted; shape Y: 40 + 20 + 2 tokens, three wanted
+        run([("a", 30, [29]), ("b", 1, [0])])                     # X, first time: eager
+        run([("c", 40, [39]), ("d", 20, [5]), ("e", 2, [1])])     # Y, first time: eager
+        run([("b", 30, [0]), ("a", 1, [0])])                      # X again, the long portion first: captured here
+        run([("e", 40, [7]), ("c", 20, [19]), ("f", 2, [0])])     # Y again: captured here
+        run([("a", 1, [0]), ("b", 1, [0])])                       # a decode step between
+        torch.cuda.synchronize()
+        run([("f", 30, [10]), ("d", 1, [0])])                     # X replayed, deeper in the cache
+        run([("d", 33, [32])])                                    # another shape: eager
+        run([("a", 40, [39]), ("b", 20, [0]), ("d", 2, [1])])     # Y replayed
+        run([("c", 30, [29]), ("e", 1, [0])])                     # X replayed
+        torch.cuda.synchronize()
+        run([("f", 40, [0]), ("e", 20, [19]), ("c", 2, [0])])     # Y replayed
+        run([("a", 30, [3]), ("f", 1, [0])])                      # X replayed
+        assert checked == 2 * 5 + 3 * 4 + 2 + 1
+        assert engine.runner.portion_graph_steps == (7 if use_graphs else 0)
+
+
 def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
     # step n+1 is launched before the host has read token n; the tokens must be those of the
     # step-by-step calls and of the plain implementation (the reference's queued mode:
