@@ -211,8 +211,9 @@ class Engine:
         self.close()
 
     def close(self) -> None:
-        """Whatever is still live or waiting ends with an error; its pages go back."""
+        """Whatever is still live or waiting ends with an error; its pages go back, and so do the captured steps."""
         self.scheduler.shutdown()
+        self.runner.drop_graphs()
 
     # --- one sequence at a time (native.py) ---------------------------------------------------------
     def forward_last(self, token_ids) -> np.ndarray:

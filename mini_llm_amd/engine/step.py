@@ -16,6 +16,8 @@ small model the host needs longer to launch the kernels than the GPU to run them
 
 from __future__ import annotations
 
+import gc
+from array import array as _array
 from collections import OrderedDict
 
 import numpy as np
@@ -71,8 +73,18 @@ def _capture(runner, batch):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize(runner.device)
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        logits = runner.forward(batch)
+    # No garbage collection while the stream is being captured: it may finalise whatever lies around in reference
+    # cycles, another engine's captured graphs among them, and giving their memory back is not permitted during a
+    # capture (the process aborts). Collected before instead, and switched back on behind the capture.
+    gc.collect()
+    collecting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            logits = runner.forward(batch)
+    finally:
+        if collecting:
+            gc.enable()
     return graph, logits
 
 
@@ -119,6 +131,14 @@ class ModelRunner:
         self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
         self.portion_graph_steps = 0
 
+    def drop_graphs(self) -> None:
+        """Gives the captured steps back now (they and the runner refer to each other, so otherwise they would lie around
+        until the garbage collector finds them)."""
+        for graph in list(self._graphs.values()) + list(self._portion_graphs.values()):
+            graph.runner = None
+        self._graphs.clear()
+        self._portion_graphs.clear()
+
     @staticmethod
     def _check_tokens(entry, vocab: int) -> None:
         """Every token an integer inside the vocabulary: a long portion is looked at as one array, and
@@ -126,10 +146,14 @@ class ModelRunner:
         tokens = entry.tokens
         entry.checked_tokens = None   # whatever an earlier step left: the list may have changed since
         if len(tokens) > 16:
-            try:
-                array = np.asarray(tokens)
-            except (ValueError, TypeError, OverflowError):
-                array = None
+            array = None
+            if isinstance(tokens, np.ndarray):
+                array = tokens
+            elif isinstance(tokens, list):
+                try:   # a third faster than numpy's own conversion of a list; anything but integers that fit is left to the loop below
+                    array = np.frombuffer(_array("i", tokens), dtype=np.int32)
+                except (ValueError, TypeError, OverflowError):
+                    array = None
             if array is not None and array.ndim == 1 and array.dtype.kind in "iu" and 0 <= int(array.min()) and int(array.max()) < vocab:
                 entry.checked_tokens = array.astype(np.int32, copy=False)
                 return
