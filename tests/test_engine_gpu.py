@@ -347,6 +347,36 @@ def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
         assert engine.runner.portion_graph_steps == (7 if use_graphs else 0)
 
 
+def test_no_garbage_collection_while_a_step_is_captured():
+    # the collector may finalise another engine's captured graphs, and giving memory back inside a capture aborts the
+    # process: it is off from the start of a capture to its end, and as it was again afterwards
+    import gc
+
+    from mini_llm_amd.engine.step import _capture
+
+    class Runner:
+        device = "cuda:0"
+        seen = []
+
+        def forward(self, batch):
+            self.seen.append(gc.isenabled())
+            return torch.ones(4, device="cuda:0") * 2
+
+    runner = Runner()
+    assert gc.isenabled()
+    graph, logits = _capture(runner, None)
+    assert runner.seen == [True, False] and gc.isenabled()   # the eager run first, then the capture
+    graph.replay()
+    torch.cuda.synchronize()
+    assert logits.tolist() == [2.0, 2.0, 2.0, 2.0]
+    gc.disable()
+    try:
+        _capture(runner, None)
+        assert not gc.isenabled()   # left as it was found
+    finally:
+        gc.enable()
+
+
 def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
     # step n+1 is launched before the host has read token n; the tokens must be those of the
     # step-by-step calls and of the plain implementation (the reference's queued mode:
