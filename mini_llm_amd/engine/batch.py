@@ -18,7 +18,7 @@ class StepEntry:
     among them whose logits are wanted."""
 
     request_id: object
-    tokens: list
+    tokens: list   # of integers, or a one-dimensional integer array
     want: list = field(default_factory=list)
     # The (single) token is the one the sampler left in the request's last-token slot on the
     # device in an earlier step; ``tokens`` then holds a placeholder the host never looks at.
@@ -145,14 +145,6 @@ def _aligned(n: int) -> int:
     return (n + 3) & ~3  # sections start on 16-byte boundaries
 
 
-def _pad(array: np.ndarray, length: int, fill: int) -> np.ndarray:
-    if len(array) >= length:
-        return array
-    out = np.full(length, fill, dtype=np.int32)
-    out[: len(array)] = array
-    return out
-
-
 def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int, capacity: int | None = None,
                      device_buffer=None, short_portion: int = SHORT_PORTION, fixed_reach: bool = False) -> StepBatch:
     """Lays out the batch on the host and uploads it in one copy. The entries have been checked
@@ -176,76 +168,92 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     short_requests = sum(1 for q in q_lens if q <= short_portion)
     short_rows = sum(q for q in q_lens if q <= short_portion)
     n_tokens = sum(q_lens)
-    contexts = [cache.length(e.request_id) for e in entries]
+    records = [cache.requests[e.request_id] for e in entries]
+    contexts = [r.length for r in records]
     n_groups = len(cache.groups)
+    page_size = cache.page_size
     max_total = max(c + q for c, q in zip(contexts, q_lens))
-    table_width = cache.max_blocks() or max(1, -(-max_total // cache.page_size))
+    table_width = cache.max_blocks() or max(1, -(-max_total // page_size))
     cap_tokens = n_tokens if capacity is None else capacity
     cap_requests = n_requests if capacity is None else capacity
     if n_tokens > cap_tokens or n_requests > cap_requests:
         raise ValueError("the batch exceeds the capacity it is laid out for")
+    n_logit_rows = sum(len(e.want) for e in entries)
+    logit_length = n_logit_rows if capacity is None else max(n_logit_rows, cap_tokens)
 
-    tokens = np.concatenate([e.token_array() for e in entries])
-    positions = np.concatenate([np.arange(c, c + q, dtype=np.int32) for c, q in zip(contexts, q_lens)])
-    token_request = np.repeat(np.arange(n_requests, dtype=np.int32), q_lens)
-    q_starts = np.full(cap_requests + 1, n_tokens, dtype=np.int32)
-    q_starts[0] = 0
-    q_starts[1 : n_requests + 1] = np.cumsum(q_lens)
-    logit_rows = np.asarray([q_starts[place[i]] + w for i, e in enumerate(given) for w in e.want], dtype=np.int32)
-    state_slots = np.asarray([cache.requests[e.request_id].state_slot for e in entries], dtype=np.int32)
-    token_sources = np.full(cap_tokens, -1, dtype=np.int32)
+    # One flat array, its sections starting on 16-byte boundaries, filled in place (no section is built apart and copied):
+    # tokens, positions, token_request, q_starts, context_lens, state_slots, logit_rows, token_sources,
+    # (block table, slots) per cache group, logit_slots.
+    lengths = [cap_tokens, cap_tokens, cap_tokens, cap_requests + 1, cap_requests, cap_requests, logit_length, cap_tokens]
+    for _ in range(n_groups):
+        lengths += [cap_requests * table_width, cap_tokens]
+    lengths.append(logit_length)
+    offsets, total = [], 0
+    for length in lengths:
+        offsets.append(total)
+        total += _aligned(length)
+    flat = np.zeros(max(total, 4), dtype=np.int32)
+    sections = [flat[o : o + n] for o, n in zip(offsets, lengths)]
+    tokens, positions, token_request, q_starts, context_lens, state_slots, logit_rows, token_sources = sections[:8]
+
+    starts = [0]
+    for q in q_lens:
+        starts.append(starts[-1] + q)
+    tokens[n_tokens:] = -1
+    token_request[n_tokens:] = -1
+    token_sources[:] = -1
+    q_starts[: n_requests + 1] = starts
+    q_starts[n_requests + 1 :] = n_tokens
+    context_lens[:n_requests] = contexts
+    state_slots[:n_requests] = [r.state_slot for r in records]
     for i, e in enumerate(entries):
+        lo, hi = starts[i], starts[i + 1]
+        tokens[lo:hi] = e.token_array()
+        positions[lo:hi] = np.arange(contexts[i], contexts[i] + q_lens[i], dtype=np.int32)
+        token_request[lo:hi] = i
         if e.from_slot:
-            token_sources[q_starts[i]] = state_slots[i]
+            token_sources[lo] = records[i].state_slot
     tables, slots = [], []
     for gi in range(n_groups):
-        table = np.full((cap_requests, table_width), -1, dtype=np.int32)
-        slot = np.full(cap_tokens, -1, dtype=np.int32)
+        table = sections[8 + 2 * gi].reshape(cap_requests, table_width)
+        slot = sections[9 + 2 * gi]
+        table[:] = -1
+        slot[n_tokens:] = -1
         for i, e in enumerate(entries):
+            lo, hi = starts[i], starts[i + 1]
             pages = np.asarray(cache.block_table(e.request_id, gi), dtype=np.int32)
             table[i, : len(pages)] = pages
-            pos = positions[q_starts[i] : q_starts[i + 1]]
-            slot[q_starts[i] : q_starts[i + 1]] = pages[pos // cache.page_size] * cache.page_size + pos % cache.page_size
+            pos = positions[lo:hi]
+            slot[lo:hi] = pages[pos // page_size] * page_size + pos % page_size
         tables.append(table)
         slots.append(slot)
-    logit_slots = np.asarray([state_slots[place[i]] for i, e in enumerate(given) for _ in e.want], dtype=np.int32)
-    n_logit_rows = len(logit_rows)
-    if capacity is not None:
-        logit_rows = _pad(logit_rows, cap_tokens, 0)
-        logit_slots = _pad(logit_slots, cap_tokens, 0)
+    logit_slots = sections[-1]
+    at = 0
+    for i, e in enumerate(given):
+        for w in e.want:
+            logit_rows[at] = starts[place[i]] + w
+            logit_slots[at] = records[place[i]].state_slot
+            at += 1
 
-    sections = [_pad(tokens, cap_tokens, -1), _pad(positions, cap_tokens, 0), _pad(token_request, cap_tokens, -1), q_starts,
-                _pad(np.asarray(contexts, dtype=np.int32), cap_requests, 0), _pad(state_slots, cap_requests, 0), logit_rows,
-                token_sources]
-    for table, slot in zip(tables, slots):
-        sections += [table.reshape(-1), slot]
-    sections.append(logit_slots)
-    offsets, total = [], 0
-    for section in sections:
-        offsets.append(total)
-        total += _aligned(len(section))
-    host = {"tokens": tokens, "positions": positions, "token_request": token_request, "q_starts": q_starts[: n_requests + 1],
-            "context_lens": sections[4][:n_requests], "state_slots": state_slots, "logit_rows": logit_rows[:n_logit_rows],
-            "token_sources": token_sources[:n_tokens], "logit_slots": logit_slots[:n_logit_rows],
+    host = {"tokens": tokens[:n_tokens], "positions": positions[:n_tokens], "token_request": token_request[:n_tokens],
+            "q_starts": q_starts[: n_requests + 1], "context_lens": context_lens[:n_requests], "state_slots": state_slots[:n_requests],
+            "logit_rows": logit_rows[:n_logit_rows], "token_sources": token_sources[:n_tokens], "logit_slots": logit_slots[:n_logit_rows],
             "block_tables": tables, "slots": slots}
     if staging is None:
         views = sections
     else:
-        flat = np.zeros(max(total, 4), dtype=np.int32)
-        for offset, section in zip(offsets, sections):
-            flat[offset : offset + len(section)] = section
         if isinstance(device_buffer, FixedBuffer):
             device_buffer = device_buffer.take(len(flat))
         device = staging.upload(flat, into=device_buffer)
-        views = [device[o : o + len(s)] for o, s in zip(offsets, sections)]
+        views = [device[o : o + n] for o, n in zip(offsets, lengths)]
     groups = [
         GroupStepData(block_tables=views[8 + 2 * gi].reshape(cap_requests, table_width), slots=views[9 + 2 * gi])
         for gi in range(n_groups)
     ]
     return StepBatch(
-        n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=len(logit_rows), max_q_len=max(q_lens),
+        n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=logit_length, max_q_len=max(q_lens),
         short_requests=short_requests, short_rows=short_rows,
-        max_total_len=max_total if capacity is None and not fixed_reach else (cache.max_length or table_width * cache.page_size),
+        max_total_len=max_total if capacity is None and not fixed_reach else (cache.max_length or table_width * page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
         request_ids=[e.request_id for e in entries], host=host, short_portion=short_portion,
