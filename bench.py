@@ -131,7 +131,10 @@ def measure_prefill(engine, runs: int = 5):
     # would be turned into one first, 25 us a thousand tokens)
     prompts = [rng.integers(0, engine.config.vocab_size, n).astype(np.int32) for n in lengths]
     times = []
-    for _ in range(runs + 2):
+    # a shape of step that keeps coming is replayed from a captured graph; the warm-up runs go past the capture
+    warm = 2 + max(0, engine.runner.portion_graph_after if engine.runner.use_graphs else 0)
+    replayed_before = engine.runner.portion_graph_steps
+    for _ in range(runs + warm):
         handles = [engine.try_take_cache() for _ in prompts]
         entries = [StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)]
         torch.cuda.synchronize()
@@ -141,11 +144,11 @@ def measure_prefill(engine, runs: int = 5):
         times.append(time.perf_counter() - begin)
         for h in handles:
             engine.release_cache(h)
-    seconds = float(np.median(times[2:]))
+    seconds = float(np.median(times[warm:]))
     tokens = sum(lengths)
     flops = prefill_flops(engine.config, lengths, len(prompts))
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(seconds * 1e3, 3),
-            "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4)}
+            "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4), "from_graph": engine.runner.portion_graph_steps - replayed_before >= runs}
 
 
 def measure_kernels(engine, batch: int = 8, context: int = 768, reps: int = 7):

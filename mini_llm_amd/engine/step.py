@@ -11,7 +11,7 @@ A step in which every request brings one token and wants its logits (a decode st
 launch-bound, as the reference found (docs/kernels/007_fewer_launches.md): it is captured once
 per batch-size bucket in a HIP graph and replayed; the batch's metadata lies in a fixed device
 buffer per bucket that is overwritten before each replay. Steps with portions of prompts are
-captured too, per shape of batch, once a shape has come twice: up to a few thousand tokens of a
+captured too, per shape of batch, once a shape has come many times: up to a few thousand tokens of a
 small model the host needs longer to launch the kernels than the GPU to run them."""
 
 from __future__ import annotations
@@ -27,8 +27,13 @@ from .batch import BatchStaging, DecodeBatchBuilder, FixedBuffer, StepBatch, Ste
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 # Steps with portions of prompts: a step of a few thousand tokens of a small model is over on the GPU before the host has
-# launched its kernels one by one, so a shape of batch that comes again is captured too. Larger steps are bound by the GPU
-# and would only hold their activations' memory; so many shapes are kept, the least recently used one going first.
+# launched its kernels one by one, so a shape of batch that keeps coming is captured too. A capture costs about 45 ms
+# (measured; most of it making the graph ready to launch) and a replay saves some tenths of a millisecond, so a shape has to
+# come PORTION_GRAPH_AFTER times before it is captured: the shapes of a serving run with a mixed load change from step to
+# step and would each be captured for nothing (measured with a capture at the second time: 7.5k generated tokens a second
+# against 28.6k without). Larger steps are bound by the GPU and would only hold their activations' memory; so many shapes
+# are kept, the least recently used one going first.
+PORTION_GRAPH_AFTER = 32
 PORTION_GRAPH_MAX_TOKENS = 8192
 PORTION_GRAPHS_KEPT = 8
 PORTION_SHAPES_COUNTED = 4096
@@ -119,7 +124,9 @@ class _PortionGraph:
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, device, use_graphs: bool = True):
+    def __init__(self, model, cache: CacheManager, device, use_graphs: bool = True, portion_graph_after: int | None = None):
+        """``portion_graph_after``: the time a shape of batch with portions of prompts has to come to be captured (None: the
+        default, PORTION_GRAPH_AFTER; 0: never)."""
         self.model, self.cache, self.device = model, cache, device
         self.staging = BatchStaging(device) if device is not None else None
         self.steps_run = 0
@@ -129,6 +136,7 @@ class ModelRunner:
         self._graphs: dict = {}
         self._portion_graphs: OrderedDict = OrderedDict()   # shape of batch -> _PortionGraph, least recently used first
         self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
+        self.portion_graph_after = PORTION_GRAPH_AFTER if portion_graph_after is None else int(portion_graph_after)
         self.portion_graph_steps = 0
 
     def drop_graphs(self) -> None:
@@ -209,7 +217,9 @@ class ModelRunner:
         return self._graphs[capacity]
 
     def _portion_graph_for(self, entries):
-        """The captured step for batches of this shape, once the shape has come a second time."""
+        """The captured step for batches of this shape, once the shape has come often enough."""
+        if self.portion_graph_after <= 0:
+            return None
         short = self.model.short_portion()
         lengths = [len(e.tokens) for e in entries]
         n_tokens = sum(lengths)
@@ -224,7 +234,7 @@ class ModelRunner:
         if len(self._shapes_seen) >= PORTION_SHAPES_COUNTED:
             self._shapes_seen.clear()
         self._shapes_seen[shape] = self._shapes_seen.get(shape, 0) + 1
-        if self._shapes_seen[shape] < 2:
+        if self._shapes_seen[shape] < self.portion_graph_after:
             return None
         while len(self._portion_graphs) >= PORTION_GRAPHS_KEPT:
             self._portion_graphs.popitem(last=False)

@@ -297,8 +297,8 @@ def test_graph_replays_match_eager_steps(model_dirs, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
-    # steps with portions of prompts whose shape of batch comes again (so many tokens, requests and wanted places) are
-    # captured at the second time and replayed from the third: here the same shapes come with other requests, at other
+    # steps with portions of prompts whose shape of batch keeps coming (so many tokens, requests and wanted places) are
+    # captured (here at the second time, by option) and replayed from then on: here the same shapes come with other requests, at other
     # depths of the cache and with other places wanted, with decode replays, eager steps of other shapes and
     # synchronisations between them; every step is checked against the plain implementation, with and without graphs
     from mini_llm_amd.engine import StepEntry
@@ -312,7 +312,7 @@ def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
     ref = replay.plain_logits(config, weights, seqs, bf16=(dtype == "bfloat16"))
     tol = replay.tolerance(dtype)
     for use_graphs in (True, False):
-        engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=8, max_tokens=2048, use_graphs=use_graphs))
+        engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=8, max_tokens=2048, use_graphs=use_graphs, portion_graph_after=2))
         handles = {name: engine.try_take_cache() for name in seqs}
         fed = {name: 0 for name in seqs}
         checked = 0
