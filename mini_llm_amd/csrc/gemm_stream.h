@@ -3,19 +3,30 @@
 //
 // What the kernel is built around, each measured on MI355X:
 //  * Operands go from memory to LDS directly (global_load_lds_dwordx4: a wave's load lands as 1 KiB
-//    of consecutive LDS in lane order), one or two tiles of K ahead of the products, and cost no
-//    registers. Which bytes a lane asks for is therefore what lays the tile out in LDS. A chunk of
-//    the packed W is taken as it lies. For the row-major A, four lanes read the 64 bytes a row has in
-//    a chunk, so that a quarter wave touches 4 cache lines (a lane per row touched 16, and the
-//    lookups in the vector cache, not the bytes, bounded the kernel: 27 -> 17 us at 2,048 x 2,304 x
-//    768); a row's four pieces lie in LDS rotated by the row (piece ^ (row / 4) % 4), so that the
+//    of consecutive LDS in lane order) and cost no registers. Which bytes a lane asks for is therefore
+//    what lays the tile out in LDS. A chunk of the packed W is taken as it lies. For the row-major A,
+//    four lanes read the 64 bytes a row has in a chunk, so that a quarter wave touches 4 cache lines
+//    (a lane per row touched 16, and the lookups in the vector cache, not the bytes, bounded the
+//    kernel); a row's four pieces lie in LDS rotated by the row (piece ^ (row / 4) % 4), so that the
 //    sixteen lanes of a fragment read fall on sixteen different groups of banks.
-//  * A wave owns 64 x 64 outputs or more: at 32 x 32 every matrix instruction needs two fragment
-//    reads of its own and the LDS, not the matrix cores, sets the pace.
+//  * A block has a compute unit to itself and a wave a SIMD: whatever a wave waits for, its matrix
+//    core waits for too. So a wave owns 64 x 64 outputs or more (at 64 x 32 the fragment reads, not
+//    the products, set the pace); fragments are asked for two steps of K before their products; a
+//    tile's loads from memory go out a few at a time between the products of earlier tiles (a compute
+//    unit takes a load of 1 KiB every 16 cycles or so: a wave that issues a whole tile's loads at
+//    once stands still meanwhile); and the order of all this is pinned (sched_barrier), because left
+//    alone the compiler gathers a tile's reads in front of the barrier and its products behind it.
+//  * With loads into LDS under way the compiler can only wait for all LDS operations at once before
+//    the first use of any value read from LDS. The fragment reads are therefore inline assembly the
+//    compiler does not see through, with the wave's own counted waits.
+//  * The blocks of one XCD take the tiles of one rectangle of the output: the eight L2 caches then
+//    each fetch a part of A and W once (taking tiles in turn, every XCD reads nearly all of both:
+//    21.4 -> 18.3 us for 2,048 x 768 x 3,072).
 //  * W is the first operand of the matrix instruction: a lane then holds four consecutive columns
 //    of one row, and the epilogue, which goes through LDS once more, stores whole rows of a wave's
 //    tile in 16-byte pieces (stored as the accumulators lie, the same tile costs 6 us of an 18 us
-//    product).
+//    product). A lone wave pays every instruction of the epilogue in full: the kind of epilogue is a
+//    compile-time constant there, and a lane's place in the rows is a constant of the lane.
 //  * One barrier a tile. Before it a wave waits for its own fragment reads of the tile that is
 //    ending: the loads issued right after the barrier overwrite that tile's stage, and a fragment
 //    read still queued in the LDS unit would see the new tile (found as a wrong row in one product
@@ -23,6 +34,7 @@
 #pragma once
 
 #include <type_traits>
+#include <utility>
 
 namespace stream {
 
@@ -36,6 +48,50 @@ template <int N>
 __device__ __forceinline__ void wait_lgkmcnt() {
     // only the counter of LDS and scalar-memory operations (as a builtin, so that the compiler counts on it too)
     __builtin_amdgcn_s_waitcnt(0xF | (0x3 << 14) | (0x7 << 4) | ((N & 0xF) << 8));
+}
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_each(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant in its body
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_each(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// A fragment read the compiler does not know to be one: with loads into LDS under way it can only wait for every LDS
+// operation at once, before the first use of anything read from LDS, which ends all reading ahead. The value is in the
+// register once a wait of the wave's own (fragments_landed) has passed; until then nothing may read the register.
+template <int OFFSET>
+__device__ __forceinline__ void ask_fragment(i32x4& to, unsigned address) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(address), "n"(OFFSET));
+}
+// waits until at most IN_FLIGHT of the wave's LDS operations are under way (they complete in order; nothing else that
+// counts there is in flight inside the loop); the fragments named are only read after it
+template <int IN_FLIGHT>
+__device__ __forceinline__ void fragments_landed(i32x4& first) {
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(first) : "n"(IN_FLIGHT));
+}
+__device__ __forceinline__ void and_this_one(i32x4& fragment) { asm volatile("" : "+v"(fragment)); }
+__device__ __forceinline__ void still_written(const i32x4& fragment) { asm volatile("" : : "v"(fragment)); }
+
+// Eight rectangles of 'wide' x 'high' tiles, 'across' of them side by side along N, cover the tiles of the output.
+struct XcdTiles {
+    int across, wide, high;
+};
+// the split of the eight rectangles (1 x 8, 2 x 4, 4 x 2 or 8 x 1) whose rectangle needs the fewest rows of A and W together
+inline XcdTiles place_tiles(int tiles_m, int tiles_n, int bm, int bn) {
+    XcdTiles best{1, tiles_n, ceil_div(tiles_m, 8)};
+    long best_rows = -1;
+    for (int across = 1; across <= 8; across *= 2) {
+        const int wide = ceil_div(tiles_n, across), high = ceil_div(tiles_m, 8 / across);
+        const long rows = (long)wide * bn + (long)high * bm;
+        if (best_rows < 0 || rows < best_rows) best = XcdTiles{across, wide, high}, best_rows = rows;
+    }
+    return best;
 }
 
 template <typename OutT>
@@ -52,13 +108,13 @@ __device__ __forceinline__ void put4<bf16_t>(bf16_t* at, f32x4 v) {
     *reinterpret_cast<bf16x4*>(at) = o;
 }
 
-// grid (N tiles, M tiles, blocks along K). gridDim.z > 1: each block takes k_per_block of K (a multiple
-// of 64) and leaves a partial product in matrix blockIdx.z of `out` (float, no bias / epilogue / residual).
+// grid: one row of blocks, placed by 'places' (tiles and blocks along K). More than one block along K: each block takes k_per_block of K (a multiple
+// of 64) and leaves a partial product in matrix 'block_k' of `out` (float, no bias / epilogue / residual).
 // WAVES_K = 2: two waves share a tile of outputs and take half of every tile of K each; their sums meet in LDS at the end.
 template <typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, int WAVES_K, int STAGES>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, const float* __restrict__ bias, const float* __restrict__ residual,
-    OutT* __restrict__ out, int M, int N, int K, int epilogue, CacheScatter scatter, int k_per_block) {
+    OutT* __restrict__ out, int M, int N, int K, int epilogue, CacheScatter scatter, int k_per_block, XcdTiles places) {
     constexpr int NW = WAVES_M * WAVES_N * WAVES_K;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, FM = WM / 32, FN = WN / 32;
     constexpr int BK = 64, KS = BK / 16 / WAVES_K;           // steps of 16 along K a wave takes of a tile
@@ -79,11 +135,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
     const int tid = threadIdx.x, lane = tid % WAVE;
     const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
     const int wave_k = wave / (WAVES_M * WAVES_N), wave_m = wave / WAVES_N % WAVES_M, wave_n = wave % WAVES_N;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    const int k_begin = blockIdx.z * k_per_block, k_end = min(K, k_begin + k_per_block);
+    // Blocks go round the eight XCDs in turn, each with an L2 of its own: the blocks of one XCD take the tiles of one
+    // rectangle of the output, so that the rows of A and of W an XCD reads are few and each is fetched into its L2 once.
+    const int xcd = blockIdx.x % 8, in_xcd = blockIdx.x / 8;
+    const int block_k = in_xcd / (places.wide * places.high), in_rectangle = in_xcd % (places.wide * places.high);
+    const int tile_m = (xcd / places.across) * places.high + in_rectangle / places.wide;
+    const int tile_n = (xcd % places.across) * places.wide + in_rectangle % places.wide;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    if (m0 >= M || n0 >= N) return;  // (the rectangles cover more than the matrix; the whole block leaves)
+    const int k_begin = block_k * k_per_block, k_end = min(K, k_begin + k_per_block);
     const int k_steps = K / 32, n_tiles = (k_end - k_begin) / BK;
     const int w_row_tiles = (N + 15) / 16;
-    out += (size_t)blockIdx.z * M * N;
+    out += (size_t)block_k * M * N;
 
     // This wave's loads of a tile: load q = wave + NW * i of the stage, the first A_LPW of them from A. An address is a
     // base that all lanes share, which moves on with the tile, and a lane's own 32-bit offset.
@@ -179,65 +242,81 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
         // A 32 x 16 fragment: lane l holds row l % 32, k (l / 32) * 8 .. + 8. W: chunk [piece][row]; A: chunk [row][piece rotated].
         const int w_frag0 = BM * 128 + (wave_n * WN / 16) * 2048 + ((lane % 32) / 16) * 2048 + (lane / 32) * 256 + (lane % 16) * 16;
         const int a_row0 = (wave_m * WM / 16) * 2048 + ((lane % 32) / 16) * 2048 + (lane % 16) * 64, a_turn = ((lane % 16) >> 2) & 3;
-        const int kk0 = wave_k * KS;
-        bf16x8 a[2][FM], w[2][FN];
-        auto read_frags = [&](int set, const unsigned char* stage, int kk) {
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-                a[set][i] = *reinterpret_cast<const bf16x8*>(stage + a_row0 + i * 4096 + (kk / 2) * 1024 + ((((kk % 2) * 2 + lane / 32) ^ a_turn) * 16));
-#pragma unroll
-            for (int j = 0; j < FN; j++) w[set][j] = *reinterpret_cast<const bf16x8*>(stage + w_frag0 + j * 4096 + (kk / 2) * 1024 + (kk % 2) * 512);
+        // Fragments are asked for two steps before their products (four sets of registers): a step's reads come from all
+        // waves at once, and the LDS takes longer over them than one step's products last. A turn of the loop is four
+        // steps: one tile, or two where two waves share the tile's steps. Step g of a turn: wait for set g; then its products,
+        // and between them the reads of step g + 2 and the step's share of the loads of a tile further on.
+        constexpr int SETS = 4, TILES_A_TURN = SETS / KS, FRAGMENTS = FM + FN, PRODUCTS = FM * FN;
+        i32x4 a[SETS][FM], w[SETS][FN];
+        const unsigned a_lane[2] = {(unsigned)(a_row0 + wave_k * (KS / 2) * 1024 + (((0 + lane / 32) ^ a_turn) * 16)),
+                                    (unsigned)(a_row0 + wave_k * (KS / 2) * 1024 + (((2 + lane / 32) ^ a_turn) * 16))};
+        const unsigned w_lane = w_frag0 + wave_k * (KS / 2) * 1024;
+        auto ask = [&](auto set, auto step, auto fragment, unsigned stage_offset) {  // fragment 'fragment' of step 'step' of a tile
+            constexpr int SET = decltype(set)::value, S = decltype(step)::value, F = decltype(fragment)::value;
+            if constexpr (F < FM) ask_fragment<F * 4096 + (S / 2) * 1024>(a[SET][F], a_lane[S % 2] + stage_offset);
+            else ask_fragment<(F - FM) * 4096 + (S / 2) * 1024 + (S % 2) * 512>(w[SET][F - FM], w_lane + stage_offset);
         };
-        // The products of step s of a tile, and between them the step's share of the loads of the tile STAGES - 1 ahead:
-        // a compute unit takes a load of 1 KiB every 16 cycles or so, and a wave that issues all of a tile's loads at
-        // once stands still until the unit has taken them, its matrix core with it.
-        auto step_loads = [](int s) { return (s * LPW + KS - 1) / KS; };  // loads 'step_loads(s) .. step_loads(s + 1)' go with step s
-        auto products = [&](int set, int s, int load_tile, int load_stage) {
+        // The loads of tile u + STAGES go into the stage of tile u, between the barrier in tile u (which every wave passes
+        // with its reads of tile u done) and the barrier in tile u + 1: KS steps, each with its share.
+        auto share = [](int e) { return (e * LPW + KS - 1) / KS; };  // loads share(e) .. share(e + 1) go with step e after the barrier
+        auto stage_of = [](int tile) { return (tile % STAGES) * STAGE_BYTES; };
+
+        // before the loop: what the turns before the first would have asked for
+        constexpr int EARLY = (KS >= 2 ? 2 : KS);
 #pragma unroll
-            for (int j = 0; j < FN; j++)
-#pragma unroll
-                for (int i = 0; i < FM; i++) {
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w[set][j], a[set][i], acc[j][i], 0, 0, 0);
-                    constexpr int PER_STEP = FM * FN;
-                    const int first = step_loads(s), count = step_loads(s + 1) - first, slot = j * FM + i;
-                    // the step's loads spread over its products: after product 'slot' come loads slot*count/PER_STEP .. (slot+1)*count/PER_STEP
-#pragma unroll
-                    for (int l = slot * count / PER_STEP; l < (slot + 1) * count / PER_STEP; l++) issue_load(load_tile, load_stage, first + l);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-        };
-        // In flight when a tile ends: the whole tiles between the next one and the one being asked for, and of that one
-        // what the steps before the last have issued.
-        constexpr int IN_FLIGHT_AT_END = (STAGES - 3) * LPW + (KS - 1) * LPW / KS + ((KS - 1) * LPW % KS ? 1 : 0);
-        static_assert(STAGES >= 3, "a tile's loads are spread over the tile before the one before it");
-        wait_vmcnt<LPW*(STAGES - 2)>();
-        wait_lgkmcnt<0>();  // kernel arguments still on their way would make every wait for fragments in the loop a wait for all of them
+        for (int i = 0; i < LPW; i++)
+            if (i < share(EARLY)) issue_load(STAGES - 1, STAGES - 1, i);
+        wait_vmcnt<LPW*(STAGES - 2) + share(EARLY)>();
+        wait_lgkmcnt<0>();  // (kernel arguments)
         asm volatile("s_barrier" ::: "memory");
-        read_frags(0, lds, kk0);
-        // The order of a step is kept as written (the compiler otherwise gathers the reads of a whole tile in front of the
-        // barrier and the products behind it): the fragments of the next step are asked for, then this step's products
-        // are issued, and the reads travel while the matrix cores work. A step begins with the wait for its own
-        // fragments, asked for a step ago: with loads into LDS under way the compiler can only wait for every LDS
-        // operation at once, and left to place that wait itself it puts it behind the reads of the next step.
-        for (int t = 0; t < n_tiles; t++) {
-            const unsigned char* stage = lds + (t % STAGES) * STAGE_BYTES;
-            const int load_tile = t + STAGES - 1, load_stage = (t + STAGES - 1) % STAGES;  // the stage of tile t - 1, which every wave has left
-#pragma unroll
-            for (int s = 0; s + 1 < KS; s++) {
-                wait_lgkmcnt<0>();
+        static_for<2>([&](auto g) {
+            constexpr int G = decltype(g)::value;
+            static_for<FRAGMENTS>([&](auto f) { ask(g, std::integral_constant<int, G % KS>{}, f, stage_of(G / KS)); });
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < n_tiles; t += TILES_A_TURN) {
+            static_for<SETS>([&](auto g) {
+                constexpr int G = decltype(g)::value, S = G % KS;
+                const int tile = t + G / KS;
+                if (TILES_A_TURN > 1 && tile >= n_tiles) return;  // an odd count of tiles: the turn's second half falls away
+                if constexpr (S == KS - 2) {
+                    // the next tile has landed in every wave, and every wave has all its fragments of this one
+                    wait_vmcnt<LPW*(STAGES - 2)>();
+                    fragments_landed<0>(a[G][0]);
+                    asm volatile("s_barrier" ::: "memory");
+                } else {
+                    fragments_landed<FRAGMENTS>(a[G][0]);  // the reads of the step after this one may still travel
+                }
+                static_for<FM>([&](auto i) { if constexpr (decltype(i)::value > 0) and_this_one(a[G][decltype(i)::value]); });
+                static_for<FN>([&](auto j) { and_this_one(w[G][decltype(j)::value]); });
                 __builtin_amdgcn_sched_barrier(0);
-                read_frags((s + 1) % 2, stage, kk0 + s + 1);
-                __builtin_amdgcn_sched_barrier(0);
-                products(s % 2, s, load_tile, load_stage);
-            }
-            // the next tile has landed in every wave, and every wave has its last fragments of this one
-            wait_vmcnt<IN_FLIGHT_AT_END>();
-            wait_lgkmcnt<0>();
-            asm volatile("s_barrier" ::: "memory");
-            read_frags(KS % 2, lds + ((t + 1) % STAGES) * STAGE_BYTES, kk0);
-            __builtin_amdgcn_sched_barrier(0);
-            products((KS - 1) % 2, KS - 1, load_tile, load_stage);
+                constexpr int NEXT = G + 2, NEXT_SET = NEXT % SETS, NEXT_STEP = NEXT % KS;
+                const unsigned next_stage = stage_of(t + NEXT / KS);
+                // after the barrier of tile u: tile u + STAGES into the stage of tile u; before it: the rest of the tile before
+                constexpr int E = S >= KS - 2 ? S - (KS - 2) : S + 2;
+                const int load_into = S >= KS - 2 ? tile : tile - 1 + STAGES;  // (as a tile whose stage it is)
+                const int load_tile = S >= KS - 2 ? tile + STAGES : tile - 1 + STAGES;
+                static_for<PRODUCTS>([&](auto p) {
+                    constexpr int P = decltype(p)::value, J = P / FM, I = P % FM;
+                    acc[J][I] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&w[G][J]), *reinterpret_cast<bf16x8*>(&a[G][I]), acc[J][I], 0, 0, 0);
+                    static_for<(P + 1) * FRAGMENTS / PRODUCTS - P * FRAGMENTS / PRODUCTS>([&](auto f) {
+                        ask(std::integral_constant<int, NEXT_SET>{}, std::integral_constant<int, NEXT_STEP>{},
+                            std::integral_constant<int, P * FRAGMENTS / PRODUCTS + decltype(f)::value>{}, next_stage);
+                    });
+                    constexpr int COUNT = share(E + 1) - share(E);
+                    static_for<(P + 1) * COUNT / PRODUCTS - P * COUNT / PRODUCTS>([&](auto l) {
+                        issue_load(load_tile, load_into % STAGES, share(E) + P * COUNT / PRODUCTS + decltype(l)::value);
+                    });
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
         }
+        // the fragments asked for last are never used, but on their way into registers that must not be given away yet
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        static_for<SETS>([&](auto g) {
+            static_for<FM>([&](auto i) { still_written(a[decltype(g)::value][decltype(i)::value]); });
+            static_for<FN>([&](auto j) { still_written(w[decltype(g)::value][decltype(j)::value]); });
+        });
     }
 
     // acc[j][i][v] is row m0 + wave_m*WM + i*32 + lane%32, column n0 + wave_n*WN + j*32 + 8*(v/4) + 4*(lane/32) + v%4.
@@ -374,9 +453,9 @@ void launch(const bf16_t* a, const bf16_t* w, const float* bias, const float* re
                                      hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
     }
     const int k_per_block = k_blocks == 1 ? K : ceil_div(ceil_div(K, k_blocks), 64) * 64;
-    dim3 grid(ceil_div(N, BN), ceil_div(M, BM), k_blocks);
-    gemm_stream_kernel<OutT, BM, BN, WAVES_M, WAVES_N, WAVES_K, STAGES><<<grid, 64 * NW, LDS_BYTES, stream>>>(
-        a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block);
+    const XcdTiles places = place_tiles(ceil_div(M, BM), ceil_div(N, BN), BM, BN);
+    gemm_stream_kernel<OutT, BM, BN, WAVES_M, WAVES_N, WAVES_K, STAGES><<<8 * places.wide * places.high * k_blocks, 64 * NW, LDS_BYTES, stream>>>(
+        a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block, places);
 }
 
 // Whether the product takes this kernel: bfloat16 with a packed W, whole tiles of K, whole 16-byte pieces of output
@@ -389,26 +468,30 @@ inline bool takes(int M, int N, int K, bool packed, const CacheScatter& scatter,
     return true;
 }
 
+// The tile is chosen by what the busiest compute unit has to do: every block keeps a compute unit to itself (its
+// stages fill most of the LDS), so the blocks run in rounds of 256, and a round costs what a tile of K costs the block
+// (measured at GPT-2's three widths, 512 to 4,096 rows: 0.57 us at 128 x 192, 0.45 at 128 x 128, 0.70 at 256 x 128,
+// 0.30 at 128 x 64). Wide tiles win where they still fill a round; narrow outputs take 128 x 64, with two waves
+// sharing each 64 x 64 tile along K and a fourth stage where K is long.
 template <typename OutT>
 void dispatch(const bf16_t* a, const bf16_t* w, const float* bias, const float* residual, OutT* o, int M, int N, int K, int epilogue,
              hipStream_t stream, CacheScatter scatter, int k_blocks) {
-    static const int variant = getenv("MLLM_GEMM_VARIANT") ? atoi(getenv("MLLM_GEMM_VARIANT")) : 0;
 #define MLLM_STREAM(BM, BN, WM_, WN_, WK_, ST) launch<OutT, BM, BN, WM_, WN_, WK_, ST>(a, w, bias, residual, o, M, N, K, epilogue, stream, scatter, k_blocks)
-    switch (variant) {
-        case 1: MLLM_STREAM(128, 192, 2, 2, 1, 3); return;
-        case 2: MLLM_STREAM(128, 128, 2, 2, 1, 3); return;
-        case 3: MLLM_STREAM(128, 64, 2, 1, 2, 3); return;
-        case 4: MLLM_STREAM(256, 128, 4, 2, 1, 3); return;
-        case 5: MLLM_STREAM(128, 128, 2, 2, 1, 4); return;
-        case 6: MLLM_STREAM(128, 64, 2, 1, 2, 4); return;
-        case 7: MLLM_STREAM(128, 64, 2, 2, 1, 3); return;
-        case 8: MLLM_STREAM(128, 128, 4, 2, 1, 3); return;
-        case 9: MLLM_STREAM(128, 64, 2, 1, 2, 5); return;
-        case 10: if constexpr (sizeof(OutT) == 2) { MLLM_STREAM(128, 192, 2, 2, 2, 3); return; } break;
-        case 12: MLLM_STREAM(128, 128, 2, 2, 2, 3); return;
-        default: break;
+    struct Choice {
+        int bm, bn;
+        float tile_us;
+    };
+    static const Choice choices[4] = {{128, 192, 0.57f}, {256, 128, 0.70f}, {128, 128, 0.45f}, {128, 64, 0.30f}};
+    int best = 0;
+    float best_cost = 0.0f;
+    for (int c = 0; c < 4; c++) {
+        const long blocks = (long)ceil_div(M, choices[c].bm) * ceil_div(N, choices[c].bn) * k_blocks;
+        const float cost = (float)((blocks + 255) / 256) * choices[c].tile_us;
+        if (c == 0 || cost < best_cost) best = c, best_cost = cost;  // (equal costs: the wider tile, which reads less)
     }
-    if (ceil_div(M, 128) * ceil_div(N, 192) * k_blocks >= 160) MLLM_STREAM(128, 192, 2, 2, 1, 3);
+    if (best == 0) MLLM_STREAM(128, 192, 2, 2, 1, 3);
+    else if (best == 1) MLLM_STREAM(256, 128, 4, 2, 1, 3);
+    else if (best == 2) MLLM_STREAM(128, 128, 2, 2, 1, 3);
     else if (K / k_blocks >= 1536) MLLM_STREAM(128, 64, 2, 1, 2, 4);
     else MLLM_STREAM(128, 64, 2, 2, 1, 3);
 #undef MLLM_STREAM
