@@ -167,10 +167,9 @@ __device__ __forceinline__ float gelu_erf(float x) {
 // tanh form: 0.5 x (1 + tanh(u)) = x / (1 + e^(-2u)), with the hardware's exp2 and reciprocal
 // (one unit in the last place each).
 __device__ __forceinline__ float gelu_tanh_for_bf16(float x) {
-    const float coefficient = 0.7978845608f;
-    const float cubic = 0.044715f;
-    float argument = coefficient * (x + cubic * x * x * x);
-    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * argument));  // 2 log2(e)
+    // -2 log2(e) u = x (a + b x^2) with a = -2 log2(e) sqrt(2/pi), b = 0.044715 a: seven instructions
+    const float a = -2.3022081986f, b = -0.1029432396f;
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * __builtin_fmaf(x * x, b, a)));
 }
 
 // erf form: erf by the rational approximation 7.1.26 of Abramowitz and Stegun (absolute error

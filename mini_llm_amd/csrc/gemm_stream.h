@@ -361,22 +361,28 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
     unsigned char* slab = lds + SHARED_SUMS + wave * (32 * SLAB_ROW);
     unsigned char* slab_write = slab + (lane % 32) * SLAB_ROW + 4 * (lane / 32) * (int)sizeof(OutT);
     const unsigned char* slab_read = slab + min(lane_row, ROWS_A_STEP - 1) * SLAB_ROW + lane_piece * 16;  // (an idling lane reads inside the slab too)
-    auto leave = [&](auto kind, auto scattered) {
-        constexpr int KIND = decltype(kind)::value;
-        constexpr bool SCATTERED = decltype(scattered)::value;
+    // 'where' the wave's columns go: 0 rows of out [M, N]; a fused q/k/v projection: 1 all of them q columns (rows of out
+    // [M, q_width]), 2 all of them key columns or all of them value columns (into the cache pages), 3 some of each.
+    auto leave = [&](auto kind, auto where) {
+        constexpr int KIND = decltype(kind)::value, WHERE = decltype(where)::value;
+        constexpr bool SCATTERED = WHERE != 0;
         // where a lane's piece goes: q columns to out [M, q_width], key and value columns into the cache page at the
         // row's slot (a piece lies inside one head: the head size is a multiple of 8)
-        OutT* out_lane = out + (size_t)m_lane * (SCATTERED ? scatter.q_width : N) + n_lane;
+        const int row_stride = SCATTERED ? scatter.q_width : N;
+        OutT* out_lane = out + (size_t)m_lane * row_stride + n_lane;
+        // A piece in the cache lies at page * (bytes of a page) + ((head << page_shift) + offset) * (bytes of a row) + the
+        // piece's place in the row: all but page and offset is the lane's own constant.
         bool to_cache = false;
-        OutT* pages = nullptr;
-        int kv_head = 0;
-        if constexpr (SCATTERED) {
+        unsigned char* pages = nullptr;
+        unsigned row_bytes = 0, page_bytes = 0;
+        if constexpr (WHERE >= 2) {
             to_cache = n_lane >= scatter.q_width;
             int c = n_lane - scatter.q_width;
-            pages = (OutT*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
+            pages = (unsigned char*)(c < scatter.kv_width ? scatter.k_pages : scatter.v_pages);
             if (c >= scatter.kv_width) c -= scatter.kv_width;
-            kv_head = c / scatter.head_size;
-            pages += c % scatter.head_size;
+            row_bytes = scatter.head_size * (int)sizeof(OutT);
+            page_bytes = (scatter.n_kv_heads * row_bytes) << scatter.page_shift;
+            pages += (size_t)((c / scatter.head_size) << scatter.page_shift) * row_bytes + (c % scatter.head_size) * sizeof(OutT);
         }
 #pragma unroll
         for (int i = 0; i < OWN; i++) {
@@ -403,37 +409,38 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
                 const int row = i * 32 + r * ROWS_A_STEP;
                 Vec16 v = *reinterpret_cast<const Vec16*>(slab_read + r * ROWS_A_STEP * SLAB_ROW);
                 if (row >= rows_left) continue;
-                if constexpr (SCATTERED) {
-                    if (to_cache) {
+                if constexpr (WHERE >= 2) {
+                    if (WHERE == 2 || to_cache) {
                         const int slot = early_slot[i][r];
                         if (slot < 0) continue;
-                        const int page = slot >> scatter.page_shift, offset = slot & ((1 << scatter.page_shift) - 1);
-                        *reinterpret_cast<Vec16*>(pages + ((((size_t)page * scatter.n_kv_heads + kv_head) << scatter.page_shift) + offset) * scatter.head_size) = v;
-                    } else {
-                        *reinterpret_cast<Vec16*>(out_lane + (size_t)row * scatter.q_width) = v;
+                        const unsigned page = slot >> scatter.page_shift, offset = slot & ((1 << scatter.page_shift) - 1);
+                        *reinterpret_cast<Vec16*>(pages + (size_t)page * page_bytes + offset * row_bytes) = v;
+                        continue;
                     }
-                } else {
-                    if constexpr (WITH_RESIDUAL) {
-                        f32x4 sum = *reinterpret_cast<f32x4*>(&v);
-                        sum = early_residual[i][r] + sum;   // zeros where there is no residual
-                        v = *reinterpret_cast<Vec16*>(&sum);
-                    }
-                    *reinterpret_cast<Vec16*>(out_lane + (size_t)row * N) = v;
                 }
+                if constexpr (WITH_RESIDUAL && !SCATTERED) {
+                    f32x4 sum = *reinterpret_cast<f32x4*>(&v);
+                    sum = early_residual[i][r] + sum;   // zeros where there is no residual
+                    v = *reinterpret_cast<Vec16*>(&sum);
+                }
+                *reinterpret_cast<Vec16*>(out_lane + (size_t)row * row_stride) = v;
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
     };
     using std::integral_constant;
     if constexpr (CAN_SCATTER) {
-        if (scatter.enabled) {
-            leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<bool, true>{});  // (a q/k/v projection has no activation)
+        if (scatter.enabled) {  // (a q/k/v projection has no activation)
+            const int first = n_wave - scatter.q_width, last = min(n_wave + WN, N) - 1 - scatter.q_width;
+            if (last < 0) leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<int, 1>{});
+            else if (first >= 0 && first / scatter.kv_width == last / scatter.kv_width) leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<int, 2>{});
+            else leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<int, 3>{});
             return;
         }
     }
-    if (epilogue == MLLM_EPI_GELU_TANH) leave(integral_constant<int, MLLM_EPI_GELU_TANH>{}, integral_constant<bool, false>{});
-    else if (epilogue == MLLM_EPI_GELU_ERF) leave(integral_constant<int, MLLM_EPI_GELU_ERF>{}, integral_constant<bool, false>{});
-    else leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<bool, false>{});
+    if (epilogue == MLLM_EPI_GELU_TANH) leave(integral_constant<int, MLLM_EPI_GELU_TANH>{}, integral_constant<int, 0>{});
+    else if (epilogue == MLLM_EPI_GELU_ERF) leave(integral_constant<int, MLLM_EPI_GELU_ERF>{}, integral_constant<int, 0>{});
+    else leave(integral_constant<int, MLLM_EPI_NONE>{}, integral_constant<int, 0>{});
 }
 
 template <typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, int WAVES_K, int STAGES>
@@ -465,6 +472,7 @@ inline bool takes(int M, int N, int K, bool packed, const CacheScatter& scatter,
     if (!packed || K % 64 != 0 || K < 64 || N % 8 != 0 || M < 192 || ceil_div(M, 128) > 65535) return false;
     if ((long long)M * K * 2 >= (1LL << 32)) return false;
     if (scatter.enabled && (out_element != 2 || scatter.head_size % 8 != 0 || scatter.q_width % 8 != 0 || scatter.kv_width % 8 != 0)) return false;
+    if (scatter.enabled && (((long long)scatter.n_kv_heads * scatter.head_size * 2) << scatter.page_shift) >= (1LL << 31)) return false;  // a page's bytes in 32 bits
     return true;
 }
 

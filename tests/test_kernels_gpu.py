@@ -187,8 +187,10 @@ GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 1
                (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20),
                (2100, 2010, 104), (4100, 2010, 40),  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
                # K in whole tiles of 64, columns in whole pieces, 192 rows or more: in bfloat16 with a packed matrix the kernel that
-               # streams its operands into LDS (128 x 64 tiles with two and, from a K of 1,536, three stages; 128 x 128 from 256 tiles on)
-               (300, 136, 192), (193, 2008, 128), (2100, 264, 64), (700, 776, 320), (300, 72, 1600), (2100, 2008, 128), (192, 8, 64)]
+               # streams its operands into LDS: tiles of 128 x 64 (with two waves sharing each 64 x 64 along K from a K of 1,536 on:
+               # here with an odd count of tiles), 128 x 192, 128 x 128 and 256 x 128, chosen by the rounds of blocks they need
+               (300, 136, 192), (193, 2008, 128), (2100, 264, 64), (700, 776, 320), (300, 72, 1600), (2100, 2008, 128), (192, 8, 64),
+               (1000, 2312, 128), (2040, 4088, 64)]
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -273,7 +275,7 @@ def guarded(values, dtype, fill=float("nan")):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k", [(5, 37, 20), (1, 16, 8), (16, 130, 72), (40, 50, 200), (64, 100, 64), (70, 37, 24), (130, 200, 96),
                                    (300, 260, 136), (33, 40, 21), (200, 70, 50), (3, 9000, 64), (300, 264, 128), (200, 72, 64), (1000, 2056, 64),
-                                   (2050, 2056, 192)])
+                                   (2050, 2056, 192), (1000, 2312, 128), (2040, 4088, 64), (300, 72, 1600)])
 def test_linear_reads_nothing_past_its_operands(K, dtype, m, n, k):
     # NaN guards right after every operand: an out-of-bounds read would poison the result; a known
     # value right after the output: nothing is written past it. Every kernel of the product: few
@@ -642,7 +644,8 @@ def test_operands_are_checked_on_the_host(K):
     (2100, 14, 14, 48, 64, 72),  # enough rows and columns for the large tile
     # a width in whole tiles of 64: in bfloat16 with a packed matrix the kernel that streams its operands into LDS; heads of 40
     # and 24 (a 16-byte piece of columns stays inside a head), grouped heads, and heads of 20 (it does not: the other kernel)
-    (300, 5, 5, 48, 64, 128), (700, 6, 2, 40, 32, 192), (2100, 14, 14, 24, 16, 64), (250, 3, 3, 20, 64, 64)])
+    (300, 5, 5, 48, 64, 128), (700, 6, 2, 40, 32, 192), (2100, 14, 14, 24, 16, 64), (250, 3, 3, 20, 64, 64),
+    (2100, 12, 12, 64, 64, 128)])  # tiles of 128 x 192 whose waves hold q columns only, or key or value columns only
 @pytest.mark.parametrize("packed", [False, True])
 def test_fused_qkv_projection_writes_the_cache(K, dtype, rows, n_heads, n_kv_heads, head_size, page_size, width, packed):
     rng = np.random.default_rng(rows)
