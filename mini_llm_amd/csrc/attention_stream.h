@@ -26,8 +26,6 @@
 namespace prefill_stream {
 
 constexpr int KEYS = 32;      // keys per tile
-constexpr int QUERIES = 64;   // queries per block: two sub-tiles of 32, both held by every wave
-constexpr int QSUB = QUERIES / 32;
 constexpr int SPLITS = 4;     // waves per block; wave w takes tiles w, w + 4, ...
 
 template <int N>
@@ -36,6 +34,15 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// A 16-byte LDS read the compiler does not know to be one (see read_transposed): the value is there once
+// fragments_landed has passed, and nothing may read the register before.
+__device__ __forceinline__ void ask_fragment(i32x4& to, unsigned address) {
+    asm volatile("ds_read_b128 %0, %1" : "=v"(to) : "v"(address));
+}
+__device__ __forceinline__ void fragments_landed(i32x4& first) { asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(first)); }
+__device__ __forceinline__ void and_this_one(i32x4& fragment) { asm volatile("" : "+v"(fragment)); }
 
 __device__ __forceinline__ unsigned lds_address(const unsigned char* p) {
     return (unsigned)(size_t)(const __attribute__((address_space(3))) unsigned char*)p;
@@ -116,19 +123,23 @@ struct Layout {
     static constexpr int WAVE_BYTES = 4 * TILE_BYTES;   // two key tiles, two value tiles
     static constexpr int LDS_BYTES = SPLITS * WAVE_BYTES;
     static_assert(HD == 32 || HD == 64 || HD == 128, "rows of 64, 128 or 256 bytes");
-    static_assert(WAVE_BYTES == QUERIES * HD * 4, "a wave's partial result takes the place of its tiles");
+    static_assert(WAVE_BYTES >= 64 * HD * 4, "a wave's partial result (of up to 64 queries) takes the place of its tiles");
     // K: sixteen consecutive keys, the same piece: their 16-byte slots must differ modulo 256 bytes.
     static __device__ __forceinline__ int k_turn(int key) { return (key / (16 / PPR)) % PPR; }
     // V: four consecutive keys, the same 64 bytes of columns: their 64-byte slots must differ modulo 256 bytes.
     static __device__ __forceinline__ int v_turn(int key) { return HD == 32 ? 0 : (HD == 64 ? ((key >> 1) & 1) * 4 : (key & 3) * 4); }
 };
 
-template <int HD>
+// QUERIES: 64 queries a block (two sub-tiles of 32, both held by every wave), or 32 where that would leave compute units
+// without a block: what the kernel waits for is the wave with the most tiles, and a tile of 32 queries takes it half as long.
+template <int HD, int QUERIES>
 __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefill_stream_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, int out_stride, const int* __restrict__ q_starts, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads, int page_shift, int window, float scale) {
     typedef Layout<HD> L;
+    constexpr int QSUB = QUERIES / 32;
+    static_assert(QUERIES == 32 || QUERIES == 64, "one or two sub-tiles of queries");
     constexpr int QSTEPS = HD / 16;  // k-steps of the score product
     constexpr int DT = HD / 32;      // 32-row tiles of the output's head dimension
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
@@ -204,25 +215,10 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
     // V^T fragment by two transposing reads: the sixteen lanes of group g = l / 16 point at keys k0 + (l % 16) / 4, columns
     // 16 (g % 2) + 4 (l % 4) .. + 4 of a 32-column tile, and lane l gets keys k0 .. k0 + 3 of column 16 (g % 2) + l % 16
     const int v_key_in_read = (lane % 16) / 4, v_col = 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-    int next_page = 0;
-    if (n_mine > 0) {
-        const int page0 = table[tile_base(0) >> page_shift], page1 = table[tile_base(1) >> page_shift];
-        next_page = table[tile_base(2) >> page_shift];
-        issue(0, page0, false);
-        issue(0, page0, true);
-        issue(1, page1, false);
-        issue(1, page1, true);
-    }
-    for (int i = 0; i < n_mine; i++) {
-        const int page = next_page;                         // of tile i + 2, looked up a step ahead of its loads
-        next_page = table[tile_base(i + 3) >> page_shift];
-        const int k0 = first_base + (wave + SPLITS * i) * KEYS;
+    // The scores of a tile: S^T = K . Q^T, a key fragment serving both sub-tiles of queries. Returns with the fragments in
+    // registers (their place may be loaded into again) and the products still running.
+    auto scores = [&](int i, f32x16 (&s_acc)[QSUB]) {
         const unsigned char* k_tile = wave_lds + (i % 2) * L::TILE_BYTES;
-        const unsigned char* v_tile = k_tile + 2 * L::TILE_BYTES;
-        wait_vmcnt<3 * L::LOADS>();  // in flight: K(i) V(i) K(i+1) V(i+1); the first has landed
-
-        // ---- S^T = K . Q^T : a key fragment serves both sub-tiles of queries ----
-        f32x16 s_acc[QSUB];
 #pragma unroll
         for (int qs = 0; qs < QSUB; qs++)
 #pragma unroll
@@ -234,12 +230,42 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
             for (int qs = 0; qs < QSUB; qs++)
                 s_acc[qs] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag, *reinterpret_cast<const bf16x8*>(&q_reg[qs][s]), s_acc[qs], 0, 0, 0);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the fragments are in registers: their place may be loaded into
-        issue(i + 2, page, false);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    // A wave alone on its SIMD pays a tile's chain in full (key fragments, score products, softmax, value fragments,
+    // output products: 2,860 cycles a tile, of which the softmax arithmetic is 1,350), and the wave with the most tiles
+    // is what the kernel waits for. So the scores of tile i + 1 are issued before the softmax of tile i and run under it.
+    // Loads, in order: K0 V0 K1 V1 K2, then with tile i: K(i+3), V(i+2); a wait that leaves the newest n tiles' worth in
+    // flight has everything older. Pages are looked up a tile before their loads.
+    int page_v = 0, page_k = 0;  // of tiles i + 2 and i + 3
+    f32x16 s_even[QSUB], s_odd[QSUB];
+    if (n_mine > 0) {
+        const int page0 = table[tile_base(0) >> page_shift], page1 = table[tile_base(1) >> page_shift];
+        page_v = table[tile_base(2) >> page_shift];
+        page_k = table[tile_base(3) >> page_shift];
+        issue(0, page0, false);
+        issue(0, page0, true);
+        issue(1, page1, false);
+        issue(1, page1, true);
+        wait_vmcnt<3 * L::LOADS>();  // in flight: V0 K1 V1
+        scores(0, s_even);
+        issue(2, page_v, false);
+    }
+
+    auto tile = [&](int i, f32x16 (&s_acc)[QSUB], f32x16 (&s_next)[QSUB]) {
+        const int page_next = table[tile_base(i + 4) >> page_shift];
+        const int k0 = first_base + (wave + SPLITS * i) * KEYS;
+        const unsigned char* v_tile = wave_lds + 2 * L::TILE_BYTES + (i % 2) * L::TILE_BYTES;
+        const unsigned char* k_next = wave_lds + ((i + 1) % 2) * L::TILE_BYTES;
+        bf16x8 p[QSUB][2];  // the probabilities of a sub-tile of queries, as the second product's operand: keys 0-15 and 16-31 of the tile
+        wait_vmcnt<2 * L::LOADS>();  // K(i+1) has landed (and V(i)); beyond the wave's last tile: that tile again, its scores never used
+        // the key fragments of tile i + 1 are asked for now and travel under the first sub-tile's softmax
+        i32x4 k_frag[QSTEPS];
+#pragma unroll
+        for (int s = 0; s < QSTEPS; s++) ask_fragment(k_frag[s], lds_address(k_next + lane32 * L::ROW_BYTES + (((2 * s + half) ^ L::k_turn(lane32)) * 16)));
 
         // ---- mask (only where the tile touches the diagonal, a window or the portion's end), maximum, exponentials ----
-#pragma unroll
-        for (int qs = 0; qs < QSUB; qs++) {
+        auto softmax = [&](int qs) {
             const int sub_first_position = context + tile_q0 + qs * 32;
             const bool interior = window == 0 && tile_q0 + qs * 32 + 31 < q_len && k0 + KEYS - 1 <= sub_first_position;
             float tile_max = -INFINITY;
@@ -275,10 +301,35 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
                 s_acc[qs][v] = p;
                 running_sum[qs] += p;
             }
-        }
+#pragma unroll
+            for (int slab = 0; slab < 2; slab++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) p[qs][slab][e] = static_cast<bf16_t>(s_acc[qs][8 * slab + e]);
+        };
+        softmax(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // the scores of tile i + 1: issued here, they run under the second sub-tile's softmax and the reads of the values
+        fragments_landed(k_frag[0]);
+#pragma unroll
+        for (int s = 1; s < QSTEPS; s++) and_this_one(k_frag[s]);
+        issue(i + 3, page_k, false);  // (the fragments are in registers: their place may be loaded into)
+#pragma unroll
+        for (int s = 0; s < QSTEPS; s++)
+#pragma unroll
+            for (int qs = 0; qs < QSUB; qs++) {
+                f32x16 start = s_next[qs];
+                if (s == 0) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) start[v] = 0.0f;
+                }
+                s_next[qs] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&k_frag[s]), *reinterpret_cast<const bf16x8*>(&q_reg[qs][s]), start, 0, 0, 0);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int qs = 1; qs < QSUB; qs++) softmax(qs);
 
         // ---- O^T += V^T . P^T : two slabs of 16 keys; a lane's eight are keys 4 half .. + 4 and 8 + 4 half .. + 4 of the slab ----
-        wait_vmcnt<3 * L::LOADS>();  // in flight: V(i) K(i+1) V(i+1) K(i+2); the first has landed
+        wait_vmcnt<3 * L::LOADS>();  // the newest three are K(i+2) V(i+1) K(i+3): V(i) has landed
         short4_t v_frag[DT][4];      // per 32 columns: slab 0 low keys, slab 0 high keys, slab 1 low, slab 1 high
         {
             unsigned address[DT];
@@ -292,11 +343,6 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
         }
 #pragma unroll
         for (int slab = 0; slab < 2; slab++) {
-            bf16x8 p[QSUB];
-#pragma unroll
-            for (int qs = 0; qs < QSUB; qs++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) p[qs][e] = static_cast<bf16_t>(s_acc[qs][8 * slab + e]);
 #pragma unroll
             for (int i2 = 0; i2 < DT; i2++) {
                 bf16x8 fragment;
@@ -304,17 +350,23 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
                 halves[0] = v_frag[i2][2 * slab];
                 halves[1] = v_frag[i2][2 * slab + 1];
 #pragma unroll
-                for (int qs = 0; qs < QSUB; qs++) acc_o[qs][i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, p[qs], acc_o[qs][i2], 0, 0, 0);
+                for (int qs = 0; qs < QSUB; qs++) acc_o[qs][i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, p[qs][slab], acc_o[qs][i2], 0, 0, 0);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        issue(i + 2, page, true);
+        issue(i + 2, page_v, true);
+        page_v = page_k;
+        page_k = page_next;
+    };
+    for (int i = 0; i < n_mine; i += 2) {
+        tile(i, s_even, s_odd);
+        if (i + 1 < n_mine) tile(i + 1, s_odd, s_even);
     }
     // the loads asked for beyond the last tile land, and the last reads return, before the tiles' place is written over
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 
     // ---- the four waves' partial results, combined: each wave writes its own where its tiles lay, then finishes a share ----
-    float* partial = reinterpret_cast<float*>(lds) + wave * (QUERIES * HD);
+    float* partial = reinterpret_cast<float*>(lds + wave * L::WAVE_BYTES);
 #pragma unroll
     for (int qs = 0; qs < QSUB; qs++) {
         running_sum[qs] += __shfl_xor(running_sum[qs], 32, WAVE);
@@ -351,7 +403,7 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
                 float sum = 0.0f;
 #pragma unroll
                 for (int w = 0; w < SPLITS; w++)
-                    sum += weight[w] * reinterpret_cast<const float*>(lds)[w * (QUERIES * HD) + (share * 16 + 4 * g + e) * WAVE + lane];
+                    sum += weight[w] * reinterpret_cast<const float*>(lds + w * L::WAVE_BYTES)[(share * 16 + 4 * g + e) * WAVE + lane];
                 o[e] = static_cast<bf16_t>(sum * inverse);
             }
             *reinterpret_cast<bf16x4*>(out_row + 8 * g + 4 * half) = o;
@@ -369,19 +421,33 @@ inline bool takes(int head_size, int page_size, int max_q_len, float scale, int 
     return q_stride % 8 == 0 && out_stride % 4 == 0 && ((size_t)q) % 16 == 0 && ((size_t)out) % 8 == 0;
 }
 
+template <int HD, int QUERIES>
+void launch_queries(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
+                    const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
+                    int page_shift, int window, float scale, hipStream_t stream) {
+    constexpr int LDS_BYTES = Layout<HD>::LDS_BYTES;
+    static bool raised = false;  // per instantiation: the limit on dynamic LDS is a property of the kernel
+    if (!raised && LDS_BYTES > 60 * 1024)  // (if this fails the launch below fails too, and the entry point reports that)
+        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD, QUERIES>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
+    // x: (request, head), so that with a multiple of eight heads the blocks of one head share an XCD's L2; y: tiles of queries
+    dim3 grid(n_heads * n_requests, ceil_div(max_q_len, QUERIES));
+    attention_prefill_stream_kernel<HD, QUERIES><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, out_stride, q_starts, context_lens,
+        block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);
+}
+
 template <int HD>
 void launch(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
             const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
             int page_shift, int window, float scale, hipStream_t stream) {
-    constexpr int LDS_BYTES = Layout<HD>::LDS_BYTES;
-    static bool raised = false;  // per instantiation: the limit on dynamic LDS is a property of the kernel
-    if (!raised && LDS_BYTES > 60 * 1024)  // (if this fails the launch below fails too, and the entry point reports that)
-        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
-    // x: (request, head), so that with a multiple of eight heads the blocks of one head share an XCD's L2; y: tiles of queries
-    dim3 grid(n_heads * n_requests, ceil_div(max_q_len, QUERIES));
-    attention_prefill_stream_kernel<HD><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, out_stride, q_starts, context_lens,
-        block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);
+    // blocks of 64 queries where they give every compute unit a block (measured: 2 x 1,024 tokens x 12 heads 15.9 against 17.2 us),
+    // else of 32 (4 x 128 tokens on 896 cached: 9.7 against 13.0 us; 512 on 7,680: 46.7 against 66.0 us)
+    if ((long)n_heads * n_requests * ceil_div(max_q_len, 64) >= 256)
+        launch_queries<HD, 64>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, n_requests, max_q_len,
+                               n_heads, n_kv_heads, page_shift, window, scale, stream);
+    else
+        launch_queries<HD, 32>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, n_requests, max_q_len,
+                               n_heads, n_kv_heads, page_shift, window, scale, stream);
 }
 
 }  // namespace prefill_stream

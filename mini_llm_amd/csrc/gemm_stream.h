@@ -5,10 +5,11 @@
 //  * Operands go from memory to LDS directly (global_load_lds_dwordx4: a wave's load lands as 1 KiB
 //    of consecutive LDS in lane order) and cost no registers. Which bytes a lane asks for is therefore
 //    what lays the tile out in LDS. A chunk of the packed W is taken as it lies. For the row-major A,
-//    four lanes read the 64 bytes a row has in a chunk, so that a quarter wave touches 4 cache lines
-//    (a lane per row touched 16, and the lookups in the vector cache, not the bytes, bounded the
-//    kernel); a row's four pieces lie in LDS rotated by the row (piece ^ (row / 4) % 4), so that the
-//    sixteen lanes of a fragment read fall on sixteen different groups of banks.
+//    eight lanes read the 128 bytes a row has in a tile of K, one whole cache line (the vector cache
+//    works by lines, not bytes: a lane per row touched 64 lines with a load, four lanes per 64 bytes
+//    of a row touched every line twice: 18.3 -> 18.0 us at 2,048 x 768 x 3,072); a row's eight pieces lie in LDS rotated by the row
+//    (piece ^ (row / 2) % 8), so that the sixteen lanes of a fragment read fall on sixteen different
+//    groups of banks.
 //  * A block has a compute unit to itself and a wave a SIMD: whatever a wave waits for, its matrix
 //    core waits for too. So a wave owns 64 x 64 outputs or more (at 64 x 32 the fragment reads, not
 //    the products, set the pace); fragments are asked for two steps of K before their products; a
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, FM = WM / 32, FN = WN / 32;
     constexpr int BK = 64, KS = BK / 16 / WAVES_K;           // steps of 16 along K a wave takes of a tile
     constexpr int OWN = FM / WAVES_K;                        // slabs of 32 rows of its tile a wave finishes
-    constexpr int A_LOADS = BM / 16 * 2, W_LOADS = BN / 16 * 2, LOADS = A_LOADS + W_LOADS;  // loads of 1 KiB a tile of K
+    constexpr int A_LOADS = BM / 8, W_LOADS = BN / 16 * 2, LOADS = A_LOADS + W_LOADS;  // loads of 1 KiB a tile of K
     static_assert(WAVES_K == 1 || WAVES_K == 2, "a tile of K is taken whole or in halves");
     static_assert(FM >= 1 && FN >= 1 && FM % WAVES_K == 0, "the waves that share a tile finish equal parts of it");
     static_assert(A_LOADS % NW == 0 && W_LOADS % NW == 0, "every wave issues the same loads of A and of W");
@@ -156,10 +157,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
     for (int i = 0; i < LPW; i++) {
         const int q = wave + NW * i;
         if (i < A_LPW) {
-            const int rt = q / 2, kc = q % 2;
-            const int r16 = lane / 4, piece = (lane % 4) ^ ((r16 >> 2) & 3);
-            const int row = min(m0 + rt * 16 + r16, M - 1);  // beyond the last row: that row again, never stored
-            base[i] = reinterpret_cast<const unsigned char*>(A + k_begin + kc * 32);
+            // eight rows of 128 bytes: eight lanes take the eight pieces of a row (a whole cache line), turned by the row
+            const int in_tile = q * 8 + lane / 8, piece = (lane % 8) ^ ((in_tile >> 1) & 7);
+            const int row = min(m0 + in_tile, M - 1);  // beyond the last row: that row again, never stored
+            base[i] = reinterpret_cast<const unsigned char*>(A + k_begin);
             lane_offset[i] = ((unsigned)row * (unsigned)K + piece * 8) * 2;
         } else {
             const int qw = q - A_LOADS, rt = qw / 2, kc = qw % 2;
@@ -239,21 +240,25 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
             for (int v = 0; v < 16; v++) acc[j][i][v] = 0.0f;
     if (n_tiles > 0) {
 
-        // A 32 x 16 fragment: lane l holds row l % 32, k (l / 32) * 8 .. + 8. W: chunk [piece][row]; A: chunk [row][piece rotated].
+        // A 32 x 16 fragment: lane l holds row l % 32, k (l / 32) * 8 .. + 8. W: chunk [piece][row]; A: rows of 128 bytes, a
+        // row's eight pieces turned by the row (piece ^ (row / 2) % 8: the sixteen rows of a quarter wave's read then fall
+        // on sixteen different groups of banks).
         const int w_frag0 = BM * 128 + (wave_n * WN / 16) * 2048 + ((lane % 32) / 16) * 2048 + (lane / 32) * 256 + (lane % 16) * 16;
-        const int a_row0 = (wave_m * WM / 16) * 2048 + ((lane % 32) / 16) * 2048 + (lane % 16) * 64, a_turn = ((lane % 16) >> 2) & 3;
+        const int a_row0 = (wave_m * WM + lane % 32) * 128, a_turn = (lane >> 1) & 7;
         // Fragments are asked for two steps before their products (four sets of registers): a step's reads come from all
         // waves at once, and the LDS takes longer over them than one step's products last. A turn of the loop is four
         // steps: one tile, or two where two waves share the tile's steps. Step g of a turn: wait for set g; then its products,
         // and between them the reads of step g + 2 and the step's share of the loads of a tile further on.
         constexpr int SETS = 4, TILES_A_TURN = SETS / KS, FRAGMENTS = FM + FN, PRODUCTS = FM * FN;
         i32x4 a[SETS][FM], w[SETS][FN];
-        const unsigned a_lane[2] = {(unsigned)(a_row0 + wave_k * (KS / 2) * 1024 + (((0 + lane / 32) ^ a_turn) * 16)),
-                                    (unsigned)(a_row0 + wave_k * (KS / 2) * 1024 + (((2 + lane / 32) ^ a_turn) * 16))};
+        const int kk0 = wave_k * KS;
+        unsigned a_lane[KS];  // step s of the wave's steps of a tile: pieces 2 (kk0 + s) and 2 (kk0 + s) + 1 of the row
+#pragma unroll
+        for (int step = 0; step < KS; step++) a_lane[step] = a_row0 + (((2 * (kk0 + step) + lane / 32) ^ a_turn) * 16);
         const unsigned w_lane = w_frag0 + wave_k * (KS / 2) * 1024;
         auto ask = [&](auto set, auto step, auto fragment, unsigned stage_offset) {  // fragment 'fragment' of step 'step' of a tile
             constexpr int SET = decltype(set)::value, S = decltype(step)::value, F = decltype(fragment)::value;
-            if constexpr (F < FM) ask_fragment<F * 4096 + (S / 2) * 1024>(a[SET][F], a_lane[S % 2] + stage_offset);
+            if constexpr (F < FM) ask_fragment<F * 4096>(a[SET][F], a_lane[S] + stage_offset);
             else ask_fragment<(F - FM) * 4096 + (S / 2) * 1024 + (S % 2) * 512>(w[SET][F - FM], w_lane + stage_offset);
         };
         // The loads of tile u + STAGES go into the stage of tile u, between the barrier in tile u (which every wave passes
@@ -466,10 +471,11 @@ void launch(const bf16_t* a, const bf16_t* w, const float* bias, const float* re
 }
 
 // Whether the product takes this kernel: bfloat16 with a packed W, whole tiles of K, whole 16-byte pieces of output
-// columns, enough rows to fill tiles of 128, an A whose bytes a 32-bit offset reaches; a fused q/k/v projection only
+// columns, more rows than the kernel for few rows takes (from 65 rows on this one is the faster, half-empty tile or not),
+// an A whose bytes a 32-bit offset reaches; a fused q/k/v projection only
 // where a piece stays inside one head.
 inline bool takes(int M, int N, int K, bool packed, const CacheScatter& scatter, size_t out_element) {
-    if (!packed || K % 64 != 0 || K < 64 || N % 8 != 0 || M < 192 || ceil_div(M, 128) > 65535) return false;
+    if (!packed || K % 64 != 0 || K < 64 || N % 8 != 0 || M <= 64 || ceil_div(M, 128) > 65535) return false;
     if ((long long)M * K * 2 >= (1LL << 32)) return false;
     if (scatter.enabled && (out_element != 2 || scatter.head_size % 8 != 0 || scatter.q_width % 8 != 0 || scatter.kv_width % 8 != 0)) return false;
     if (scatter.enabled && (((long long)scatter.n_kv_heads * scatter.head_size * 2) << scatter.page_shift) >= (1LL << 31)) return false;  // a page's bytes in 32 bits

@@ -186,11 +186,11 @@ def test_pack_matrix(K, rows, cols, src, dst, transpose):
 GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 192, 200), (65, 130, 72),
                (130, 257, 136), (200, 777, 240), (257, 96, 1024), (5, 50, 36), (40, 33, 20),
                (2100, 2010, 104), (4100, 2010, 40),  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
-               # K in whole tiles of 64, columns in whole pieces, 192 rows or more: in bfloat16 with a packed matrix the kernel that
+               # K in whole tiles of 64, columns in whole pieces, 65 rows or more: in bfloat16 with a packed matrix the kernel that
                # streams its operands into LDS: tiles of 128 x 64 (with two waves sharing each 64 x 64 along K from a K of 1,536 on:
                # here with an odd count of tiles), 128 x 192, 128 x 128 and 256 x 128, chosen by the rounds of blocks they need
                (300, 136, 192), (193, 2008, 128), (2100, 264, 64), (700, 776, 320), (300, 72, 1600), (2100, 2008, 128), (192, 8, 64),
-               (1000, 2312, 128), (2040, 4088, 64)]
+               (1000, 2312, 128), (2040, 4088, 64), (70, 136, 128), (130, 264, 64)]
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -275,7 +275,7 @@ def guarded(values, dtype, fill=float("nan")):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m,n,k", [(5, 37, 20), (1, 16, 8), (16, 130, 72), (40, 50, 200), (64, 100, 64), (70, 37, 24), (130, 200, 96),
                                    (300, 260, 136), (33, 40, 21), (200, 70, 50), (3, 9000, 64), (300, 264, 128), (200, 72, 64), (1000, 2056, 64),
-                                   (2050, 2056, 192), (1000, 2312, 128), (2040, 4088, 64), (300, 72, 1600)])
+                                   (2050, 2056, 192), (1000, 2312, 128), (2040, 4088, 64), (300, 72, 1600), (70, 136, 128)])
 def test_linear_reads_nothing_past_its_operands(K, dtype, m, n, k):
     # NaN guards right after every operand: an out-of-bounds read would poison the result; a known
     # value right after the output: nothing is written past it. Every kernel of the product: few
@@ -406,14 +406,16 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     [(3, 3, 32, 16, 0), (2, 2, 64, 64, 0), (4, 2, 64, 16, 150), (2, 1, 128, 8, 0), (2, 2, 128, 256, 0), (3, 3, 32, 32, 70),
      (2, 2, 48, 32, 0), (5, 5, 64, 4, 0)],
 )
-def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head_size, page_size, window):
+@pytest.mark.parametrize("copies", [1, 12])
+def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head_size, page_size, window, copies):
     # portions of several query tiles over several key tiles, requests of different lengths in one call (one
     # with a single token, one that starts at position 0, one whose portion ends one past a tile), pages
     # scrambled and unwritten places holding NaN. In the longest request some queries look hard at one far
     # key each (the first key, keys at the two sides of tile and page edges), so that a tile that is
-    # skipped, read twice or read from a wrong page shows in those rows.
+    # skipped, read twice or read from a wrong page shows in those rows. Once as they are (few blocks: the
+    # bfloat16 kernel takes 32 queries a block) and once twelve times over (64 queries a block).
     rng = np.random.default_rng(head_size * 10 + page_size)
-    shapes = [(0, 300), (200, 129), (500, 1), (70, 65), (0, 2)]
+    shapes = [(0, 300), (200, 129), (500, 1), (70, 65), (0, 2)] * copies
     need = sum((c + n + page_size - 1) // page_size for c, n in shapes)
     num_pages = need + 5
     order = rng.permutation(num_pages).tolist()
