@@ -97,8 +97,12 @@ class DecodeBench:
         seconds, bytes_read, done = 0.0, 0.0, 0
         config, dtype = self.engine.config, self.engine.options.dtype
         while done < steps:
-            if self.length >= CONTEXT:
+            if self.length >= CONTEXT - 1:
+                # new sequences: one untimed step from the host's tokens leaves every sequence's newest token on the
+                # device, where the queued steps below take it from
                 self.start()
+                self.last = self.engine.decode_batch(self.handles, self.last)
+                self.length += 1
             n = min(steps - done, CONTEXT - self.length)
             torch.cuda.synchronize()
             begin = time.perf_counter()
