@@ -183,18 +183,35 @@ __global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefi
     // used), so that the count of loads in flight is the same in every step.
     unsigned char* const wave_lds = lds + wave * L::WAVE_BYTES;
     auto tile_base = [&](int i) { return first_base + (wave + SPLITS * min(i, n_mine - 1)) * KEYS; };
+    // a lane's place among the rows of a whole tile, in bytes: the same for every tile, so an address is a base all lanes
+    // share plus this (worked out anew for every load it was a sixth of the loop's vector instructions)
+    unsigned k_lane[L::LOADS], v_lane[L::LOADS];
+#pragma unroll
+    for (int l = 0; l < L::LOADS; l++) {
+        const int row = l * L::ROWS_PER_LOAD + lane / L::PPR, slot = lane % L::PPR;
+        k_lane[l] = (row * HD + (slot ^ L::k_turn(row)) * 8) * 2;
+        v_lane[l] = (row * HD + (slot ^ L::v_turn(row)) * 8) * 2;
+    }
     auto issue = [&](int i, int page, bool is_value) {  // page: the one that holds the whole tile
         const int k_base = tile_base(i);
-        const int last_row = min(KEYS - 1, block_last_position - k_base);
-        const bf16_t* base = (is_value ? v_pages : k_pages) + ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (k_base & page_mask)) * HD;
+        const int last_row = block_last_position - k_base;
+        const unsigned char* base = reinterpret_cast<const unsigned char*>(
+            (is_value ? v_pages : k_pages) + ((((size_t)page * n_kv_heads + kv_head) << page_shift) + (k_base & page_mask)) * HD);
         unsigned char* place = wave_lds + (is_value ? 2 * L::TILE_BYTES : 0) + (i % 2) * L::TILE_BYTES;
+        if (last_row >= KEYS - 1) {
 #pragma unroll
-        for (int l = 0; l < L::LOADS; l++) {
-            const int row = l * L::ROWS_PER_LOAD + lane / L::PPR, slot = lane % L::PPR;
-            const int piece = slot ^ (is_value ? L::v_turn(row) : L::k_turn(row));
-            const bf16_t* src = base + min(row, last_row) * HD + piece * 8;
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
-                                             (void __attribute__((address_space(3)))*)(place + l * 1024), 16, 0, 0);
+            for (int l = 0; l < L::LOADS; l++)
+                __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)(base + (is_value ? v_lane[l] : k_lane[l])),
+                                                 (void __attribute__((address_space(3)))*)(place + l * 1024), 16, 0, 0);
+        } else {  // the tile that holds the last key: the rows behind it are that key's row again
+#pragma unroll
+            for (int l = 0; l < L::LOADS; l++) {
+                const int row = l * L::ROWS_PER_LOAD + lane / L::PPR, slot = lane % L::PPR;
+                const int piece = slot ^ (is_value ? L::v_turn(row) : L::k_turn(row));
+                const unsigned char* src = base + (min(row, last_row) * HD + piece * 8) * 2;
+                __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                                 (void __attribute__((address_space(3)))*)(place + l * 1024), 16, 0, 0);
+            }
         }
     };
 
