@@ -70,8 +70,9 @@ template <int OFFSET>
 __device__ __forceinline__ void ask_fragment(i32x4& to, unsigned address) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(address), "n"(OFFSET));
 }
-// waits until at most IN_FLIGHT of the wave's LDS operations are under way (they complete in order; nothing else that
-// counts there is in flight inside the loop); the fragments named are only read after it
+// waits until at most IN_FLIGHT of the wave's LDS operations are under way (they complete in order; a scalar load,
+// which counts there too and completes out of order, must not be under way: the loop has none, which a test of the
+// compiled code checks); the fragments named are only read after it
 template <int IN_FLIGHT>
 __device__ __forceinline__ void fragments_landed(i32x4& first) {
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(first) : "n"(IN_FLIGHT));
