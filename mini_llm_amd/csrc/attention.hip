@@ -121,6 +121,7 @@ MLLM_API int mllm_cache_write(const void* k_src, const void* v_src, int src_stri
     if (n_rows == 0) return 0;
     int width = n_kv_heads * head_size;
     int threads = width >= 256 ? 256 : (width >= 128 ? 128 : 64);
+    mllm_count_kernel(MLLM_K_CACHE_WRITE);
     if (dtype == MLLM_F32)
         cache_write_kernel<float><<<n_rows, threads, 0, stream>>>(
             (const float*)k_src, (const float*)v_src, src_stride, (float*)k_pages, (float*)v_pages,
@@ -149,6 +150,7 @@ MLLM_API int mllm_attention(const void* q, int q_stride, const void* k_pages, co
                  "attention: rows are too short for the heads");
     if (n_tokens == 0) return 0;
     dim3 grid(n_tokens, ceil_div(n_heads, 4));
+    mllm_count_kernel(MLLM_K_ATTENTION_GENERAL);
     if (dtype == MLLM_F32)
         attention_general_kernel<float><<<grid, 256, 0, stream>>>(
             (const float*)q, q_stride, (const float*)k_pages, (const float*)v_pages, (float*)out,
@@ -296,6 +298,7 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
     const bool together = sizeof(T) == 2 || rounds <= 12;
 #define MLLM_DECODE_CASE(HD)                                                                                   \
     case HD:                                                                                                   \
+        mllm_count_kernel(MLLM_K_ATTENTION_DECODE);                                                            \
         if (together)                                                                                          \
             attention_decode_kernel<T, HD, true><<<grid, block, 0, stream>>>(                                  \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
@@ -701,6 +704,7 @@ void launch_prefill(const void* q, int q_stride, const void* k_pages, const void
 #define MLLM_PREFILL_LAUNCH(QG, KS)                                                                                   \
     {                                                                                                                  \
         dim3 grid(ceil_div(max_q_len, 32 * QG), n_heads, n_requests);                                                  \
+        mllm_count_kernel(MLLM_K_ATTENTION_PREFILL);                                                                   \
         attention_prefill_kernel<T, HD_PAD, QG, KS><<<grid, 64 * QG * KS, 0, stream>>>(                                \
             (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens, \
             block_tables, max_blocks, n_heads, n_kv_heads, head_size, page_shift, window, scale);                      \

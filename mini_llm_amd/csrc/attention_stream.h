@@ -448,6 +448,7 @@ void launch_queries(const void* q, int q_stride, const void* k_pages, const void
         raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD, QUERIES>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
     // x: (request, head), so that with a multiple of eight heads the blocks of one head share an XCD's L2; y: tiles of queries
     dim3 grid(n_heads * n_requests, ceil_div(max_q_len, QUERIES));
+    mllm_count_kernel(MLLM_K_ATTENTION_PREFILL_STREAM);
     attention_prefill_stream_kernel<HD, QUERIES><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, out_stride, q_starts, context_lens,
         block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);

@@ -59,6 +59,17 @@ __host__ __device__ __forceinline__ size_t packed_element(int row, int col, int 
 void mllm_set_error(const char* format, ...);
 int mllm_check_launch(const char* what);
 
+// Every kernel launch is counted by kind, on the host (what the reference's launch counter is for,
+// engine/include/cuda_check.h:21-41: a test can tell which kernels a step took and how many).
+// Launches recorded into a graph count when they are captured, not when the graph is replayed.
+enum MllmKernel : int {
+    MLLM_K_EMBED = 0, MLLM_K_LAYERNORM, MLLM_K_ADD, MLLM_K_CACHE_WRITE, MLLM_K_ATTENTION_GENERAL, MLLM_K_ATTENTION_DECODE,
+    MLLM_K_ATTENTION_PREFILL, MLLM_K_ATTENTION_PREFILL_STREAM, MLLM_K_PACK, MLLM_K_CONVERT, MLLM_K_DECODE_ATTENTION_HALF,
+    MLLM_K_DECODE_MLP_HALF, MLLM_K_PENDING_SUM, MLLM_K_PENDING_LAYERNORM, MLLM_K_GEMM_SKINNY, MLLM_K_GEMM_TILED, MLLM_K_GEMM_STREAM,
+    MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_KINDS
+};
+void mllm_count_kernel(MllmKernel kind);
+
 #define MLLM_REQUIRE(condition, ...)      \
     do {                                  \
         if (!(condition)) {               \

@@ -55,12 +55,14 @@ __global__ __launch_bounds__(256) void pack_kernel(const S* __restrict__ src, D*
 template <typename S, typename D>
 void launch_pack(const void* src, void* dst, int rows, int cols, int transpose, hipStream_t stream) {
     const size_t chunks = (size_t)ceil_div(rows, 16) * ceil_div(cols, 4 * (16 / (int)sizeof(D)));
+    mllm_count_kernel(MLLM_K_PACK);
     pack_kernel<S, D><<<(unsigned)((chunks + 3) / 4), 256, 0, stream>>>((const S*)src, (D*)dst, rows, cols, transpose);
 }
 
 template <typename S, typename D>
 void launch_convert(const void* src, void* dst, int rows, int cols, int transpose, hipStream_t stream) {
     dim3 grid(ceil_div(cols, 32), ceil_div(rows, 32)), block(32, 8);
+    mllm_count_kernel(MLLM_K_CONVERT);
     convert_kernel<S, D><<<grid, block, 0, stream>>>((const S*)src, (D*)dst, rows, cols, transpose);
 }
 

@@ -844,6 +844,7 @@ int launch_mlp_half(PendingSum in, float* summed, const float* gamma, const floa
     // matrices are read fewer times.
     const int tokens_per_block = stage_pieces == 0 ? DL_TOKENS : (n_tokens <= 4 ? 1 : (n_tokens <= 8 ? 2 : (n_tokens <= 16 ? 4 : (n_tokens <= 64 ? 8 : DL_TOKENS))));
     dim3 grid((inner + U - 1) / U, (n_tokens + tokens_per_block - 1) / tokens_per_block);
+    mllm_count_kernel(MLLM_K_DECODE_MLP_HALF);
     decode_mlp_half_kernel<NV, U><<<grid, DL_THREADS, lds, stream>>>(in, summed, gamma, beta, eps, w_up, b_up, w_down, partial_out,
                                                                       n_tokens, width, inner, epilogue, stage_pieces, tokens_per_block);
     return 0;
@@ -890,6 +891,7 @@ MLLM_API int mllm_decode_attention_half(
     dim3 grid(n_heads, n_tokens);
 #define MLLM_HALF_CASE(HD)                                                                                              \
     case HD:                                                                                                            \
+        mllm_count_kernel(MLLM_K_DECODE_ATTENTION_HALF);                                                                \
         decode_attention_half_kernel<HD><<<grid, DL_THREADS, 0, stream>>>(                                              \
             in, summed, gamma, beta, eps, (const bf16_t*)w_qkv, b_qkv, (const bf16_t*)w_out, (bf16_t*)k_pages,          \
             (bf16_t*)v_pages, slots, token_request, positions, block_tables, max_blocks, partial_out, n_tokens, width,  \
@@ -945,6 +947,7 @@ MLLM_API int mllm_pending_sum(const float* base, const float* partials, const fl
     if (n_rows == 0) return 0;
     PendingSum in{base, partials, pending_bias, n_partials, n_rows};
     dim3 grid((width / 4 + 255) / 256, n_rows);
+    mllm_count_kernel(MLLM_K_PENDING_SUM);
     pending_sum_kernel<<<grid, 256, 0, stream>>>(in, out, width);
     return mllm_check_launch("pending_sum");
 }
@@ -963,6 +966,7 @@ MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, co
     if (n_rows == 0) return 0;
     PendingSum in{base, partials, pending_bias, n_partials, pending_rows};
     const size_t lds = (size_t)width * 4;
+    mllm_count_kernel(MLLM_K_PENDING_LAYERNORM);
     if (out_dtype == MLLM_F32)
         pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, summed, width, eps, packed_out);
     else if (out_dtype == MLLM_BF16)

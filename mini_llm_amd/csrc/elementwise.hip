@@ -43,6 +43,7 @@ MLLM_API int mllm_embed(int* tokens, const int* positions, const int* sources, c
     MLLM_REQUIRE(sources == nullptr || token_slots != nullptr, "embed: sources without token slots");
     if (n_rows == 0) return 0;
     int threads = width >= 256 ? 256 : 64;
+    mllm_count_kernel(MLLM_K_EMBED);
     if (table_dtype == MLLM_F32)
         embed_kernel<float><<<n_rows, threads, 0, stream>>>(tokens, positions, sources, token_slots, (const float*)wte,
                                                             (const float*)wpe, out, width);
@@ -195,6 +196,7 @@ static void launch_layernorm(const float* x, const int* row_index, const float* 
     const int waves = 4;
     dim3 grid(ceil_div(n_rows, waves)), block(waves * WAVE);
     OutT* o = (OutT*)out;
+    mllm_count_kernel(MLLM_K_LAYERNORM);
     const bool aligned = (((size_t)x | (size_t)gamma | (size_t)beta | (size_t)out) & 15) == 0;  // 16-byte pieces need it
     if (aligned && width % 4 == 0 && width <= 16 * 4 * WAVE) {
         if (width <= 1 * 4 * WAVE)
@@ -252,6 +254,7 @@ MLLM_API int mllm_add(const float* a, const void* b, float* out, long long n, in
     MLLM_REQUIRE(n >= 0, "add: negative size");
     if (n == 0) return 0;
     unsigned blocks = (unsigned)((n + 255) / 256);
+    mllm_count_kernel(MLLM_K_ADD);
     if (b_dtype == MLLM_F32)
         add_kernel<float><<<blocks, 256, 0, stream>>>(a, (const float*)b, out, (size_t)n);
     else if (b_dtype == MLLM_BF16)

@@ -468,6 +468,7 @@ void launch_skinny(const T* a, const T* w, bool packed, const float* bias, const
     int split = 1;  // waves per block, along K: enough waves to fill the chip, each with work to do
     while (split < 16 && tiles * k_blocks * split < 2048 && steps_per_block >= 8 * split) split *= 2;
     dim3 grid(tiles, k_blocks);
+    mllm_count_kernel(MLLM_K_GEMM_SKINNY);
 #define MLLM_SKINNY_CASE(SPLIT)                                                                                                   \
     if (packed) gemm_skinny_kernel<T, OutT, MT, SPLIT, true><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block, x_packed, out_packed); \
     else gemm_skinny_kernel<T, OutT, MT, SPLIT, false><<<grid, 64 * SPLIT, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, steps_per_block, x_packed, out_packed);
@@ -514,6 +515,7 @@ void launch_tile(const T* a, const T* w, bool packed, const float* bias, const f
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM), k_blocks);
     constexpr int PAIR = 2 * Tile<T>::BK;  // the kernel's loop takes two LDS tiles a turn
     int k_per_block = k_blocks == 1 ? ceil_div(K, PAIR) * PAIR : ceil_div(ceil_div(K, k_blocks), PAIR) * PAIR;
+    mllm_count_kernel(MLLM_K_GEMM_TILED);
     if (packed) gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block);
     else gemm_kernel<T, OutT, BM, BN, WAVES_M, WAVES_N, ALIGNED, false><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block);
 }
@@ -597,6 +599,7 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
     MLLM_REQUIRE((!x_packed && !out_packed) || mllm_gemm_takes_packed_rows(M, N, K, in_dtype),
                  "gemm: rows in the packed layout are for the kernel for few rows, which M=%d N=%d K=%d do not take", M, N, K);
     MLLM_REQUIRE(!out_packed || residual == nullptr, "gemm: a residual sum is not written in the packed layout");
+    MLLM_REQUIRE(residual == nullptr || out_dtype == MLLM_F32, "gemm: a residual sum is 32-bit, the output asked for is not");
     if (M == 0) return 0;
     if (in_dtype == MLLM_F32 && out_dtype == MLLM_F32)
         launch_gemm<float, float>(A, W, w_packed != 0, bias, residual, out, M, N, K, epilogue, x_packed, out_packed, stream);
@@ -735,6 +738,7 @@ MLLM_API int mllm_linear_split_static(const void* A, const void* W, int w_packed
     if (static_scratch(&partials)) return 1;
     if (mllm_gemm_split(A, W, w_packed, partials, M, N, K, in_dtype, k_blocks, 0, stream)) return 1;
     dim3 grid(ceil_div(N, 256), M);
+    mllm_count_kernel(MLLM_K_STATIC_SUM);
     static_sum_kernel<<<grid, 256, 0, stream>>>(partials, bias, residual, out, M, N, k_blocks);
     return mllm_check_launch("linear_split_static");
 }

@@ -467,6 +467,7 @@ void launch(const bf16_t* a, const bf16_t* w, const float* bias, const float* re
     }
     const int k_per_block = k_blocks == 1 ? K : ceil_div(ceil_div(K, k_blocks), 64) * 64;
     const XcdTiles places = place_tiles(ceil_div(M, BM), ceil_div(N, BN), BM, BN);
+    mllm_count_kernel(MLLM_K_GEMM_STREAM);
     gemm_stream_kernel<OutT, BM, BN, WAVES_M, WAVES_N, WAVES_K, STAGES><<<8 * places.wide * places.high * k_blocks, 64 * NW, LDS_BYTES, stream>>>(
         a, w, bias, residual, o, M, N, K, epilogue, scatter, k_per_block, places);
 }

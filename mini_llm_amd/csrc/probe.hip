@@ -50,6 +50,7 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ out
 // Reads n_bytes (a multiple of 16) once with `blocks` blocks of 256 threads; out needs one float.
 MLLM_API int mllm_probe_read(const void* buffer, long long n_bytes, float* out, int blocks, hipStream_t stream) {
     MLLM_REQUIRE(n_bytes >= 0 && n_bytes % 16 == 0 && blocks > 0, "probe_read: bad size");
+    mllm_count_kernel(MLLM_K_PROBE);
     probe_read_kernel<<<blocks, 256, 0, stream>>>((const f32x4*)buffer, out, (size_t)n_bytes / 16);
     return mllm_check_launch("probe_read");
 }
@@ -58,6 +59,7 @@ MLLM_API int mllm_probe_read(const void* buffer, long long n_bytes, float* out, 
 // is blocks * 4 * iterations * 4 * (32768 flops for bfloat16, 4096 for float32).
 MLLM_API int mllm_probe_mfma(float* out, int blocks, int iterations, int dtype, hipStream_t stream) {
     MLLM_REQUIRE(blocks > 0 && iterations > 0, "probe_mfma: bad size");
+    mllm_count_kernel(MLLM_K_PROBE);
     if (dtype == MLLM_BF16) probe_mfma_kernel<true><<<blocks, 256, 0, stream>>>(out, iterations);
     else if (dtype == MLLM_F32) probe_mfma_kernel<false><<<blocks, 256, 0, stream>>>(out, iterations);
     else MLLM_REQUIRE(false, "probe_mfma: unknown dtype %d", dtype);

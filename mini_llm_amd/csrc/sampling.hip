@@ -182,6 +182,7 @@ MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float
                          int* out_tokens, int* token_slots, const int* slot_of_row, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", n_rows, vocab);
     if (n_rows == 0) return 0;
+    mllm_count_kernel(MLLM_K_SAMPLE);
     sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, vocab, temperatures, top_ps,
                                                          (const uint64_t*)seeds, steps, out_tokens, token_slots, slot_of_row);
     return mllm_check_launch("sample");

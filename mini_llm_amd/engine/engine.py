@@ -30,7 +30,7 @@ class EngineOptions:
     max_tokens: int | None = None        # cache capacity in tokens; None: max_sessions full contexts
     cache_gib: float | None = None       # or the capacity as memory: GiB of page pools (an MI355X has 288 GB to give)
     page_size: int = DEFAULT_PAGE_SIZE
-    max_length: int | None = None        # longest sequence, for a model without a position limit of its own
+    max_length: int | None = None        # longest sequence a request may reach: needed for a model without a position limit of its own, and narrows a model's own
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
     use_graphs: bool = True              # replay decode steps from captured HIP graphs
     portion_graph_after: int | None = None   # a shape of batch with prompt portions is captured when it comes this often (None: the step function's default; 0: never)
@@ -47,8 +47,8 @@ class _Executor:
         self._hosts, self._turn = [], 0
 
     def max_positions(self):
-        """The model's own limit, else the longest sequence the cache was made for."""
-        return self._engine.model.max_positions() or self._engine.cache.max_length
+        """The longest sequence a request may reach: the model's own limit or the one the cache was made for."""
+        return self._engine.runner.longest_sequence()
 
     def check_prompt(self, tokens):
         limit, vocab = self.max_positions(), self._engine.model.vocab_size
@@ -170,8 +170,12 @@ class Engine:
         library()  # fails loudly here if the kernels are missing
         self.options = options
         self.model = model if model is not None else load_model(model_dir, options.dtype, options.device)
-        # the longest sequence a request may reach: the model's own limit, else the caller's
-        limit = self.model.max_positions() or options.max_length
+        # the longest sequence a request may reach: the model's own limit, narrowed by the caller's if one is given
+        if options.max_length is not None and options.max_length < 1:
+            raise ValueError(f"max_length must be at least 1, not {options.max_length}")
+        limit = self.model.max_positions()
+        if options.max_length is not None:
+            limit = options.max_length if limit is None else min(limit, options.max_length)
         if options.max_tokens is not None and options.cache_gib is not None:
             raise ValueError("give the cache's capacity as max_tokens or as cache_gib, not both")
         if options.cache_gib is not None:
@@ -180,12 +184,15 @@ class Engine:
         elif options.max_tokens is not None:
             max_tokens = options.max_tokens
         elif limit is not None:
-            max_tokens = options.max_sessions * limit
+            # max_sessions whole sequences: each takes whole pages
+            max_tokens = options.max_sessions * (-(-limit // options.page_size) * options.page_size)
         else:
-            raise ValueError("this model has no position limit of its own: size the cache with max_tokens or cache_gib, "
-                             "or give max_length")
+            raise ValueError("this model has no position limit of its own: give max_length (the cache then holds max_sessions "
+                             "sequences of that length), or size the cache with max_tokens or cache_gib as well")
         if limit is None:
-            limit = max_tokens   # one request may fill the whole cache, never more
+            # Block tables and the buffers of captured steps are as wide as the longest sequence: it has to be named,
+            # not taken from the size of the pool (which may be millions of tokens).
+            raise ValueError("this model has no position limit of its own: give max_length, the longest sequence a request may reach")
         self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
                                 max_requests=options.max_sessions, device=options.device, max_length=limit)
         self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs, portion_graph_after=options.portion_graph_after)
@@ -311,7 +318,7 @@ class Engine:
         """Continues every prompt (a list of token ids) through the scheduler; returns the new
         tokens of each. A prompt too long for the model is cut from the left so that the new
         tokens fit, as the reference's script does (scripts/complete.py:92-110)."""
-        limit = self.model.max_positions()
+        limit = self.runner.longest_sequence()
         outputs: list[list[int]] = [[] for _ in prompts]
         errors: list[str | None] = [None] * len(prompts)
         for i, prompt in enumerate(prompts):

@@ -40,6 +40,7 @@ from __future__ import annotations
 
 import collections
 import logging
+import threading
 from typing import Protocol
 
 from ..sampling import SamplingParams
@@ -177,13 +178,18 @@ class Scheduler:
         self._ids = self._admissions = 0
         self._tally = _Tally()
         self._closed_with: str | None = None
+        self._gate = threading.Lock()   # submit against shutdown; nothing else is shared between threads
 
     # --- the caller's side -----------------------------------------------------------------------
     def submit(self, request: Request) -> None:
-        if self._closed_with is not None:
-            request.on_error(self._closed_with)
-            return
-        self._queue.append(request)
+        """May be called from another thread than the one that steps. A request either reaches the queue before
+        ``shutdown`` drains it, or hears the shutdown's message: never neither."""
+        with self._gate:
+            closed = self._closed_with
+            if closed is None:
+                self._queue.append(request)
+        if closed is not None:
+            request.on_error(closed)
 
     def has_work(self) -> bool:
         return bool(self._live or self._queue or self._in_flight is not None)
@@ -195,10 +201,12 @@ class Scheduler:
     def shutdown(self, message: str = "the engine is shutting down") -> None:
         """Every live and waiting request hears ``message`` as its error and gives its pages back; a
         step in flight is forgotten; what is submitted afterwards fails at once."""
-        self._closed_with = message
+        with self._gate:   # whoever submits now has either appended already or will see the message
+            self._closed_with = message
+            waiting = list(self._queue)
+            self._queue.clear()
         self._abandon_live(message)
-        while self._queue:
-            item = self._queue.popleft()
+        for item in waiting:
             (item.request if isinstance(item, _Live) else item).on_error(message)
 
     def stats(self) -> dict:

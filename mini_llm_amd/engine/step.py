@@ -138,6 +138,8 @@ class ModelRunner:
         self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
         self.portion_graph_after = PORTION_GRAPH_AFTER if portion_graph_after is None else int(portion_graph_after)
         self.portion_graph_steps = 0
+        self.portion_graphs_made = 0      # captures of steps with prompt portions, and those given up for a newer shape
+        self.portion_graphs_dropped = 0
 
     def drop_graphs(self) -> None:
         """Gives the captured steps back now (they and the runner refer to each other, so otherwise they would lie around
@@ -171,11 +173,16 @@ class ModelRunner:
             if not 0 <= int(token) < vocab:
                 raise StepError(f"request {entry.request_id!r}: token {token} is outside the vocabulary [0, {vocab})")
 
+    def longest_sequence(self) -> int | None:
+        """The longest sequence a request may reach: the model's position limit or the cache's, whichever is less."""
+        limits = [n for n in (self.model.max_positions(), self.cache.max_length) if n is not None]
+        return min(limits) if limits else None
+
     def validate(self, entries) -> None:
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
-        vocab, limit = self.model.vocab_size, self.model.max_positions()
+        vocab, limit = self.model.vocab_size, self.longest_sequence()
         for entry in entries:
             if entry.request_id in seen:
                 raise StepError(f"request {entry.request_id!r} appears twice in one step")
@@ -193,7 +200,7 @@ class ModelRunner:
                 self._check_tokens(entry, vocab)
             length = self.cache.length(entry.request_id)
             if limit is not None and length + n > limit:
-                raise StepError(f"request {entry.request_id!r}: {length} + {n} tokens exceed the model's {limit} positions")
+                raise StepError(f"request {entry.request_id!r}: {length} + {n} tokens exceed the {limit} positions a sequence may have")
             for w in entry.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
@@ -237,8 +244,13 @@ class ModelRunner:
         if self._shapes_seen[shape] < self.portion_graph_after:
             return None
         while len(self._portion_graphs) >= PORTION_GRAPHS_KEPT:
-            self._portion_graphs.popitem(last=False)
+            # A shape that loses its graph starts counting again: with more hot shapes than graphs are kept, each would
+            # otherwise be captured anew every time its turn comes (a capture costs some forty steps' time).
+            evicted, _ = self._portion_graphs.popitem(last=False)
+            self._shapes_seen[evicted] = 0
+            self.portion_graphs_dropped += 1
         graph = self._portion_graphs[shape] = _PortionGraph(self)
+        self.portion_graphs_made += 1
         return graph
 
     def step(self, entries: list[StepEntry], observer=None):

@@ -484,15 +484,25 @@ _layer_kernel_rows: dict = {}
 
 def layer_kernel_rows(width: int) -> int:
     """Rows up to which the layer kernels for decoding beat the separate kernels at this width: the
-    library's own answer (mllm_decode_layer_rows, where the measurements behind it are written
-    down), or MINI_LLM_LAYER_KERNEL_ROWS from the environment, for measuring the crossover again."""
+    library's own answer (mllm_decode_layer_rows, where the measurements behind it are written down)."""
     if width not in _layer_kernel_rows:
-        import os
-
-        forced = os.environ.get("MINI_LLM_LAYER_KERNEL_ROWS")
-        rows = int(forced) if forced is not None else int(library().mllm_decode_layer_rows(int(width)))
+        rows = int(library().mllm_decode_layer_rows(int(width)))
         _layer_kernel_rows[width] = max(0, min(rows, LAYER_KERNEL_MAX_ROWS))
     return _layer_kernel_rows[width]
+
+
+def launch_counts() -> dict:
+    """kind of kernel -> how often this process has launched it so far (a launch recorded into a graph counts once, at its
+    capture; replays do not count). The difference of two calls tells which kernels the work between them took, as the
+    reference's launch counter does for its tests (engine/include/cuda_check.h:21-41)."""
+    lib = library()
+    return {lib.mllm_kernel_name(kind).decode(): int(lib.mllm_launch_count(kind)) for kind in range(lib.mllm_kernel_kinds())}
+
+
+def launches_since(before: dict) -> dict:
+    """The launches since ``before`` (an earlier ``launch_counts()``), kinds that were not launched left out."""
+    now = launch_counts()
+    return {name: now[name] - before.get(name, 0) for name in now if now[name] != before.get(name, 0)}
 
 
 def _pending(hidden):

@@ -75,6 +75,9 @@ def library() -> ctypes.CDLL:
         lib.mllm_static_scratch_bytes.argtypes = []
         lib.mllm_last_error.restype = ctypes.c_char_p
         lib.mllm_last_error.argtypes = []
+        lib.mllm_kernel_kinds.restype, lib.mllm_kernel_kinds.argtypes = c_int, []
+        lib.mllm_kernel_name.restype, lib.mllm_kernel_name.argtypes = ctypes.c_char_p, [c_int]
+        lib.mllm_launch_count.restype, lib.mllm_launch_count.argtypes = ctypes.c_ulonglong, [c_int]
         lib.path = path
         _library = lib
     return _library

@@ -73,3 +73,37 @@ def test_short_portions_are_laid_out_first_and_logit_rows_keep_the_given_order()
     for i, name in enumerate("acebd"):
         pages = cache.block_table(name, 0)
         assert batch.groups[0].block_tables[i, : len(pages)].tolist() == list(pages)
+
+
+def test_hot_shapes_beyond_the_kept_graphs_are_not_captured_at_every_turn():
+    # more shapes of batch than graphs are kept, taking turns: a shape that loses its graph starts counting again, so
+    # the number of captures stays far below the number of steps (a capture costs some forty steps' time)
+    from mini_llm_amd.engine import step as step_module
+    from mini_llm_amd.engine.step import ModelRunner
+
+    class NoModel:
+        vocab_size = 100
+
+        def short_portion(self):
+            return 8
+
+        def all_graph_safe(self):
+            return True
+
+    groups = [CacheGroupSpec("full", (0,), 2, 16, None)]
+    cache = CacheManager(groups, {}, num_pages=8, page_size=16, max_requests=4, max_length=64)
+    runner = ModelRunner(NoModel(), cache, None, portion_graph_after=2)
+    shapes = [[StepEntry("r", [0] * n, [n - 1])] for n in range(10, 10 + step_module.PORTION_GRAPHS_KEPT + 1)]   # nine shapes
+    rounds = 40
+    for _ in range(rounds):
+        for entries in shapes:
+            runner._portion_graph_for(entries)
+    steps = rounds * len(shapes)
+    assert runner.portion_graphs_made <= steps // 4, (runner.portion_graphs_made, steps)
+    assert len(runner._portion_graphs) <= step_module.PORTION_GRAPHS_KEPT
+    # eight shapes fit: each is captured once and kept
+    runner = ModelRunner(NoModel(), cache, None, portion_graph_after=2)
+    for _ in range(rounds):
+        for entries in shapes[:-1]:
+            runner._portion_graph_for(entries)
+    assert runner.portion_graphs_made == step_module.PORTION_GRAPHS_KEPT and runner.portion_graphs_dropped == 0

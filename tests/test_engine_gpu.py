@@ -345,6 +345,71 @@ def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
         run([("a", 30, [3]), ("f", 1, [0])])                      # X replayed
         assert checked == 2 * 5 + 3 * 4 + 2 + 1
         assert engine.runner.portion_graph_steps == (7 if use_graphs else 0)
+        # shape Z: a portion of 131 tokens (the products and the prompt attention for many rows) beside a single decoded
+        # token and a portion of two; replayed at two depths of the cache, the second one starting inside a page and
+        # inside a tile of 32 keys
+        for name in "abc":
+            engine.release_cache(handles[name])
+            handles[name] = engine.try_take_cache()
+            fed[name] = 0
+        run([("a", 40, []), ("b", 50, [49]), ("c", 3, [])])       # some history first
+        run([("a", 131, [130]), ("b", 1, [0]), ("c", 2, [1])])    # Z: eager
+        for name in "ab":
+            engine.release_cache(handles[name])
+            handles[name] = engine.try_take_cache()
+            fed[name] = 0
+        run([("b", 131, [130]), ("c", 1, [0]), ("a", 2, [0])])    # Z again: captured here, the long portion from an empty cache
+        run([("a", 43, [42]), ("c", 5, [])])                      # depths 45 (a), 11 (c)
+        run([("a", 131, [7]), ("b", 1, [0]), ("c", 2, [1])])      # Z replayed: the long portion starts at 45, inside a page and a tile
+        assert engine.runner.portion_graph_steps == (9 if use_graphs else 0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_takes_the_kernels_it_is_meant_to(tmp_path, dtype):
+    # Logits stay right whichever kernels compute them; which ones a step took shows only in the library's launch
+    # counts (the reference pins its launches per step the same way: engine/tests/test_gpt2_gpu_batch.c:170-194,
+    # engine/tests/test_gpt2_gpu_half.c:108-118). Two layers at GPT-2 small's width, steps run eagerly.
+    import json
+
+    from mini_llm_amd.config import config_from_dict
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.ops import kernels
+
+    raw = {"architectures": ["GPT2LMHeadModel"], "n_layer": 2, "n_embd": 768, "n_head": 12, "n_inner": 3072, "vocab_size": 9001,
+           "n_positions": 512, "layer_norm_epsilon": 1e-5, "activation_function": "gelu_new"}
+    engine = Engine.from_random(config_from_dict(raw), 3, EngineOptions(dtype=dtype, max_sessions=8, use_graphs=False))
+    layers = raw["n_layer"]
+    handles = [engine.try_take_cache() for _ in range(8)]
+    rng = np.random.default_rng(0)
+    before = kernels.launch_counts()
+    engine.runner.step([StepEntry(handles[0], rng.integers(0, 9001, 300).tolist(), [299])])
+    prompt_step = kernels.launches_since(before)
+    for h in handles[1:]:
+        engine.runner.step([StepEntry(h, rng.integers(0, 9001, 20).tolist(), [])])
+    before = kernels.launch_counts()
+    logits = engine.runner.step([StepEntry(h, [int(rng.integers(0, 9001))], [0]) for h in handles])
+    decode_step = kernels.launches_since(before)
+    before = kernels.launch_counts()
+    kernels.sample(logits)
+    assert kernels.launches_since(before) == {"sample": 1}
+    if dtype == "bfloat16":
+        # a portion of 300 rows: the four products of a layer stream their operands into LDS, the attention is the streaming one
+        assert prompt_step.get("gemm_stream") == 4 * layers, prompt_step
+        assert prompt_step.get("attention_prefill_stream") == layers and "attention_prefill" not in prompt_step, prompt_step
+        # eight single tokens: the two layer kernels a layer, and embedding, final norm and head around them
+        assert decode_step == {"embed": 1, "decode_attention_half": layers, "decode_mlp_half": layers, "pending_layernorm": 1,
+                               "gemm_tiled": 1}, decode_step
+        assert sum(decode_step.values()) == 2 * layers + 3
+    else:
+        assert prompt_step.get("gemm_tiled") == 4 * layers + 1 and "gemm_stream" not in prompt_step, prompt_step
+        assert prompt_step.get("attention_prefill") == layers, prompt_step
+        # the separate kernels: norm, q/k/v with the cache write, attention, output product cut along K, norm taking its
+        # partial products, up product, down product cut along K; the final norm takes the last partial products
+        assert decode_step == {"embed": 1, "layernorm": 1, "pending_layernorm": 2 * layers, "gemm_skinny": 4 * layers,
+                               "attention_decode": layers, "gemm_tiled": 1}, decode_step
+        assert sum(decode_step.values()) == 7 * layers + 3
+    engine.close()
 
 
 def test_no_garbage_collection_while_a_step_is_captured():
@@ -483,6 +548,53 @@ def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dt
         assert results[True, temperature] == results[False, temperature]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_mixed_steps_take_tokens_from_slots(model_dirs, dtype):
+    # The default serving path: the scheduler one step ahead (decode rows take their token from the last-token slot)
+    # with steps of prompt portions beside decodes replayed from captured graphs once their shape of batch has come
+    # twice. Long prompts under a small budget keep one shape coming (three decodes beside a portion that fills the
+    # budget); the pool is so small that requests are preempted and recomputed. Every request's tokens must be the
+    # plain implementation's greedy ones.
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.step import _PortionGraph
+
+    folder, config, weights = model_dirs["C"]
+    vocab = config["vocab_size"]
+    prompts = [random_tokens(300 + i, n, vocab) for i, n in enumerate((150, 151, 149, 152, 150, 148, 153, 150))]
+    engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=4, max_tokens=42 * 16, page_size=16, max_tokens_per_step=32,
+                                          portion_graph_after=2, step_ahead=True))
+    runner = engine.runner
+    replayed_with_slot_rows, mixed_replays = 0, 0
+    plain_step = runner.step
+
+    def watched_step(entries, observer=None):
+        nonlocal replayed_with_slot_rows, mixed_replays
+        before = runner.portion_graph_steps
+        logits = plain_step(entries, observer)
+        if runner.portion_graph_steps > before:
+            mixed_replays += 1
+            if any(e.from_slot for e in entries) and any(len(e.tokens) > 1 for e in entries):
+                replayed_with_slot_rows += 1
+        return logits
+
+    runner.step = watched_step
+    generated = engine.generate(prompts, max_new_tokens=20)
+    stats = engine.stats()
+    assert stats["preemptions"] >= 1, stats                 # the pool is that small
+    assert runner.portion_graph_steps > 0 and runner.portion_graphs_made >= 1
+    assert replayed_with_slot_rows >= 3, (replayed_with_slot_rows, mixed_replays, runner.portion_graphs_made)
+    assert engine.cache.free_pages() == [engine.cache.pools[0].num_pages] and not engine.cache.requests
+    if dtype == "float32":
+        for prompt, new in zip(prompts, generated):
+            assert new == plain_gpt2.greedy(config, weights, prompt, 20)
+    else:
+        rounded = plain_gpt2.bf16_weights(weights)
+        for prompt, new in zip(prompts, generated):
+            assert len(new) == 20
+            plain_check_greedy(config, rounded, prompt, new, margin=0.03, stored=plain_gpt2.stored_as_bf16)
+    engine.close()
+
+
 def test_cache_sized_by_memory(model_dirs):
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
@@ -494,6 +606,30 @@ def test_cache_sized_by_memory(model_dirs):
     assert engine.generate([prompt], max_new_tokens=6)[0] == plain_gpt2.greedy(config, weights, prompt, 6)
     with pytest.raises(ValueError):
         Engine(folder, EngineOptions(dtype="float32", cache_gib=1.0, max_tokens=1024))
+
+
+def test_the_callers_longest_sequence_narrows_the_models_own(model_dirs):
+    from mini_llm_amd.engine import StepEntry, StepError
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.scheduler import Request
+
+    folder, config, weights = model_dirs["A"]     # 128 positions
+    engine = Engine(folder, EngineOptions(dtype="float32", max_sessions=2, max_length=40, page_size=16))
+    assert engine.cache.max_length == 40 and engine.cache.max_blocks() == 3 and engine.cache.free_pages() == [2 * 3]
+    wider = Engine(folder, EngineOptions(dtype="float32", max_sessions=2, max_length=4096))
+    assert wider.cache.max_length == 128           # never beyond the model's positions
+    wider.close()
+    prompt = random_tokens(90, 30, config["vocab_size"])
+    handle = engine.try_take_cache()
+    with pytest.raises(StepError, match="exceed the 40 positions"):
+        engine.runner.step([StepEntry(handle, prompt + prompt, [0])])
+    assert engine.cache.length(handle) == 0
+    engine.release_cache(handle)
+    got = []
+    engine.submit(Request(prompt, on_token=lambda token, finish: got.append((token, finish)), on_error=got.append, max_new_tokens=30))
+    engine.scheduler.run_until_idle()
+    assert [token for token, _ in got] == plain_gpt2.greedy(config, weights, prompt, 10) and got[-1][1] == "context"
+    engine.close()
 
 
 @pytest.mark.parametrize("seed", [0, 1])

@@ -638,6 +638,18 @@ def test_operands_are_checked_on_the_host(K):
         K.layernorm(x, torch.ones(7, device=DEV), torch.ones(8, device=DEV), 1e-5)
     with pytest.raises(OperandError):
         K.linear(x.t(), torch.zeros((3, 4), device=DEV))  # not contiguous
+    # the library's own entry point refuses a residual sum with a 2-byte output, at every shape (a caller through
+    # ctypes is not behind the checks above): no kernel would add it for some shapes and drop it for others
+    from mini_llm_amd.ops.library import library
+
+    lib = library()
+    for rows in (8, 300):
+        a = torch.zeros((rows, 64), device=DEV, dtype=torch.bfloat16)
+        w = K.pack_matrix(torch.zeros((128, 64), device=DEV, dtype=torch.bfloat16))
+        residual = torch.zeros((rows, 128), device=DEV)
+        out = torch.zeros((rows, 128), device=DEV, dtype=torch.bfloat16)
+        status = lib.mllm_gemm(a.data_ptr(), w.data.data_ptr(), 1, None, residual.data_ptr(), out.data_ptr(), rows, 128, 64, K.BF16, K.BF16, 0, 0, 0, None)
+        assert status != 0 and b"residual" in lib.mllm_last_error()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

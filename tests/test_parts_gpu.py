@@ -531,3 +531,95 @@ def test_toy_with_positions_inside_a_mixer_and_a_routed_feed_forward(tmp_path):
             fed[name] += n
     for name in seqs:
         np.testing.assert_allclose(np.concatenate(got[name]), ref[name], atol=5e-5, rtol=2e-4, err_msg=name)
+
+
+# ------------------------------------------------------------------------------------------------
+# a third toy: no position encoding at all, so the model has no limit of its own and the engine's
+# caller has to name the longest sequence
+# ------------------------------------------------------------------------------------------------
+def define_unbounded_toy():
+    from mini_llm_amd.config import ModelConfig, register_architecture
+    from mini_llm_amd.models import LayerCall, Model
+    from mini_llm_amd.parts import TiedHead, TokenEmbedding, make_part
+
+    @dataclass(frozen=True)
+    class UnboundedConfig(ModelConfig):
+        width: int
+        heads: int
+        inner: int
+        vocab: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["architectures"][0], raw["width"], raw["heads"], raw["inner"], raw["vocab"], raw["eps"])
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "width": self.width, "heads": self.heads, "inner": self.inner,
+                    "vocab": self.vocab, "eps": self.eps}
+
+    def build(config, precision):
+        norm = lambda: make_part("norm", "layernorm", width=config.width, eps=config.eps)
+        block = lambda: make_part(
+            "block", "pre_norm", norm_1=norm(), mixer=make_part("mixer", "causal_attention", width=config.width, n_heads=config.heads),
+            norm_2=norm(), feed_forward=make_part("feed_forward", "dense_mlp", width=config.width, inner=config.inner, activation="gelu_new"),
+            compute_dtype=precision.compute, names=("ln_1.", "mix.", "ln_2.", "mlp."))
+        embedding = TokenEmbedding(config.vocab, config.width)
+        return Model(config, precision, embedding=embedding, position_encoding=None, blocks=[block(), block()],
+                     schedule=[LayerCall(0, 0), LayerCall(1, 1)], final_norm=norm(), head=TiedHead(embedding),
+                     names={"embedding": "wte.", "block": "layers.{i}.", "final_norm": "norm."})
+
+    register_architecture("ToyUnboundedLM", UnboundedConfig, build)
+
+
+def plain_unbounded_toy(raw, w, tokens):
+    d, eps, H = raw["width"], raw["eps"], raw["heads"]
+    w = {k: v.astype(np.float64) for k, v in w.items()}
+    h = w["wte.weight"][tokens]
+    for i in range(2):
+        layer = {name[len(f"layers.{i}."):].replace("mix.", "attn."): t for name, t in w.items() if name.startswith(f"layers.{i}.")}
+        h = P.block(h, layer, H, eps, "gelu_new")
+    return P.lm_head(P.layernorm(h, w["norm.weight"], w["norm.bias"], eps), w["wte.weight"])
+
+
+def test_engine_over_a_model_without_a_position_limit(tmp_path):
+    from mini_llm_amd.config import load_config
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.loading import load_model
+    from mini_llm_amd.weights import write_model_dir
+
+    define_unbounded_toy()
+    raw = {"architectures": ["ToyUnboundedLM"], "width": 64, "heads": 4, "inner": 80, "vocab": 190, "eps": 1e-5}
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    write_model_dir(load_config(tmp_path), 9, tmp_path)
+    weights = P.read_safetensors(tmp_path / "model.safetensors")
+    assert not any(name.startswith("wpe") for name in weights)
+    model = load_model(tmp_path, "float32")
+    assert model.max_positions() is None
+    # nothing says how long a sequence may get: refused, also with the pool's size given
+    for options in (EngineOptions(dtype="float32", max_sessions=3), EngineOptions(dtype="float32", max_sessions=3, max_tokens=512),
+                    EngineOptions(dtype="float32", max_sessions=3, cache_gib=0.01)):
+        with pytest.raises(ValueError, match="max_length"):
+            Engine(model=model, options=options)
+    engine = Engine(model=model, options=EngineOptions(dtype="float32", max_sessions=3, max_length=96, page_size=16, max_tokens_per_step=20))
+    assert engine.cache.max_length == 96 and engine.cache.max_blocks() == 6
+    assert engine.cache.free_pages() == [3 * 6]           # max_sessions sequences of max_length
+    assert engine.runner.use_graphs                        # its decode steps are captured like any other model's
+    prompts = [random_tokens(40 + i, n, 190) for i, n in enumerate((3, 31, 50, 17))]
+    generated = engine.generate(prompts, max_new_tokens=12)
+    assert engine.runner.graph_steps > 0
+    for prompt, new in zip(prompts, generated):
+        tokens = list(prompt)
+        for token in new:
+            logits = plain_unbounded_toy(raw, weights, tokens)[-1]
+            assert logits[token] >= logits.max() - 1e-5, (len(tokens), token, int(logits.argmax()))
+            tokens.append(token)
+        assert len(new) == 12
+    # the caller's limit ends a request as a model's own would
+    from mini_llm_amd.engine.scheduler import Request
+
+    got = []
+    engine.submit(Request(random_tokens(50, 90, 190), on_token=lambda token, finish: got.append(finish), on_error=got.append, max_new_tokens=30))
+    engine.scheduler.run_until_idle()
+    assert got == [None] * 5 + ["context"]
+    engine.close()

@@ -165,6 +165,26 @@ def test_qkv_column_order():
     np.testing.assert_allclose(P.block(x, w, 2, 1e-5, "gelu_new"), x + running_mean, atol=1e-12)
 
 
+def test_query_and_key_columns_are_not_interchangeable():
+    # The reference's own attention vector (engine/tests/test_attention.c:24-54: q = [[1,0],[1,0]],
+    # k = [[1,0],[0,1]], v = [[10,1],[0,20]] -> second row [6.6976156, 7.2745287]) routed through the
+    # whole block, so that it fixes WHICH columns of c_attn are q and which are k
+    # (engine/src/gpt2.c:79-90: q = [0,d), k = [d,2d)). With the two swapped the second row's scores
+    # are equal and it comes out as the mean of v, [5, 10.5].
+    d = 2
+    w = _block_weights(d, 2)
+    x = np.eye(2)                                    # ln_1(x) = [[1,-1],[-1,1]] (eps next to nothing)
+    w["attn.c_attn.bias"][0:2] = [1.0, 0.0]          # q: the bias alone, the same in both rows
+    w["attn.c_attn.weight"][:, 2:4] = [[0.25, -0.25], [-0.25, 0.25]]
+    w["attn.c_attn.bias"][2:4] = [0.5, 0.5]          # k = [[1,0],[0,1]]
+    w["attn.c_attn.weight"][:, 4:6] = [[5.0, -9.5], [0.0, 0.0]]
+    w["attn.c_attn.bias"][4:6] = [5.0, 10.5]         # v = [[10,1],[0,20]]
+    w["attn.c_proj.weight"] = np.eye(d)
+    y = P.block(x, w, 1, 1e-14, "gelu_new")
+    np.testing.assert_allclose(y - x, [[10.0, 1.0], [6.6976156, 7.2745287]], atol=2e-6)
+    assert np.abs((y - x)[1] - [5.0, 10.5]).max() > 1.0
+
+
 def test_model_reduces_to_embedding_head_when_blocks_are_zero():
     cfg = dict(TINY_A, n_inner=256)
     w = P.random_weights(cfg, 0)

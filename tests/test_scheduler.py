@@ -506,3 +506,27 @@ def test_thread_runs_one_step_ahead_and_stops_with_a_step_in_flight():
         time.sleep(0.001)
     s.stop()                                                          # whatever is in flight is forgotten
     assert endless.error is not None and "shutting down" in endless.error and ex.all_free()
+
+
+def test_a_submit_that_races_shutdown_is_always_answered():
+    # another thread submits while this one shuts down: every request either reached the queue before it was drained
+    # or hears the message at once; none is left in a queue nobody looks at again
+    import threading
+
+    for trial in range(20):
+        scheduler = Scheduler(FakeExecutor())
+        sinks, started = [], threading.Event()
+
+        def feed():
+            for i in range(400):
+                sinks.append(submit(scheduler, [100 + i, 1])[0])
+                if i == 20:
+                    started.set()
+
+        thread = threading.Thread(target=feed)
+        thread.start()
+        started.wait()
+        scheduler.shutdown("closing")
+        thread.join()
+        assert len(sinks) == 400 and all(sink.error == "closing" for sink in sinks), trial
+        assert not scheduler.has_work()
