@@ -31,6 +31,7 @@ class RequestCache:
     state_slot: int = NO_PAGE
     reserved: int = 0                                 # tokens beyond ``length`` that have pages
     token_in_slot: bool = False                       # a sampler has left a token in the last-token slot since admission
+    table_changes: int = 0                            # how often a block table of the request has changed (pages taken, given back)
 
 
 class CacheManager:
@@ -147,6 +148,7 @@ class CacheManager:
                 raise OutOfPages(f"request {request_id!r} needs {n} pages of group {self.groups[gi].name}, {pool.num_free} are free")
         for table, n, pool in zip(entry.tables, need, self.pools):
             table.extend(pool.take(n))
+        entry.table_changes += any(need)
         entry.reserved = max(entry.reserved, n_new)
 
     def commit(self, request_id, n_new: int) -> None:
@@ -165,6 +167,7 @@ class CacheManager:
             pool.give([table[b] for b in passed])
             for b in passed:
                 table[b] = NO_PAGE
+            entry.table_changes += bool(passed)
 
     def rollback(self, request_id) -> None:
         """Undoes a reserve whose step did not run: pages beyond the stored length go back."""
@@ -172,6 +175,7 @@ class CacheManager:
         keep = blocks_for(entry.length, self.page_size)
         for pool, table in zip(self.pools, entry.tables):
             pool.give([p for p in table[keep:] if p != NO_PAGE])
+            entry.table_changes += len(table) > keep
             del table[keep:]
         entry.reserved = 0
 

@@ -66,7 +66,7 @@ enum MllmKernel : int {
     MLLM_K_EMBED = 0, MLLM_K_LAYERNORM, MLLM_K_ADD, MLLM_K_CACHE_WRITE, MLLM_K_ATTENTION_GENERAL, MLLM_K_ATTENTION_DECODE,
     MLLM_K_ATTENTION_PREFILL, MLLM_K_ATTENTION_PREFILL_STREAM, MLLM_K_PACK, MLLM_K_CONVERT, MLLM_K_DECODE_ATTENTION_HALF,
     MLLM_K_DECODE_MLP_HALF, MLLM_K_PENDING_SUM, MLLM_K_PENDING_LAYERNORM, MLLM_K_GEMM_SKINNY, MLLM_K_GEMM_TILED, MLLM_K_GEMM_STREAM,
-    MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_KINDS
+    MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_GEMM_BEST, MLLM_K_CHOOSE, MLLM_K_KINDS
 };
 void mllm_count_kernel(MllmKernel kind);
 
@@ -116,6 +116,27 @@ __device__ __forceinline__ float wave_total(float v) {
     float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
     return (r0 + r1) + (r2 + r3);
 }
+
+// (value, index) a comes before b: a NaN beats every number, a larger number a smaller one, and
+// among equals (-0 equals +0) the smaller index wins. These are numpy.argmax's rules, which the
+// reference keeps (engine/include/argmax.h:10-16, engine/src/argmax.cu:8-18). A total order: the
+// best of a set does not depend on the order in which its members are compared.
+__device__ __forceinline__ bool beats(float value, int index, float best, int best_index) {
+    bool value_nan = value != value, best_nan = best != best;
+    if (value_nan != best_nan) return value_nan;
+    if (value_nan || value == best) return index < best_index;
+    return value > best;
+}
+
+// Where a product leaves, instead of its sums, the best of them per row: each wave of each block
+// writes the best (value, column) among its columns of a row to values/indices[row * per_row + block
+// along N * waves along N + wave]. Whoever picks the row's best among them gets the argmax of the
+// row by the rules above, and the sums themselves need not be written (a greedy step's logits).
+struct BestOfColumns {
+    float* values;
+    int* indices;
+    int per_row;
+};
 
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

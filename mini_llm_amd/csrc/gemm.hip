@@ -80,12 +80,14 @@ __device__ __forceinline__ Vec16 mask_piece(Vec16 v, bool valid) {
 // Tiles of A and W go memory -> registers -> LDS; the loads run two tiles ahead of the products
 // (two register sets used in turn), so that one block per compute unit still hides the memory
 // latency: these products are small enough that the grid often is no more than that.
-template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, bool PACKED>
+// BEST: the block leaves no sums but, per row, the best (sum, column) of each of its waves (BestOfColumns).
+template <typename T, typename OutT, int BM, int BN, int WAVES_M, int WAVES_N, bool ALIGNED, bool PACKED, bool BEST = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* __restrict__ A, const T* __restrict__ W,
                                                    const float* __restrict__ bias,
                                                    const float* __restrict__ residual,
                                                    OutT* __restrict__ out, int M, int N, int K,
-                                                   int epilogue, CacheScatter scatter, int k_per_block) {
+                                                   int epilogue, CacheScatter scatter, int k_per_block,
+                                                   BestOfColumns best_out = BestOfColumns{}) {
     constexpr int BK = Tile<T>::BK, VEC = Tile<T>::VEC, PAD = Tile<T>::PAD;
     constexpr int LDK = BK + PAD;
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
@@ -246,6 +248,45 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
     }
 
     // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
+    if constexpr (BEST) {
+        // Per row the best of this wave's columns: first among the lane's own (one per tile along N), then among the
+        // 32 lanes that hold the row (xor steps below 32 stay inside a half of the wave).
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int rows_from = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4);  // the same for the whole wave
+                if (rows_from >= M) continue;
+                const int row = rows_from + 4 * half + (v % 4);
+                float best = -INFINITY;
+                int best_index = 0x7fffffff;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
+                    float value = acc[i][j][v] + early_bias[j];
+                    if (col < N && beats(value, col, best, best_index)) {
+                        best = value;
+                        best_index = col;
+                    }
+                }
+#pragma unroll
+                for (int offset = 16; offset > 0; offset >>= 1) {
+                    float other = __shfl_xor(best, offset, WAVE);
+                    int other_index = __shfl_xor(best_index, offset, WAVE);
+                    if (beats(other, other_index, best, best_index)) {
+                        best = other;
+                        best_index = other_index;
+                    }
+                }
+                if (lane32 == 0 && row < M) {
+                    size_t at = (size_t)row * best_out.per_row + blockIdx.x * WAVES_N + wave_n;
+                    best_out.values[at] = best;
+                    best_out.indices[at] = best_index;
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -610,6 +651,63 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
     else
         MLLM_REQUIRE(false, "gemm: no kernel for input dtype %d with output dtype %d", in_dtype, out_dtype);
     return mllm_check_launch("gemm");
+}
+
+// The tile a product of M rows takes when it leaves the best of its columns instead of its sums
+// (mllm_gemm_best): the tiles the plain product takes for a wide matrix at these row counts.
+namespace {
+struct BestTile { int bm, bn, waves_n; };
+BestTile best_tile(int M) {
+    if (M <= 32) return {32, 128, 4};
+    if (M <= 64) return {64, 64, 2};
+    return {128, 64, 2};
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+void launch_best(const T* a, const T* w, bool packed, const float* bias, int M, int N, int K, BestOfColumns best, hipStream_t stream) {
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM), 1);
+    constexpr int PAIR = 2 * Tile<T>::BK;
+    int k_per_block = ceil_div(K, PAIR) * PAIR;
+    mllm_count_kernel(MLLM_K_GEMM_BEST);
+    if (packed) gemm_kernel<T, float, BM, BN, WAVES_M, WAVES_N, true, true, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, nullptr, nullptr, M, N, K, 0, CacheScatter{}, k_per_block, best);
+    else gemm_kernel<T, float, BM, BN, WAVES_M, WAVES_N, true, false, true><<<grid, 64 * WAVES_M * WAVES_N, 0, stream>>>(a, w, bias, nullptr, nullptr, M, N, K, 0, CacheScatter{}, k_per_block, best);
+}
+
+template <typename T>
+void launch_best_of(const void* A, const void* W, bool packed, const float* bias, int M, int N, int K, BestOfColumns best, hipStream_t stream) {
+    if (M <= 32) launch_best<T, 32, 128, 1, 4>((const T*)A, (const T*)W, packed, bias, M, N, K, best, stream);
+    else if (M <= 64) launch_best<T, 64, 64, 2, 2>((const T*)A, (const T*)W, packed, bias, M, N, K, best, stream);
+    else launch_best<T, 128, 64, 4, 2>((const T*)A, (const T*)W, packed, bias, M, N, K, best, stream);
+}
+}  // namespace
+
+// How many (value, column) pairs per row mllm_gemm_best leaves for a product of M rows with an
+// [N, K] matrix; 0 where it does not take the sizes (K no whole number of 16-byte pieces).
+MLLM_API int mllm_gemm_best_per_row(int M, int N, int K, int in_dtype) {
+    if (M <= 0 || N <= 0 || K <= 0 || (in_dtype != MLLM_F32 && in_dtype != MLLM_BF16)) return 0;
+    if (K % (in_dtype == MLLM_F32 ? 4 : 8)) return 0;
+    BestTile tile = best_tile(M);
+    return ceil_div(N, tile.bn) * tile.waves_n;
+}
+
+// A . W^T (+ bias) whose sums are not written: per row, every wave of every block leaves the best
+// (sum, column) of its columns in values / indices [M, per_row] (per_row as mllm_gemm_best_per_row
+// says; every entry is written, an entry without a column holds -inf and the largest index). The
+// best entry of a row by numpy's argmax rules is the row's argmax: the head of a greedy step,
+// whose logits nobody reads (the reference takes the argmax on the device for the same reason:
+// engine/src/argmax.cu).
+MLLM_API int mllm_gemm_best(const void* A, const void* W, int w_packed, const float* bias, float* values, int* indices,
+                            int per_row, int M, int N, int K, int in_dtype, hipStream_t stream) {
+    MLLM_REQUIRE(M >= 0 && N > 0 && K > 0 && ceil_div(M, 32) <= 65535, "gemm_best: bad sizes M=%d N=%d K=%d", M, N, K);
+    MLLM_REQUIRE(values != nullptr && indices != nullptr, "gemm_best: nowhere to leave the best columns");
+    int expected = mllm_gemm_best_per_row(M, N, K, in_dtype);
+    MLLM_REQUIRE(expected > 0, "gemm_best: no kernel for K=%d in dtype %d", K, in_dtype);
+    MLLM_REQUIRE(per_row == expected, "gemm_best: %d entries per row were given room, the product leaves %d", per_row, expected);
+    if (M == 0) return 0;
+    BestOfColumns best{values, indices, per_row};
+    if (in_dtype == MLLM_F32) launch_best_of<float>(A, W, w_packed != 0, bias, M, N, K, best, stream);
+    else launch_best_of<bf16_t>(A, W, w_packed != 0, bias, M, N, K, best, stream);
+    return mllm_check_launch("gemm_best");
 }
 
 // How many partial products mllm_gemm_split should be asked for at these sizes (1: the product is

@@ -5,16 +5,6 @@ namespace {
 
 constexpr int SAMPLE_THREADS = 1024;
 
-// (value, index) a comes before b: a NaN beats every number, a larger number a smaller one, and
-// among equals (-0 equals +0) the smaller index wins. These are numpy.argmax's rules, which the
-// reference keeps (engine/include/argmax.h:10-16, engine/src/argmax.cu:8-18).
-__device__ __forceinline__ bool beats(float value, int index, float best, int best_index) {
-    bool value_nan = value != value, best_nan = best != best;
-    if (value_nan != best_nan) return value_nan;
-    if (value_nan || value == best) return index < best_index;
-    return value > best;
-}
-
 __device__ __forceinline__ void block_best(float& value, int& index, float* shared_values,
                                            int* shared_indices) {
 #pragma unroll
@@ -175,6 +165,84 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
 }
 
+// The end of a decode step that chooses its tokens on the device: per row the best of its candidates
+// (what mllm_gemm_best left of a greedy step's logits; or one candidate a row, the token another
+// kernel drew), and everything the next step of the same requests needs, so that the host neither
+// reads nor writes device memory between two steps (the reference feeds the token back on the
+// device and reads it from the host later: engine/src/gpt2_gpu_greedy.cu:80-123,
+// docs/kernels/007_fewer_launches.md:54).
+//
+// Per live row r (state_slots[r] >= 0; other rows are padding and give -1): the token goes to out_tokens[r], to the
+// request's last-token slot token_slots[state_slots[r]], and to row *cursor of the ring of token rows in page-locked host
+// memory (one store of the whole row by the first lanes: the host reads it after the event that
+// follows the step). With `advance` the row's position and stored length grow by one, its cache row
+// of every group is looked up in the block table for the new position (-1 where the table has no page
+// there yet: the host brings the table before that step runs), and its token source becomes its own
+// slot. One block; wave w picks the rows w, w + waves, ...
+struct StepGroups {
+    const int* tables[4];
+    int* slots[4];
+    int count, table_width, page_shift;
+};
+
+constexpr int CHOOSE_THREADS = 1024;
+
+__global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
+    const float* __restrict__ values, const int* __restrict__ indices, int per_row, int n_rows,
+    const int* __restrict__ state_slots, int* __restrict__ token_slots,
+    int* __restrict__ out_tokens, int* __restrict__ host_ring, int ring_rows, int ring_stride, int* __restrict__ cursor,
+    int advance, int* __restrict__ positions, int* __restrict__ context_lens, int* __restrict__ token_sources,
+    StepGroups groups) {
+    extern __shared__ int chosen[];  // [n_rows]
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+    const int ring_row = cursor ? *cursor : 0;
+    for (int row = wave; row < n_rows; row += CHOOSE_THREADS / WAVE) {
+        float best = -INFINITY;
+        int best_index = 0x7fffffff;
+        for (int c = lane; c < per_row; c += WAVE) {
+            size_t at = (size_t)row * per_row + c;
+            float value = values ? values[at] : 0.0f;
+            int index = indices[at];
+            if (beats(value, index, best, best_index)) {
+                best = value;
+                best_index = index;
+            }
+        }
+#pragma unroll
+        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+            float other = __shfl_xor(best, offset, WAVE);
+            int other_index = __shfl_xor(best_index, offset, WAVE);
+            if (beats(other, other_index, best, best_index)) {
+                best = other;
+                best_index = other_index;
+            }
+        }
+        if (lane == 0) chosen[row] = best_index;
+    }
+    __syncthreads();
+    for (int row = tid; row < n_rows; row += CHOOSE_THREADS) {
+        const int slot = state_slots[row];
+        const bool live = slot >= 0;
+        const int token = live ? chosen[row] : -1;
+        out_tokens[row] = token;
+        if (host_ring) host_ring[(size_t)ring_row * ring_stride + row] = token;
+        if (!live) continue;
+        token_slots[slot] = token;
+        if (advance) {
+            const int position = positions[row] + 1;
+            positions[row] = position;
+            context_lens[row] = position;
+            token_sources[row] = slot;
+            const int block = position >> groups.page_shift, offset = position & ((1 << groups.page_shift) - 1);
+            for (int g = 0; g < groups.count; g++) {
+                int page = block < groups.table_width ? groups.tables[g][(size_t)row * groups.table_width + block] : -1;
+                groups.slots[g][row] = page >= 0 ? (page << groups.page_shift) + offset : -1;
+            }
+        }
+    }
+    if (cursor && tid == 0) *cursor = (ring_row + 1) % ring_rows;  // every thread has read it before the barrier above
+}
+
 }  // namespace
 
 MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float* temperatures,
@@ -186,4 +254,38 @@ MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float
     sample_kernel<<<n_rows, SAMPLE_THREADS, 0, stream>>>(logits, vocab, temperatures, top_ps,
                                                          (const uint64_t*)seeds, steps, out_tokens, token_slots, slot_of_row);
     return mllm_check_launch("sample");
+}
+
+// See choose_kernel. values may be null (every row has candidates of equal rank: the first index
+// wins, with per_row = 1 the one given); host_ring and cursor may be null; without `advance` the
+// arrays behind it are not touched. group_tables / group_slots: n_groups pointers each.
+MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, int n_rows,
+                         const int* state_slots, int* token_slots, int* out_tokens, int* host_ring, int ring_rows,
+                         int ring_stride, int* cursor, int advance, int* positions, int* context_lens, int* token_sources,
+                         const int* const* group_tables, int* const* group_slots, int n_groups, int table_width,
+                         int page_size, hipStream_t stream) {
+    MLLM_REQUIRE(n_rows >= 0 && n_rows <= 8192 && per_row >= 1, "choose: bad sizes rows=%d candidates=%d", n_rows, per_row);
+    MLLM_REQUIRE(indices && state_slots && token_slots && out_tokens, "choose: an operand is missing");
+    MLLM_REQUIRE(!host_ring || (ring_rows >= 1 && ring_stride >= n_rows), "choose: the ring's rows are shorter than the batch");
+    MLLM_REQUIRE(!cursor || host_ring, "choose: a cursor without a ring");
+    StepGroups groups{};
+    if (advance) {
+        MLLM_REQUIRE(positions && context_lens && token_sources, "choose: nothing to advance");
+        MLLM_REQUIRE(n_groups >= 0 && n_groups <= 4, "choose: %d cache groups, at most 4 are advanced on the device", n_groups);
+        MLLM_REQUIRE(page_size > 0 && (page_size & (page_size - 1)) == 0 && (n_groups == 0 || table_width > 0), "choose: bad page size or table width");
+        for (int g = 0; g < n_groups; g++) {
+            MLLM_REQUIRE(group_tables[g] && group_slots[g], "choose: group %d has no table or slots", g);
+            groups.tables[g] = group_tables[g];
+            groups.slots[g] = group_slots[g];
+        }
+        groups.count = n_groups;
+        groups.table_width = table_width;
+        while ((1 << groups.page_shift) < page_size) groups.page_shift++;
+    }
+    if (n_rows == 0) return 0;
+    mllm_count_kernel(MLLM_K_CHOOSE);
+    choose_kernel<<<1, CHOOSE_THREADS, (size_t)n_rows * sizeof(int), stream>>>(
+        values, indices, per_row, n_rows, state_slots, token_slots, out_tokens, host_ring, ring_rows, ring_stride,
+        cursor, advance, positions, context_lens, token_sources, groups);
+    return mllm_check_launch("choose");
 }

@@ -206,6 +206,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     q_starts[n_requests + 1 :] = n_tokens
     context_lens[:n_requests] = contexts
     state_slots[:n_requests] = [r.state_slot for r in records]
+    state_slots[n_requests:] = -1    # padding: no request, no slot
     for i, e in enumerate(entries):
         lo, hi = starts[i], starts[i + 1]
         tokens[lo:hi] = e.token_array()
@@ -228,6 +229,7 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         tables.append(table)
         slots.append(slot)
     logit_slots = sections[-1]
+    logit_slots[:] = -1
     at = 0
     for i, e in enumerate(given):
         for w in e.want:
@@ -273,6 +275,7 @@ class DecodeBatchBuilder:
         lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
         for _ in range(n_groups):
             lengths += [capacity * self.table_width, capacity]
+        lengths.append(1)   # the row of the token ring that a step which chooses its tokens on the device writes next
         self.offsets, total = [], 0
         for n in lengths:
             self.offsets.append(total)
@@ -284,6 +287,7 @@ class DecodeBatchBuilder:
         self.context_lens, self.state_slots, self.logit_rows, self.token_sources = view(4), view(5), view(6), view(7)
         self.tables = [view(8 + 2 * g).reshape(capacity, self.table_width) for g in range(n_groups)]
         self.slots = [view(9 + 2 * g) for g in range(n_groups)]
+        self.cursor = view(8 + 2 * n_groups)
         self.filled = capacity  # rows that held a request in the previous step (all, so the first fill pads all)
 
     def fill(self, entries) -> np.ndarray:
@@ -294,7 +298,7 @@ class DecodeBatchBuilder:
         self.token_request[:stale] = -1
         self.q_starts[:] = n
         self.context_lens[:stale] = 0
-        self.state_slots[:stale] = 0
+        self.state_slots[:stale] = -1
         self.logit_rows[:] = 0
         self.token_sources[:stale] = -1
         for table, slots in zip(self.tables, self.slots):
@@ -331,3 +335,7 @@ class DecodeBatchBuilder:
             logit_slots=views[5],  # every request has one logit row, in its own place
             groups=groups, request_ids=[e.request_id for e in entries], host={},
         )
+
+    def cursor_view(self, device_flat):
+        at = self.offsets[8 + 2 * len(self.tables)]
+        return device_flat[at : at + 1]

@@ -44,7 +44,6 @@ class _Executor:
     def __init__(self, engine: "Engine"):
         self._engine = engine
         self.page_size = engine.cache.page_size
-        self._hosts, self._turn = [], 0
 
     def max_positions(self):
         """The longest sequence a request may reach: the model's own limit or the one the cache was made for."""
@@ -88,38 +87,23 @@ class _Executor:
     # One step ahead: launch() queues the step, the sampling (each token also goes to its request's
     # last-token slot, where the next step finds it) and the copy of the tokens into pinned host
     # memory; collect() waits for that copy alone, not for what was launched after it.
-    RING = 4
-
     def launch(self, entries, sampling, steps):
-        import torch
-
         engine = self._engine
         entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want, e.from_slot) for e in entries]
+        if all(p.greedy for p in sampling):
+            return engine.runner.step(entries, choose=True)     # greedy: chosen inside the step
         logits = engine.runner.step(entries)
         if logits is None:
             return None
-        n = logits.shape[0]
         tokens = engine.sampler.sample(logits, sampling, steps, token_slots=engine.cache.last_token,
                                        slot_of_row=engine.runner.last_batch.logit_slots)
         for entry in entries:
             if entry.want:
                 engine.cache.note_sampled(entry.request_id)
-        if not self._hosts or self._hosts[0].shape[0] < n:
-            size = max(n, engine.options.max_sessions)
-            self._hosts = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
-        host = self._hosts[self._turn % self.RING]
-        self._turn += 1
-        host[:n].copy_(tokens, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
-        return host, n, event
+        return engine.runner.tokens_to_host(tokens, logits.shape[0])
 
     def collect(self, handle):
-        if handle is None:
-            return []
-        host, n, event = handle
-        event.synchronize()
-        return host[:n].tolist()
+        return [] if handle is None else handle.tolist()
 
 
 class Session:
@@ -200,8 +184,7 @@ class Engine:
         self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step,
                                    step_ahead=options.step_ahead)
         self._next_handle = 0
-        self._queued = collections.deque()   # (pinned tokens, count, event) of steps whose tokens were not taken yet
-        self._token_buffers, self._queue_turn = [], 0
+        self._queued = collections.deque()   # the chosen tokens of steps that were not taken yet
 
     @classmethod
     def from_random(cls, config, seed: int, options: EngineOptions = EngineOptions()):
@@ -248,27 +231,17 @@ class Engine:
     def release_cache(self, handle) -> None:
         self.cache.close(handle)
 
-    def _greedy(self, logits, handles):
-        """argmax per row on the device; each token is also left in its request's last-token slot."""
-        n = len(handles)
-        tokens = self.sampler.sample(logits, [SamplingParams()] * n, [0] * n, token_slots=self.cache.last_token,
-                                     slot_of_row=self.runner.last_batch.state_slots)
-        for handle in handles:
-            self.cache.note_sampled(handle)
-        return tokens
-
     def prefill_greedy(self, handle, token_ids) -> int:
+        """The prompt in one step; returns its greedy next token, which also stays in the sequence's last-token slot."""
         tokens = [int(t) for t in token_ids]
         if not tokens:
             raise RuntimeError("the prompt has no tokens")
-        logits = self.runner.step([StepEntry(handle, tokens, [len(tokens) - 1])])
-        return int(self._greedy(logits, [handle]).cpu()[0])
+        return self.runner.step([StepEntry(handle, tokens, [len(tokens) - 1])], choose=True).tolist()[0]
 
     def decode_batch(self, handles, tokens) -> list[int]:
         if len(handles) != len(tokens) or not handles:
             raise RuntimeError("a batch has one token per sequence and at least one sequence")
-        logits = self.runner.step([StepEntry(h, [int(t)], [0]) for h, t in zip(handles, tokens)])
-        return self._greedy(logits, list(handles)).cpu().tolist()
+        return self.runner.step([StepEntry(h, [int(t)], [0]) for h, t in zip(handles, tokens)], choose=True).tolist()
 
     # --- queued decoding: step n+1 is launched before the host has read token n ------------------------
     # (the reference's enqueue / take: engine/src/gpt2_gpu_greedy.cu:80-123, native.py:123-155)
@@ -284,24 +257,13 @@ class Engine:
             raise RuntimeError("a batch has at least one sequence")
         if len(self._queued) >= self.MAX_QUEUED:
             raise RuntimeError(f"{self.MAX_QUEUED} steps are queued already: take one first")
-        logits = self.runner.step([StepEntry(h, [0], [0], from_slot=True) for h in handles])
-        tokens = self._greedy(logits, list(handles))
-        if len(self._token_buffers) < self.MAX_QUEUED:
-            self._token_buffers.append(torch.empty(self.options.max_sessions, dtype=torch.int32, pin_memory=True))
-        host = self._token_buffers[self._queue_turn % self.MAX_QUEUED]
-        self._queue_turn += 1
-        host[: len(handles)].copy_(tokens, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
-        self._queued.append((host, len(handles), event))
+        self._queued.append(self.runner.step([StepEntry(h, [0], [0], from_slot=True) for h in handles], choose=True))
 
     def take(self) -> list[int]:
         """The tokens of the oldest queued step (waits for it)."""
         if not self._queued:
             raise RuntimeError("no step is queued")
-        host, n, event = self._queued.popleft()
-        event.synchronize()
-        return host[:n].tolist()
+        return self._queued.popleft().tolist()
 
     # --- continuous batching ------------------------------------------------------------------------------
     def submit(self, request: Request) -> None:

@@ -43,21 +43,52 @@ class StepError(ValueError):
     """The batch cannot be run; nothing has been changed."""
 
 
-class _DecodeGraph:
-    """One captured decode step for up to ``capacity`` requests."""
+TOKEN_RING_ROWS = 8   # steps whose chosen tokens stay readable on the host after they were launched
 
-    def __init__(self, runner: "ModelRunner", capacity: int):
+
+class ChosenTokens:
+    """The tokens a step chose on the device: ``device`` (int32, one per wanted row, valid until the next step) and, on
+    the host, a row of page-locked memory that is complete once ``event`` has passed (``tolist`` waits for it). A row
+    is used again ``TOKEN_RING_ROWS`` steps later."""
+
+    __slots__ = ("device", "_host", "_n", "_event")
+
+    def __init__(self, device, host, n, event):
+        self.device, self._host, self._n, self._event = device, host, n, event
+
+    def __len__(self):
+        return self._n
+
+    def tolist(self) -> list:
+        self._event.synchronize()
+        return self._host[: self._n].tolist()
+
+
+class _DecodeGraph:
+    """One captured decode step for up to ``capacity`` requests. ``chooses``: the captured step ends with the greedy
+    choice of its tokens (models.TokenChoice) and moves its batch on by one token on the device, so that the next step
+    of the same requests, each taking its token from its last-token slot, is replayed without anything being copied to
+    the device before it or from the device after it: the tokens arrive in a ring of rows in page-locked host memory."""
+
+    def __init__(self, runner: "ModelRunner", capacity: int, chooses: bool = False):
         import torch
 
-        self.runner, self.capacity = runner, capacity
+        self.runner, self.capacity, self.chooses = runner, capacity, chooses
         self.builder = DecodeBatchBuilder(runner.cache, capacity)
         self.buffer = torch.zeros(len(self.builder.flat), dtype=torch.int32, device=runner.device)
         self.static_batch = self.builder.batch(self.buffer, [])
         self.graph = None
         self.logits = None
+        if chooses:
+            self.ring = torch.full((TOKEN_RING_ROWS, capacity), -1, dtype=torch.int32).pin_memory()
+            self.ring_at = 0        # the ring row the next step writes: the host's count of the device's cursor
+            self.on_device = None   # per row (request's cache entry, its table_changes, its length) that the device's batch stands at
+            self.uploads = 0
 
     def run(self, entries):
         runner = self.runner
+        if self.chooses:
+            return self._run_choosing(entries)
         runner.staging.upload(self.builder.fill(entries), into=self.buffer)
         batch = self.static_batch
         batch.request_ids = [e.request_id for e in entries]
@@ -66,15 +97,53 @@ class _DecodeGraph:
         self.graph.replay()
         return batch, self.logits[: len(entries)]
 
+    def _run_choosing(self, entries):
+        import torch
 
-def _capture(runner, batch):
-    """Runs the batch once eagerly (on a side stream, as capture needs), then captures the same."""
+        from ..models.base import TokenChoice
+
+        runner, cache = self.runner, self.runner.cache
+        records = [cache.requests[e.request_id] for e in entries]
+        stands = self.on_device
+        # The device has moved the last step's batch on by itself. It is this step's batch if the same requests come
+        # again in the same rows, each with the token in its slot, and no block table has changed since (a request that
+        # reaches a new page, or gives one back, has: then everything is brought from the host as ever).
+        carried_on = (stands is not None and len(stands) == len(records) and all(e.from_slot for e in entries)
+                      and all(r is at[0] and r.table_changes == at[1] and r.length == at[2] for r, at in zip(records, stands)))
+        if not carried_on:
+            flat = self.builder.fill(entries)
+            self.builder.cursor[0] = self.ring_at
+            runner.staging.upload(flat, into=self.buffer)
+            self.uploads += 1
+        batch = self.static_batch
+        batch.request_ids = [e.request_id for e in entries]
+        if self.graph is None:
+            choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True)
+            self.graph, self.logits = _capture(runner, batch, choice)
+        self.graph.replay()
+        row = self.ring[self.ring_at]
+        self.ring_at = (self.ring_at + 1) % TOKEN_RING_ROWS
+        self.on_device = [(r, r.table_changes, r.length + 1) for r in records]
+        event = torch.cuda.Event()
+        event.record()
+        return batch, ChosenTokens(self.logits[: len(entries)], row, len(entries), event)
+
+
+def _capture(runner, batch, choice=None):
+    """Runs the batch once eagerly (on a side stream, as capture needs), then captures the same. With ``choice`` the
+    captured step ends with the choice of its tokens; the eager run then chooses into memory of its own and moves
+    nothing on, so that the first replay finds everything as the eager run found it."""
     import torch
 
+    warm = {}
+    if choice is not None:
+        from dataclasses import replace
+
+        warm["choice"] = replace(choice, token_slots=torch.empty_like(choice.token_slots), host_ring=None, cursor=None, advance=False)
     side = torch.cuda.Stream(device=runner.device)
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        runner.forward(batch)
+        runner.forward(batch, **warm)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize(runner.device)
     graph = torch.cuda.CUDAGraph()
@@ -86,7 +155,7 @@ def _capture(runner, batch):
     gc.disable()
     try:
         with torch.cuda.graph(graph):
-            logits = runner.forward(batch)
+            logits = runner.forward(batch) if choice is None else runner.forward(batch, choice=choice)
     finally:
         if collecting:
             gc.enable()
@@ -138,6 +207,7 @@ class ModelRunner:
         self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
         self.portion_graph_after = PORTION_GRAPH_AFTER if portion_graph_after is None else int(portion_graph_after)
         self.portion_graph_steps = 0
+        self._token_rows, self._token_turn = [], 0
         self.portion_graphs_made = 0      # captures of steps with prompt portions, and those given up for a newer shape
         self.portion_graphs_dropped = 0
 
@@ -205,23 +275,26 @@ class ModelRunner:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
 
-    def forward(self, batch, resolve: bool = True, observer=None):
+    def forward(self, batch, resolve: bool = True, observer=None, choice=None):
         """Tokens that come from last-token slots are fetched on the device, then the model runs."""
-        if observer is None:
-            return self.model.forward(batch, self.cache, resolve_tokens=resolve)
-        return self.model.forward(batch, self.cache, resolve_tokens=resolve, observer=observer)
+        extra = {}
+        if observer is not None:
+            extra["observer"] = observer
+        if choice is not None:
+            extra["choice"] = choice
+        return self.model.forward(batch, self.cache, resolve_tokens=resolve, **extra)
 
-    def _graph_for(self, entries):
+    def _graph_for(self, entries, choose: bool = False):
         if not self.use_graphs:
             return None
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
-            return self._portion_graph_for(entries)
+            return self._portion_graph_for(entries)   # its tokens, if asked for, are chosen from its logits behind the replay
         if len(entries) > GRAPH_BUCKETS[-1]:
             return None
         capacity = next(b for b in GRAPH_BUCKETS if b >= len(entries))
-        if capacity not in self._graphs:
-            self._graphs[capacity] = _DecodeGraph(self, capacity)
-        return self._graphs[capacity]
+        if (capacity, choose) not in self._graphs:
+            self._graphs[capacity, choose] = _DecodeGraph(self, capacity, chooses=choose)
+        return self._graphs[capacity, choose]
 
     def _portion_graph_for(self, entries):
         """The captured step for batches of this shape, once the shape has come often enough."""
@@ -253,13 +326,17 @@ class ModelRunner:
         self.portion_graphs_made += 1
         return graph
 
-    def step(self, entries: list[StepEntry], observer=None):
+    def step(self, entries: list[StepEntry], observer=None, choose: bool = False):
         """Runs the entries as one batch. Returns float32 logits [wanted places, vocab] on the
         device (None if nothing is wanted), in the order of the entries and of each ``want``;
         they are valid until the next step. Raises StepError / OutOfPages before anything has
         changed. ``observer(name, rows)`` is shown the residual stream after the embedding and
         after each layer, the rows in the order of the entries and of their tokens (such a step
-        is not replayed from a graph)."""
+        is not replayed from a graph).
+
+        ``choose``: the step also chooses the greedy token at every wanted place, on the device, leaves it in the
+        request's last-token slot and returns ``ChosenTokens`` instead of logits (a decode step does all of it inside
+        its captured graph, and is replayed without a copy to or from the device while the same requests go on)."""
         self.validate(entries)
         reserved = []
         try:
@@ -271,7 +348,7 @@ class ModelRunner:
                 self.cache.rollback(request_id)
             raise
         try:
-            graph = self._graph_for(entries) if observer is None else None
+            graph = self._graph_for(entries, choose) if observer is None else None
             if graph is not None:
                 batch, logits = graph.run(entries)
                 if isinstance(graph, _PortionGraph):
@@ -285,12 +362,40 @@ class ModelRunner:
                     rows = batch.rows_in_order_of([e.request_id for e in entries])
                     in_given_order = lambda name, hidden: observer(name, hidden[rows])
                 logits = self.forward(batch, resolve=any(e.from_slot for e in entries), observer=in_given_order)
+            if choose and not isinstance(logits, ChosenTokens):
+                logits = self._choose_from_logits(logits, batch)
         except Exception:
             for request_id in reserved:
                 self.cache.rollback(request_id)
             raise
         for entry in entries:
             self.cache.commit(entry.request_id, len(entry.tokens))
+            if choose and entry.want:
+                self.cache.note_sampled(entry.request_id)
         self.steps_run += 1
         self.last_batch = batch
         return logits
+
+    def _choose_from_logits(self, logits, batch):
+        """The greedy tokens of a step that was not captured with its choice: the sampler's argmax over the logits, each
+        token left in its request's last-token slot."""
+        if logits is None:
+            return None
+        from ..ops import kernels
+
+        tokens = kernels.sample(logits, token_slots=self.cache.last_token, slot_of_row=batch.logit_slots)
+        return self.tokens_to_host(tokens, logits.shape[0])
+
+    def tokens_to_host(self, tokens, n: int) -> ChosenTokens:
+        """Queues the copy of ``n`` chosen tokens into page-locked host memory; ``ChosenTokens.tolist`` waits for that
+        copy alone, not for what is launched after it."""
+        import torch
+
+        if not self._token_rows or self._token_rows[0].shape[0] < n:
+            self._token_rows = [torch.empty(max(n, 64), dtype=torch.int32, pin_memory=True) for _ in range(TOKEN_RING_ROWS)]
+        row = self._token_rows[self._token_turn % TOKEN_RING_ROWS]
+        self._token_turn += 1
+        row[:n].copy_(tokens[:n], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return ChosenTokens(tokens, row, n, event)

@@ -32,6 +32,19 @@ class CacheGroupSpec:
     window: int | None
 
 
+@dataclass
+class TokenChoice:
+    """Asks a step to choose its tokens on the device, greedily, as its last kernel: one token per wanted row, left in
+    the request's last-token slot (``token_slots``: the cache's), and, with ``host_ring`` / ``cursor``, in a ring of
+    rows in page-locked host memory (kernels.choose). ``advance``: a step of single tokens also moves its batch on by
+    one token on the device, so that the same requests' next step needs nothing from the host."""
+
+    token_slots: object
+    host_ring: object = None
+    cursor: object = None
+    advance: bool = False
+
+
 class Model(Part):
     def __init__(self, config, precision, *, embedding: TokenEmbedding, position_encoding: PositionEncoding | None,
                  blocks: list, schedule: list, final_norm: Norm, head, names: dict):
@@ -107,9 +120,10 @@ class Model(Part):
                 out[call.cache] = need
         return out
 
-    def forward(self, batch, cache, resolve_tokens: bool = False, observer=None):
+    def forward(self, batch, cache, resolve_tokens: bool = False, observer=None, choice: TokenChoice | None = None):
         """The whole step: embeds the batch's tokens, runs the schedule over the cache, and
-        returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only. With
+        returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only (with
+        ``choice``: the greedy token of each wanted row instead, int32 on the device). With
         ``resolve_tokens`` the rows that name a last-token slot take their token from it.
         ``observer(name, rows)``, if given, is shown the residual stream (float32 [tokens, width],
         rows in the batch's order) after the embedding (name "embedding") and after each entry of
@@ -133,4 +147,20 @@ class Model(Part):
             hidden = kernels.settle(hidden)
         # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
         normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
-        return self.head.forward(normed)
+        if choice is None:
+            return self.head.forward(normed)
+        # Greedy tokens on the device. A head that can leave the best of its columns instead of all of them does (the
+        # logits of a greedy step are read by nobody); any other head's logits go through the sampler's argmax.
+        best = self.head.forward_best(normed) if hasattr(self.head, "forward_best") else None
+        if best is None:
+            values, indices = None, kernels.sample(self.head.forward(normed)).view(-1, 1)
+        else:
+            values, indices = best
+        advance = None
+        if choice.advance:
+            if batch.max_q_len != 1 or batch.n_logit_rows != batch.n_tokens:
+                raise ValueError("only a step of single tokens that all want their logits can be moved on by one on the device")
+            advance = kernels.StepAdvance(batch.positions, batch.context_lens, batch.token_sources, [g.block_tables for g in batch.groups],
+                                          [g.slots for g in batch.groups], cache.page_size)
+        return kernels.choose(values, indices, batch.logit_slots, choice.token_slots, host_ring=choice.host_ring, cursor=choice.cursor,
+                              advance=advance)

@@ -459,6 +459,102 @@ def sample(logits, temperatures=None, top_ps=None, seeds=None, steps=None, out=N
     return out
 
 
+def best_per_row(rows: int, weight, dtype) -> int:
+    """How many (value, column) pairs a row ``linear_best`` leaves for so many rows with this weight; 0 where it has no
+    kernel for the sizes."""
+    _, _, n, k = _matrix(weight, "weight", dtype)
+    return int(library().mllm_gemm_best_per_row(int(rows), n, k, _code(dtype)))
+
+
+def linear_best(x, weight, bias=None):
+    """x @ weight.T (+ bias) without writing the sums: (values float32 [rows, c], indices int32 [rows, c]), for every row
+    the best (sum, column) of c disjoint sets of columns that together are all columns. The best pair of a row by
+    numpy's argmax rules (``choose``) is the row's argmax. For the head of a step that decodes greedily."""
+    _device_tensor(x, "x", dim=2)
+    m, k = x.shape
+    w_ptr, w_packed, n, w_cols = _matrix(weight, "weight", x.dtype)
+    if not (w_cols == k):
+        raise OperandError(f"x has {k} columns but weight has {w_cols}")
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == n, "bias does not match weight")
+    per_row = int(library().mllm_gemm_best_per_row(m, n, k, _code(x.dtype)))
+    _require(per_row > 0, f"no kernel leaves the best columns of a product with K = {k}")
+    values = torch.empty((m, per_row), dtype=torch.float32, device=x.device)
+    indices = torch.empty((m, per_row), dtype=torch.int32, device=x.device)
+    check(library().mllm_gemm_best(_ptr(x), w_ptr, w_packed, _ptr(bias), _ptr(values), _ptr(indices), per_row, m, n, k, _code(x.dtype), _stream()))
+    return values, indices
+
+
+@dataclass
+class StepAdvance:
+    """What ``choose`` moves on by one token for every live row, so that the same requests' next step finds its batch on
+    the device: positions and stored lengths, the source of each row's token (its own last-token slot from then on), and
+    per cache group the row a token's key and value go to, looked up in the group's block table ([rows, table_width],
+    int32; pages of ``page_size`` tokens)."""
+
+    positions: torch.Tensor
+    context_lens: torch.Tensor
+    token_sources: torch.Tensor
+    block_tables: list
+    slots: list
+    page_size: int
+
+
+def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, cursor=None, advance: StepAdvance | None = None):
+    """One token per row from its candidates: the best (value, index) pair by numpy's argmax rules (``values`` None: the
+    smallest index; one candidate a row: that one). Rows whose ``state_slots`` entry is negative are padding and give -1. The
+    token of a live row also goes to token_slots[state_slots[row]] and, with ``host_ring`` (int32 [ring rows, >= rows] in
+    page-locked host memory) to the ring row that ``cursor`` (int32 [1] on the device) names, which then moves on by one.
+    ``advance``: see StepAdvance. Returns the tokens (int32 [rows], on the device)."""
+    _device_tensor(indices, "indices", torch.int32, 2)
+    rows, per_row = indices.shape
+    _require(per_row >= 1, "a row needs at least one candidate")
+    if values is not None:
+        _device_tensor(values, "values", torch.float32, 2)
+        _require(values.shape == indices.shape, "values and indices differ in shape")
+    _device_tensor(state_slots, "state_slots", torch.int32, 1)
+    _require(state_slots.shape[0] >= rows, "state_slots has fewer entries than rows")
+    _device_tensor(token_slots, "token_slots", torch.int32, 1)
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=indices.device)
+    _device_tensor(out, "out", torch.int32, 1)
+    _require(out.shape[0] >= rows, "out is too short")
+    ring_rows = ring_stride = 0
+    if host_ring is not None:
+        _require(isinstance(host_ring, torch.Tensor) and host_ring.dtype == torch.int32 and host_ring.dim() == 2 and host_ring.is_contiguous()
+                 and host_ring.is_pinned(), "the ring must be a contiguous int32 matrix in page-locked host memory")
+        ring_rows, ring_stride = host_ring.shape
+        _require(ring_stride >= rows, "the ring's rows are shorter than the batch")
+        _device_tensor(cursor, "cursor", torch.int32, 1)
+    else:
+        _require(cursor is None, "a cursor without a ring")
+    tables = slots = None
+    n_groups = table_width = page_size = 0
+    positions = context_lens = sources = None
+    if advance is not None:
+        positions, context_lens, sources = advance.positions, advance.context_lens, advance.token_sources
+        for t, name in ((positions, "positions"), (context_lens, "context_lens"), (sources, "token_sources")):
+            _device_tensor(t, name, torch.int32, 1)
+            _require(t.shape[0] >= rows, f"{name} has fewer entries than rows")
+        n_groups, page_size = len(advance.block_tables), int(advance.page_size)
+        _require(len(advance.slots) == n_groups and n_groups <= 4, "one row of slots per block table, at most four groups")
+        import ctypes
+
+        for g, (table, slot) in enumerate(zip(advance.block_tables, advance.slots)):
+            _device_tensor(table, f"block table {g}", torch.int32, 2)
+            _device_tensor(slot, f"slots {g}", torch.int32, 1)
+            _require(table.shape[0] >= rows and slot.shape[0] >= rows, f"group {g} has fewer rows than the batch")
+            _require(g == 0 or table.shape[1] == advance.block_tables[0].shape[1], "the groups' block tables differ in width")
+        table_width = advance.block_tables[0].shape[1] if n_groups else 0
+        tables = (ctypes.c_void_p * max(n_groups, 1))(*[t.data_ptr() for t in advance.block_tables])
+        slots = (ctypes.c_void_p * max(n_groups, 1))(*[t.data_ptr() for t in advance.slots])
+    check(library().mllm_choose(_ptr(values), _ptr(indices), per_row, rows, _ptr(state_slots), _ptr(token_slots), _ptr(out),
+                                _ptr(host_ring), ring_rows, ring_stride, _ptr(cursor), int(advance is not None), _ptr(positions), _ptr(context_lens),
+                                _ptr(sources), tables, slots, n_groups, table_width, page_size, _stream()))
+    return out
+
+
 # -- a whole layer for rows that bring one token each -------------------------------------------------
 @dataclass
 class PendingRows:

@@ -35,3 +35,12 @@ class TiedHead(Part):
         import torch
 
         return kernels.linear(x, self.embedding.weight, out_dtype=torch.float32)
+
+    def forward_best(self, x):
+        """For a step that decodes greedily: instead of the logits, per row the best (logit, token) of each of a few
+        hundred disjoint parts of the vocabulary (kernels.linear_best), among which ``kernels.choose`` finds the row's
+        argmax; None where that kernel does not take the sizes (the caller then takes the logits). A head without this
+        method is asked for its logits."""
+        if not kernels.best_per_row(x.shape[0], self.embedding.weight, x.dtype):
+            return None
+        return kernels.linear_best(x, self.embedding.weight)

@@ -567,10 +567,10 @@ def test_captured_mixed_steps_take_tokens_from_slots(model_dirs, dtype):
     replayed_with_slot_rows, mixed_replays = 0, 0
     plain_step = runner.step
 
-    def watched_step(entries, observer=None):
+    def watched_step(entries, *args, **kwargs):
         nonlocal replayed_with_slot_rows, mixed_replays
         before = runner.portion_graph_steps
-        logits = plain_step(entries, observer)
+        logits = plain_step(entries, *args, **kwargs)
         if runner.portion_graph_steps > before:
             mixed_replays += 1
             if any(e.from_slot for e in entries) and any(len(e.tokens) > 1 for e in entries):

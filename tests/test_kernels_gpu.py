@@ -963,3 +963,91 @@ def test_embed_takes_tokens_from_slots(K):
                   token_slots=dev([40, 41, 42], torch.int32))
     assert tokens.tolist() == [7, 42, 9, 40]
     np.testing.assert_allclose(host(out), np.stack([wte[t] + wpe[p] for t, p in zip([7, 42, 9, 40], [0, 3, 1, 15])]), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,n,k", [(8, 50257, 768), (1, 777, 240), (40, 1000, 96), (100, 409, 72), (256, 5000, 64), (33, 130, 1600)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_the_best_columns_of_a_product_give_the_argmax(K, dtype, rows, n, k, packed):
+    # the head of a greedy step: the product's sums are not written, only the best (sum, column) of each of its waves'
+    # columns; choosing among them must give numpy's argmax of the sums, ties to the smaller index
+    rng = np.random.default_rng(rows + n)
+    x, w = rng.standard_normal((rows, k)), rng.standard_normal((n, k)) / 8
+    w[n // 2] = w[3]            # equal columns, far apart: equal sums, whatever the order of a kernel's additions
+    w[n - 1] = w[3]
+    x[rows // 2] = w[3] * 50    # a row whose best columns are those three
+    xr, wr = (x.astype(np.float32).astype(np.float64), w.astype(np.float32).astype(np.float64)) if dtype == torch.float32 else (bf16_round(x), bf16_round(w))
+    ref = xr @ wr.T
+    values, indices = K.linear_best(dev(x, dtype), as_weight(K, w, dtype, packed))
+    per_row = K.best_per_row(rows, as_weight(K, w, dtype, packed), dtype)
+    assert values.shape == indices.shape == (rows, per_row) and per_row >= 1
+    v, i = host(values), indices.cpu().numpy()
+    # every column lies in exactly one wave's share, and each entry is the best of its share
+    real = i < n
+    assert (i[~real] == 0x7FFFFFFF).all() and np.isneginf(v[~real]).all()
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for r in range(rows):
+        np.testing.assert_allclose(v[r][real[r]], ref[r, i[r][real[r]]], rtol=tol, atol=tol * 4)
+    slots = np.arange(rows, dtype=np.int32)[::-1].copy()
+    last = torch.full((rows + 3,), -7, dtype=torch.int32, device=DEV)
+    tokens = K.choose(values, indices, dev(slots, torch.int32), last).cpu().numpy()
+    for r in range(rows):
+        assert ref[r, tokens[r]] >= ref[r].max() - tol * 4 * max(1.0, abs(ref[r]).max()), (r, tokens[r], ref[r].argmax())
+    assert tokens[rows // 2] == 3                                        # of the three equal columns the first
+    assert last.cpu().numpy()[:rows].tolist() == tokens[::-1].tolist() and (last.cpu().numpy()[rows:] == -7).all()
+    # the same tokens as the sampler's argmax over the logits the plain product writes
+    logits = K.linear(dev(x, dtype), as_weight(K, w, dtype, packed), out_dtype=torch.float32)
+    assert tokens.tolist() == K.sample(logits).cpu().numpy().tolist()
+
+
+def test_the_best_column_of_a_row_with_a_nan_is_the_first_nan(K):
+    x = np.ones((3, 64), dtype=np.float32)
+    w = np.random.default_rng(0).standard_normal((300, 64)).astype(np.float32)
+    w[170, 5] = np.nan
+    w[40, 9] = np.nan
+    values, indices = K.linear_best(dev(x), dev(w))
+    tokens = K.choose(values, indices, dev([0, 1, 2], torch.int32), torch.zeros(3, dtype=torch.int32, device=DEV))
+    assert tokens.cpu().tolist() == [40, 40, 40]
+
+
+def test_choose_moves_a_decode_batch_on_by_one_token(K):
+    # what the end of a captured decode step does besides choosing: positions, stored lengths, the cache row of the next
+    # token in every group (-1 where the table has no page yet), the token's source, a ring row in page-locked memory
+    rng = np.random.default_rng(5)
+    rows, width, page = 6, 5, 16
+    live = np.array([3, 0, -1, 2, 7, -1], dtype=np.int32)         # state slots; negative: padding
+    positions = np.array([15, 31, 0, 40, 79, 0], dtype=np.int32)  # the next ones: 16 (a new page), 32 (no page yet), 41, 80 (beyond the table)
+    tables = [rng.integers(0, 90, (rows, width)).astype(np.int32) for _ in range(2)]
+    tables[0][1, 2] = -1
+    tables[1][1, 2] = -1
+    indices = rng.integers(0, 1000, (rows, 1)).astype(np.int32)
+    d = lambda a: dev(a, torch.int32)
+    pos_d, ctx_d, src_d = d(positions), d(positions), d(np.full(rows, -1))
+    tab_d, slot_d = [d(t) for t in tables], [d(np.full(rows, -5)) for _ in tables]
+    last = torch.full((9,), -1, dtype=torch.int32, device=DEV)
+    ring = torch.full((3, 8), -9, dtype=torch.int32).pin_memory()
+    cursor = d([2])
+    advance = K.StepAdvance(pos_d, ctx_d, src_d, tab_d, slot_d, page)
+    for turn in range(2):
+        tokens = K.choose(None, d(indices), d(live), last, host_ring=ring, cursor=cursor, advance=advance)
+        torch.cuda.synchronize()
+        want = np.where(live >= 0, indices[:, 0], -1)
+        assert tokens.cpu().numpy().tolist() == want.tolist()
+        ring_row = (2 + turn) % 3
+        assert ring[ring_row, :rows].tolist() == want.tolist() and cursor.cpu().item() == (ring_row + 1) % 3
+        now = positions + (turn + 1) * (live >= 0)
+        assert pos_d.cpu().numpy().tolist() == now.tolist() and ctx_d.cpu().numpy().tolist() == now.tolist()
+        assert src_d.cpu().numpy().tolist() == np.where(live >= 0, live, -1).tolist()
+        for table, slots in zip(tables, slot_d):
+            expect = []
+            for r in range(rows):
+                block = now[r] // page
+                if live[r] < 0:
+                    expect.append(-5)
+                elif block >= width or table[r, block] < 0:
+                    expect.append(-1)
+                else:
+                    expect.append(int(table[r, block]) * page + now[r] % page)
+            assert slots.cpu().numpy().tolist() == expect
+    assert last.cpu().numpy().tolist() == [indices[1, 0], -1, indices[3, 0], indices[0, 0], -1, -1, -1, indices[4, 0], -1]
+    assert (ring[:, rows:] == -9).all()
