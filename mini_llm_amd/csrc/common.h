@@ -128,9 +128,8 @@ __device__ __forceinline__ bool beats(float value, int index, float best, int be
     return value > best;
 }
 
-// Where a product leaves, instead of its sums, the best of them per row: each wave of each block
-// writes the best (value, column) among its columns of a row to values/indices[row * per_row + block
-// along N * waves along N + wave]. Whoever picks the row's best among them gets the argmax of the
+// Where a product leaves, instead of its sums, the best of them per row: each block writes the best
+// (value, column) among its columns of a row to values/indices[row * per_row + block along N]. Whoever picks the row's best among them gets the argmax of the
 // row by the rules above, and the sums themselves need not be written (a greedy step's logits).
 struct BestOfColumns {
     float* values;

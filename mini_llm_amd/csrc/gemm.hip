@@ -249,15 +249,19 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 
     // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
     if constexpr (BEST) {
-        // Per row the best of this wave's columns: first among the lane's own (one per tile along N), then among the
-        // 32 lanes that hold the row (xor steps below 32 stay inside a half of the wave).
+        // Per row the best of this block's columns: first among the lane's own (one per tile along N), then among the
+        // 32 lanes that hold the row (xor steps below 32 stay inside a half of the wave), then among the waves that
+        // share the row, through LDS (the tiles' memory: every wave has left the loop behind the last barrier).
+        float* shared_values = reinterpret_cast<float*>(&a_tiles[0][0]);   // [WAVES_N][BM]
+        int* shared_indices = reinterpret_cast<int*>(&w_tiles[0][0]);
+        static_assert(sizeof(a_tiles) >= WAVES_N * BM * 4 && sizeof(w_tiles) >= WAVES_N * BM * 4, "room for the waves' best columns");
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int rows_from = m0 + wave_m * TM * 32 + i * 32 + 8 * (v / 4);  // the same for the whole wave
-                if (rows_from >= M) continue;
-                const int row = rows_from + 4 * half + (v % 4);
+                const int local_from = wave_m * TM * 32 + i * 32 + 8 * (v / 4);  // the same for the whole wave
+                if (m0 + local_from >= M) continue;
+                const int local_row = local_from + 4 * half + (v % 4);
                 float best = -INFINITY;
                 int best_index = 0x7fffffff;
 #pragma unroll
@@ -278,12 +282,25 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
                         best_index = other_index;
                     }
                 }
-                if (lane32 == 0 && row < M) {
-                    size_t at = (size_t)row * best_out.per_row + blockIdx.x * WAVES_N + wave_n;
-                    best_out.values[at] = best;
-                    best_out.indices[at] = best_index;
+                if (lane32 == 0) {
+                    shared_values[wave_n * BM + local_row] = best;
+                    shared_indices[wave_n * BM + local_row] = best_index;
                 }
             }
+        }
+        __syncthreads();
+        for (int local_row = tid; local_row < BM && m0 + local_row < M; local_row += THREADS) {
+            float best = shared_values[local_row];
+            int best_index = shared_indices[local_row];
+#pragma unroll
+            for (int w = 1; w < WAVES_N; w++)
+                if (beats(shared_values[w * BM + local_row], shared_indices[w * BM + local_row], best, best_index)) {
+                    best = shared_values[w * BM + local_row];
+                    best_index = shared_indices[w * BM + local_row];
+                }
+            size_t at = (size_t)(m0 + local_row) * best_out.per_row + blockIdx.x;
+            best_out.values[at] = best;
+            best_out.indices[at] = best_index;
         }
         return;
     }
@@ -656,11 +673,11 @@ MLLM_API int mllm_gemm(const void* A, const void* W, int w_packed, const float* 
 // The tile a product of M rows takes when it leaves the best of its columns instead of its sums
 // (mllm_gemm_best): the tiles the plain product takes for a wide matrix at these row counts.
 namespace {
-struct BestTile { int bm, bn, waves_n; };
+struct BestTile { int bm, bn; };
 BestTile best_tile(int M) {
-    if (M <= 32) return {32, 128, 4};
-    if (M <= 64) return {64, 64, 2};
-    return {128, 64, 2};
+    if (M <= 32) return {32, 128};
+    if (M <= 64) return {64, 64};
+    return {128, 64};
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
@@ -686,11 +703,10 @@ void launch_best_of(const void* A, const void* W, bool packed, const float* bias
 MLLM_API int mllm_gemm_best_per_row(int M, int N, int K, int in_dtype) {
     if (M <= 0 || N <= 0 || K <= 0 || (in_dtype != MLLM_F32 && in_dtype != MLLM_BF16)) return 0;
     if (K % (in_dtype == MLLM_F32 ? 4 : 8)) return 0;
-    BestTile tile = best_tile(M);
-    return ceil_div(N, tile.bn) * tile.waves_n;
+    return ceil_div(N, best_tile(M).bn);
 }
 
-// A . W^T (+ bias) whose sums are not written: per row, every wave of every block leaves the best
+// A . W^T (+ bias) whose sums are not written: per row, every block leaves the best
 // (sum, column) of its columns in values / indices [M, per_row] (per_row as mllm_gemm_best_per_row
 // says; every entry is written, an entry without a column holds -inf and the largest index). The
 // best entry of a row by numpy's argmax rules is the row's argmax: the head of a greedy step,

@@ -178,7 +178,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 // follows the step). With `advance` the row's position and stored length grow by one, its cache row
 // of every group is looked up in the block table for the new position (-1 where the table has no page
 // there yet: the host brings the table before that step runs), and its token source becomes its own
-// slot. One block; wave w picks the rows w, w + waves, ...
+// slot. One block.
 struct StepGroups {
     const int* tables[4];
     int* slots[4];
@@ -194,22 +194,37 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
     int advance, int* __restrict__ positions, int* __restrict__ context_lens, int* __restrict__ token_sources,
     StepGroups groups) {
     extern __shared__ int chosen[];  // [n_rows]
-    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
-    const int ring_row = cursor ? *cursor : 0;
-    for (int row = wave; row < n_rows; row += CHOOSE_THREADS / WAVE) {
+    const int tid = threadIdx.x;
+    const int ring_row = cursor ? cursor[0] : 0;
+    const int sequence = cursor ? cursor[1] : 0;
+    // A row's candidates are shared among the `group` lanes next to each other that take the row (a whole wave for
+    // few rows, down to four lanes for hundreds), and asked for eight at a time before any is compared: a candidate
+    // was written by some other compute unit and comes from memory.
+    int group = WAVE;
+    while (group > 4 && (CHOOSE_THREADS / group) < n_rows) group >>= 1;
+    const int in_group = tid % group, groups_in_block = CHOOSE_THREADS / group;
+    constexpr int BATCH = 8;
+    for (int row = tid / group; row < n_rows; row += groups_in_block) {
         float best = -INFINITY;
         int best_index = 0x7fffffff;
-        for (int c = lane; c < per_row; c += WAVE) {
-            size_t at = (size_t)row * per_row + c;
-            float value = values ? values[at] : 0.0f;
-            int index = indices[at];
-            if (beats(value, index, best, best_index)) {
-                best = value;
-                best_index = index;
-            }
-        }
+        const size_t base = (size_t)row * per_row;
+        for (int c0 = in_group; c0 < per_row; c0 += group * BATCH) {
+            float value[BATCH];
+            int index[BATCH];
 #pragma unroll
-        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
+            for (int u = 0; u < BATCH; u++) {
+                int c = min(c0 + u * group, per_row - 1);
+                value[u] = values ? values[base + c] : 0.0f;
+                index[u] = indices[base + c];
+            }
+#pragma unroll
+            for (int u = 0; u < BATCH; u++)
+                if (c0 + u * group < per_row && beats(value[u], index[u], best, best_index)) {
+                    best = value[u];
+                    best_index = index[u];
+                }
+        }
+        for (int offset = group / 2; offset > 0; offset >>= 1) {
             float other = __shfl_xor(best, offset, WAVE);
             int other_index = __shfl_xor(best_index, offset, WAVE);
             if (beats(other, other_index, best, best_index)) {
@@ -217,7 +232,7 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
                 best_index = other_index;
             }
         }
-        if (lane == 0) chosen[row] = best_index;
+        if (in_group == 0) chosen[row] = best_index;
     }
     __syncthreads();
     for (int row = tid; row < n_rows; row += CHOOSE_THREADS) {
@@ -225,7 +240,10 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
         const bool live = slot >= 0;
         const int token = live ? chosen[row] : -1;
         out_tokens[row] = token;
-        if (host_ring) host_ring[(size_t)ring_row * ring_stride + row] = token;
+        if (host_ring) {
+            host_ring[(size_t)ring_row * ring_stride + row] = token;
+            __threadfence_system();   // the token is in host memory before the row's number (below) can be
+        }
         if (!live) continue;
         token_slots[slot] = token;
         if (advance) {
@@ -240,7 +258,16 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
             }
         }
     }
-    if (cursor && tid == 0) *cursor = (ring_row + 1) % ring_rows;  // every thread has read it before the barrier above
+    if (cursor) {
+        // The row's last entry says which step's tokens the row holds: whoever reads the ring on the host waits for
+        // that number instead of an event behind the step (which costs the device about 6 us between two steps).
+        __syncthreads();
+        if (tid == 0) {
+            host_ring[(size_t)ring_row * ring_stride + ring_stride - 1] = sequence;
+            cursor[0] = (ring_row + 1) % ring_rows;   // every thread has read both before the first barrier
+            cursor[1] = (sequence + 1) & 0x3fffffff;
+        }
+    }
 }
 
 }  // namespace
@@ -266,7 +293,7 @@ MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, i
                          int page_size, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_rows <= 8192 && per_row >= 1, "choose: bad sizes rows=%d candidates=%d", n_rows, per_row);
     MLLM_REQUIRE(indices && state_slots && token_slots && out_tokens, "choose: an operand is missing");
-    MLLM_REQUIRE(!host_ring || (ring_rows >= 1 && ring_stride >= n_rows), "choose: the ring's rows are shorter than the batch");
+    MLLM_REQUIRE(!host_ring || (ring_rows >= 1 && ring_stride >= n_rows + (cursor ? 1 : 0)), "choose: the ring's rows are shorter than the batch (and, with a cursor, one entry for the step's number)");
     MLLM_REQUIRE(!cursor || host_ring, "choose: a cursor without a ring");
     StepGroups groups{};
     if (advance) {

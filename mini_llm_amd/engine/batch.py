@@ -275,7 +275,7 @@ class DecodeBatchBuilder:
         lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
         for _ in range(n_groups):
             lengths += [capacity * self.table_width, capacity]
-        lengths.append(1)   # the row of the token ring that a step which chooses its tokens on the device writes next
+        lengths.append(2)   # for a step that chooses its tokens on the device: the row of the token ring it writes next, and its number
         self.offsets, total = [], 0
         for n in lengths:
             self.offsets.append(total)
@@ -338,4 +338,4 @@ class DecodeBatchBuilder:
 
     def cursor_view(self, device_flat):
         at = self.offsets[8 + 2 * len(self.tables)]
-        return device_flat[at : at + 1]
+        return device_flat[at : at + 2]

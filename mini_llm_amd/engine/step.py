@@ -17,6 +17,7 @@ small model the host needs longer to launch the kernels than the GPU to run them
 from __future__ import annotations
 
 import gc
+import time
 from array import array as _array
 from collections import OrderedDict
 
@@ -48,20 +49,39 @@ TOKEN_RING_ROWS = 8   # steps whose chosen tokens stay readable on the host afte
 
 class ChosenTokens:
     """The tokens a step chose on the device: ``device`` (int32, one per wanted row, valid until the next step) and, on
-    the host, a row of page-locked memory that is complete once ``event`` has passed (``tolist`` waits for it). A row
-    is used again ``TOKEN_RING_ROWS`` steps later."""
+    the host, a row of page-locked memory. The row is complete once ``event`` has passed or, where the step's last
+    kernel writes the row itself, once the row's last entry shows the step's ``number`` (``tolist`` waits for either).
+    A row is used again ``TOKEN_RING_ROWS`` steps later."""
 
-    __slots__ = ("device", "_host", "_n", "_event")
+    __slots__ = ("device", "_host", "_n", "_event", "_number")
+    WAIT_SECONDS = 30.0
 
-    def __init__(self, device, host, n, event):
-        self.device, self._host, self._n, self._event = device, host, n, event
+    def __init__(self, device, host, n, event=None, number=None):
+        self.device, self._host, self._n, self._event, self._number = device, host, n, event, number
 
     def __len__(self):
         return self._n
 
     def tolist(self) -> list:
-        self._event.synchronize()
+        if self._event is not None:
+            self._event.synchronize()
+        else:
+            self._await_number()
         return self._host[: self._n].tolist()
+
+    def _await_number(self) -> None:
+        """Spins on the row's last entry (written by the device behind the tokens, with a fence between); gives the
+        processor away between looks once the first few thousand have found nothing."""
+        row, number = self._host, self._number
+        looks, deadline = 0, None
+        while row[-1] != number:
+            looks += 1
+            if looks > 2000:
+                time.sleep(0)
+                if deadline is None:
+                    deadline = time.monotonic() + self.WAIT_SECONDS
+                elif time.monotonic() > deadline:
+                    raise RuntimeError(f"the tokens of step {number} have not arrived after {self.WAIT_SECONDS:.0f} s (the row shows step {int(row[-1])})")
 
 
 class _DecodeGraph:
@@ -80,8 +100,10 @@ class _DecodeGraph:
         self.graph = None
         self.logits = None
         if chooses:
-            self.ring = torch.full((TOKEN_RING_ROWS, capacity), -1, dtype=torch.int32).pin_memory()
-            self.ring_at = 0        # the ring row the next step writes: the host's count of the device's cursor
+            self.ring = torch.full((TOKEN_RING_ROWS, capacity + 1), -1, dtype=torch.int32).pin_memory()
+            self.ring_rows = self.ring.numpy()   # the same memory, for the host's reads
+            self.ring_at = 0        # the ring row the next step writes and that step's number: the host's count of the
+            self.number = 0         # device's cursor
             self.on_device = None   # per row (request's cache entry, its table_changes, its length) that the device's batch stands at
             self.uploads = 0
 
@@ -112,7 +134,7 @@ class _DecodeGraph:
                       and all(r is at[0] and r.table_changes == at[1] and r.length == at[2] for r, at in zip(records, stands)))
         if not carried_on:
             flat = self.builder.fill(entries)
-            self.builder.cursor[0] = self.ring_at
+            self.builder.cursor[:] = (self.ring_at, self.number)
             runner.staging.upload(flat, into=self.buffer)
             self.uploads += 1
         batch = self.static_batch
@@ -121,12 +143,11 @@ class _DecodeGraph:
             choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True)
             self.graph, self.logits = _capture(runner, batch, choice)
         self.graph.replay()
-        row = self.ring[self.ring_at]
+        chosen = ChosenTokens(self.logits[: len(entries)], self.ring_rows[self.ring_at], len(entries), number=self.number)
         self.ring_at = (self.ring_at + 1) % TOKEN_RING_ROWS
+        self.number = (self.number + 1) & 0x3FFFFFFF
         self.on_device = [(r, r.table_changes, r.length + 1) for r in records]
-        event = torch.cuda.Event()
-        event.record()
-        return batch, ChosenTokens(self.logits[: len(entries)], row, len(entries), event)
+        return batch, chosen
 
 
 def _capture(runner, batch, choice=None):
@@ -398,4 +419,4 @@ class ModelRunner:
         row[:n].copy_(tokens[:n], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        return ChosenTokens(tokens, row, n, event)
+        return ChosenTokens(tokens, row.numpy(), n, event=event)

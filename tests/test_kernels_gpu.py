@@ -1026,7 +1026,7 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
     tab_d, slot_d = [d(t) for t in tables], [d(np.full(rows, -5)) for _ in tables]
     last = torch.full((9,), -1, dtype=torch.int32, device=DEV)
     ring = torch.full((3, 8), -9, dtype=torch.int32).pin_memory()
-    cursor = d([2])
+    cursor = d([2, 41])
     advance = K.StepAdvance(pos_d, ctx_d, src_d, tab_d, slot_d, page)
     for turn in range(2):
         tokens = K.choose(None, d(indices), d(live), last, host_ring=ring, cursor=cursor, advance=advance)
@@ -1034,7 +1034,8 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
         want = np.where(live >= 0, indices[:, 0], -1)
         assert tokens.cpu().numpy().tolist() == want.tolist()
         ring_row = (2 + turn) % 3
-        assert ring[ring_row, :rows].tolist() == want.tolist() and cursor.cpu().item() == (ring_row + 1) % 3
+        assert ring[ring_row, :rows].tolist() == want.tolist() and cursor.cpu().tolist() == [(ring_row + 1) % 3, 42 + turn]
+        assert ring[ring_row, 7].item() == 41 + turn          # the step's number, behind its tokens
         now = positions + (turn + 1) * (live >= 0)
         assert pos_d.cpu().numpy().tolist() == now.tolist() and ctx_d.cpu().numpy().tolist() == now.tolist()
         assert src_d.cpu().numpy().tolist() == np.where(live >= 0, live, -1).tolist()
@@ -1050,4 +1051,4 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
                     expect.append(int(table[r, block]) * page + now[r] % page)
             assert slots.cpu().numpy().tolist() == expect
     assert last.cpu().numpy().tolist() == [indices[1, 0], -1, indices[3, 0], indices[0, 0], -1, -1, -1, indices[4, 0], -1]
-    assert (ring[:, rows:] == -9).all()
+    assert (ring[:, rows:7] == -9).all() and ring[1, 7].item() == -9
