@@ -446,6 +446,7 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--lanes-from", type=int, default=None, help="decode steps of at least so many sequences run two halves side by side (0: never; default: the engine's)")
     parser.add_argument("--shape", default="small", choices=("small", "medium", "xl"), help="the GPT-2 shape that is run (the headline is small)")
     parser.add_argument("--prompt-len", "--prompt-tokens", dest="prompt_len", type=int, default=PROMPT_LEN,
                         help="tokens of each sequence's prompt before decoding is timed (--prompt-tokens is the reference's name: engine/bench/bench_options.c:25-94)")
@@ -491,7 +492,7 @@ def main() -> int:
         if not tensors:
             tensors.update(random_tensors(model, seed))
         bind_tensors(model, tensors, require_gpu())
-        return Engine(options=EngineOptions(dtype=dtype, max_sessions=largest, max_tokens=largest * CONTEXT), model=model)
+        return Engine(options=EngineOptions(dtype=dtype, max_sessions=largest, max_tokens=largest * CONTEXT, decode_lanes_from=args.lanes_from), model=model)
 
     def host_weights():
         return {name: tensor.numpy() for name, tensor in tensors.items()}

@@ -71,6 +71,23 @@ class StepBatch:
     request_ids: list = field(default_factory=list)
     host: dict = field(default_factory=dict)   # the same arrays as numpy, for parts that plan on the host
 
+    def rows_of_requests(self, lo: int, hi: int) -> "StepBatch":
+        """Requests lo..hi-1 of a batch in which every request brings one token (a decode step) as a batch of their own,
+        over the same device memory: row r of it is row lo + r of this one. The block tables stay whole (a row's
+        ``token_request`` still names its line there)."""
+        if self.max_q_len != 1 or self.n_requests != self.n_tokens or not 0 <= lo < hi <= self.n_tokens:
+            raise ValueError("only a batch of single tokens can be cut between requests")
+        n = hi - lo
+        cut = lambda t: t[lo:hi]
+        return StepBatch(
+            n_tokens=n, n_requests=n, n_logit_rows=n, max_q_len=1, short_requests=n, short_rows=n, short_portion=self.short_portion,
+            max_total_len=self.max_total_len, tokens=cut(self.tokens), positions=cut(self.positions), token_request=cut(self.token_request),
+            q_starts=self.q_starts[lo : hi + 1], context_lens=cut(self.context_lens), state_slots=cut(self.state_slots),
+            logit_rows=cut(self.logit_rows), token_sources=cut(self.token_sources), logit_slots=cut(self.logit_slots),
+            groups=[GroupStepData(block_tables=g.block_tables, slots=cut(g.slots)) for g in self.groups],
+            request_ids=self.request_ids[lo:hi], host={},
+        )
+
     def rows_in_order_of(self, request_ids) -> list:
         """The batch's rows, listed request by request in the given order of the requests (the
         batch itself may lay the requests out in another order)."""

@@ -34,6 +34,7 @@ class EngineOptions:
     max_tokens_per_step: int = 2048      # token budget of one scheduler step
     use_graphs: bool = True              # replay decode steps from captured HIP graphs
     portion_graph_after: int | None = None   # a shape of batch with prompt portions is captured when it comes this often (None: the step function's default; 0: never)
+    decode_lanes_from: int | None = None     # captured decode steps of at least so many requests run two halves of them side by side (None: the step function's default; 0: never)
     step_ahead: bool = True              # the scheduler launches a step before it has read the one before
     device: str = "cuda:0"
 
@@ -179,7 +180,8 @@ class Engine:
             raise ValueError("this model has no position limit of its own: give max_length, the longest sequence a request may reach")
         self.cache = make_cache(self.model, max_tokens=max_tokens, page_size=options.page_size,
                                 max_requests=options.max_sessions, device=options.device, max_length=limit)
-        self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs, portion_graph_after=options.portion_graph_after)
+        self.runner = ModelRunner(self.model, self.cache, options.device, use_graphs=options.use_graphs, portion_graph_after=options.portion_graph_after,
+                                  lanes_from=options.decode_lanes_from)
         self.sampler = Sampler(self.runner.staging)
         self.scheduler = Scheduler(_Executor(self), max_batch=options.max_sessions, max_tokens_per_step=options.max_tokens_per_step,
                                    step_ahead=options.step_ahead)

@@ -44,6 +44,11 @@ class StepError(ValueError):
     """The batch cannot be run; nothing has been changed."""
 
 
+# A decode step of many requests is one kernel bound by memory (attention over the cache) among six that wait for trips
+# to memory with most compute units idle. From so many requests on the captured step runs two halves of the requests
+# side by side (graph branches), so that one half's small kernels run under the other half's attention.
+DECODE_LANES_FROM = 32
+DECODE_LANE_ROWS = 64    # the most requests of a group (the kernels for few rows take up to 64)
 TOKEN_RING_ROWS = 8   # steps whose chosen tokens stay readable on the host after they were launched
 
 
@@ -84,6 +89,44 @@ class ChosenTokens:
                     raise RuntimeError(f"the tokens of step {number} have not arrived after {self.WAIT_SECONDS:.0f} s (the row shows step {int(row[-1])})")
 
 
+class _Lanes:
+    """Streams side by side, for a step whose requests run their layers in groups (Model._layers_in_lanes): the first
+    group stays on the stream the step runs on, every other gets a stream of its own, which waits for that stream at
+    the fork and is waited for at the join. Inside a capture this gives the graph branches that the device runs at
+    the same time. All streams have the default priority."""
+
+    def __init__(self, device, parts: int = 2):
+        import torch
+
+        self.parts = parts
+        self._streams = [torch.cuda.Stream(device=device) for _ in range(parts - 1)]
+        self._main = None
+
+    def cuts(self, rows: int) -> list:
+        """Where the rows are cut: equal groups, in whole sixteens while there are that many rows."""
+        unit = 16 if rows >= 16 * self.parts else 1
+        per = -(-rows // (self.parts * unit)) * unit
+        return [(lo, min(rows, lo + per)) for lo in range(0, rows, per)]
+
+    def fork(self) -> None:
+        import torch
+
+        self._main = torch.cuda.current_stream()
+        for stream in self._streams:
+            stream.wait_stream(self._main)
+
+    def lane(self, index: int):
+        import contextlib
+
+        import torch
+
+        return contextlib.nullcontext() if index == 0 else torch.cuda.stream(self._streams[index - 1])
+
+    def join(self) -> None:
+        for stream in self._streams:
+            self._main.wait_stream(stream)
+
+
 class _DecodeGraph:
     """One captured decode step for up to ``capacity`` requests. ``chooses``: the captured step ends with the greedy
     choice of its tokens (models.TokenChoice) and moves its batch on by one token on the device, so that the next step
@@ -99,6 +142,8 @@ class _DecodeGraph:
         self.static_batch = self.builder.batch(self.buffer, [])
         self.graph = None
         self.logits = None
+        # from so many rows on the requests go through the layers in two groups side by side
+        self.lanes = _Lanes(runner.device, max(2, capacity // DECODE_LANE_ROWS)) if runner.lanes_from and capacity >= runner.lanes_from else None
         if chooses:
             self.ring = torch.full((TOKEN_RING_ROWS, capacity + 1), -1, dtype=torch.int32).pin_memory()
             self.ring_rows = self.ring.numpy()   # the same memory, for the host's reads
@@ -115,7 +160,7 @@ class _DecodeGraph:
         batch = self.static_batch
         batch.request_ids = [e.request_id for e in entries]
         if self.graph is None:
-            self.graph, self.logits = _capture(runner, batch)
+            self.graph, self.logits = _capture(runner, batch, lanes=self.lanes)
         self.graph.replay()
         return batch, self.logits[: len(entries)]
 
@@ -141,7 +186,7 @@ class _DecodeGraph:
         batch.request_ids = [e.request_id for e in entries]
         if self.graph is None:
             choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True)
-            self.graph, self.logits = _capture(runner, batch, choice)
+            self.graph, self.logits = _capture(runner, batch, choice, self.lanes)
         self.graph.replay()
         chosen = ChosenTokens(self.logits[: len(entries)], self.ring_rows[self.ring_at], len(entries), number=self.number)
         self.ring_at = (self.ring_at + 1) % TOKEN_RING_ROWS
@@ -150,14 +195,17 @@ class _DecodeGraph:
         return batch, chosen
 
 
-def _capture(runner, batch, choice=None):
+def _capture(runner, batch, choice=None, lanes=None):
     """Runs the batch once eagerly (on a side stream, as capture needs), then captures the same. With ``choice`` the
     captured step ends with the choice of its tokens; the eager run then chooses into memory of its own and moves
     nothing on, so that the first replay finds everything as the eager run found it."""
     import torch
 
-    warm = {}
+    warm, extra = {}, {}
+    if lanes is not None:
+        warm["lanes"] = extra["lanes"] = lanes
     if choice is not None:
+        extra["choice"] = choice
         from dataclasses import replace
 
         warm["choice"] = replace(choice, token_slots=torch.empty_like(choice.token_slots), host_ring=None, cursor=None, advance=False)
@@ -176,7 +224,7 @@ def _capture(runner, batch, choice=None):
     gc.disable()
     try:
         with torch.cuda.graph(graph):
-            logits = runner.forward(batch) if choice is None else runner.forward(batch, choice=choice)
+            logits = runner.forward(batch, **extra)
     finally:
         if collecting:
             gc.enable()
@@ -214,9 +262,12 @@ class _PortionGraph:
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, device, use_graphs: bool = True, portion_graph_after: int | None = None):
+    def __init__(self, model, cache: CacheManager, device, use_graphs: bool = True, portion_graph_after: int | None = None,
+                 lanes_from: int | None = None):
         """``portion_graph_after``: the time a shape of batch with portions of prompts has to come to be captured (None: the
-        default, PORTION_GRAPH_AFTER; 0: never)."""
+        default, PORTION_GRAPH_AFTER; 0: never). ``lanes_from``: captured decode steps for at least so many requests run
+        their layers in two groups side by side (None: the default, DECODE_LANES_FROM; 0: never)."""
+        self.lanes_from = DECODE_LANES_FROM if lanes_from is None else int(lanes_from)
         self.model, self.cache, self.device = model, cache, device
         self.staging = BatchStaging(device) if device is not None else None
         self.steps_run = 0
@@ -296,13 +347,15 @@ class ModelRunner:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {entry.request_id!r}: wanted place {w} is not among its {n} tokens")
 
-    def forward(self, batch, resolve: bool = True, observer=None, choice=None):
+    def forward(self, batch, resolve: bool = True, observer=None, choice=None, lanes=None):
         """Tokens that come from last-token slots are fetched on the device, then the model runs."""
         extra = {}
         if observer is not None:
             extra["observer"] = observer
         if choice is not None:
             extra["choice"] = choice
+        if lanes is not None:
+            extra["lanes"] = lanes
         return self.model.forward(batch, self.cache, resolve_tokens=resolve, **extra)
 
     def _graph_for(self, entries, choose: bool = False):

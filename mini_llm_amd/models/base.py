@@ -120,11 +120,50 @@ class Model(Part):
                 out[call.cache] = need
         return out
 
-    def forward(self, batch, cache, resolve_tokens: bool = False, observer=None, choice: TokenChoice | None = None):
+    def _layers(self, hidden, batch, cache, observer=None):
+        """The schedule over the rows of ``batch``; the stream comes back as the last layer leaves it."""
+        for index, call in enumerate(self.schedule):
+            block = self.blocks[call.block]
+            if not block.takes_pending:
+                hidden = kernels.settle(hidden)
+            hidden = block.forward(hidden, cache.layer_context(batch, call))
+            if observer is not None:
+                observer(index, kernels.settle(hidden))
+        return hidden
+
+    def _layers_in_lanes(self, hidden, batch, cache, lanes):
+        """A decode step's requests in ``lanes.parts`` groups of neighbouring rows, each group through all layers and the
+        final norm on a lane (a stream) of its own: nothing in a layer connects two requests, and while one group's
+        attention reads its keys and values (bound by memory) the other's products, which wait for one trip to memory
+        after the other, find the compute units free. Returns the normalised rows of all groups, [rows, width], for the
+        head, which reads its matrix once for all of them."""
+        import torch
+
+        rows = batch.n_tokens
+        normed = torch.empty((rows, hidden.shape[1]), dtype=self.precision.compute, device=hidden.device)
+        hidden = kernels.settle(hidden)
+        cuts = lanes.cuts(rows)
+        lanes.fork()
+        kept = []   # what one lane made stays alive until all have joined: its memory must not go to another lane meanwhile
+        for lane, (lo, hi) in enumerate(cuts):
+            with lanes.lane(lane):
+                part = batch.rows_of_requests(lo, hi)
+                out = self._layers(hidden[lo:hi], part, cache)
+                if not self.final_norm.takes_pending:
+                    out = kernels.settle(out)
+                self.final_norm.forward_into(out, normed[lo:hi])
+                kept.append((part, out))
+        lanes.join()
+        del kept
+        return normed
+
+    def forward(self, batch, cache, resolve_tokens: bool = False, observer=None, choice: TokenChoice | None = None, lanes=None):
         """The whole step: embeds the batch's tokens, runs the schedule over the cache, and
         returns float32 logits [len(batch.logit_rows), vocab] at the wanted rows only (with
         ``choice``: the greedy token of each wanted row instead, int32 on the device). With
         ``resolve_tokens`` the rows that name a last-token slot take their token from it.
+        ``lanes`` (fork(), lane(i), join(), cuts(rows)): a step of single tokens runs its layers in groups of requests
+        side by side (``_layers_in_lanes``).
         ``observer(name, rows)``, if given, is shown the residual stream (float32 [tokens, width],
         rows in the batch's order) after the embedding (name "embedding") and after each entry of
         the schedule (its index): what the reference's block_outputs are for, finding the layer
@@ -134,19 +173,16 @@ class Model(Part):
                                         token_slots=cache.last_token if resolve_tokens else None)
         if observer is not None:
             observer("embedding", kernels.settle(hidden))
-        for index, call in enumerate(self.schedule):
-            block = self.blocks[call.block]
-            if not block.takes_pending:
+        if lanes is not None:
+            normed = self._layers_in_lanes(hidden, batch, cache, lanes)
+        else:
+            hidden = self._layers(hidden, batch, cache, observer)
+            if batch.n_logit_rows == 0:
+                return None
+            if not self.final_norm.takes_pending:
                 hidden = kernels.settle(hidden)
-            hidden = block.forward(hidden, cache.layer_context(batch, call))
-            if observer is not None:
-                observer(index, kernels.settle(hidden))
-        if batch.n_logit_rows == 0:
-            return None
-        if not self.final_norm.takes_pending:
-            hidden = kernels.settle(hidden)
-        # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
-        normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
+            # the final norm runs on the wanted rows only (engine/src/gpt2_gpu.cu:254-258)
+            normed = self.final_norm.forward(hidden, self.precision.compute, row_index=batch.logit_rows)
         if choice is None:
             return self.head.forward(normed)
         # Greedy tokens on the device. A head that can leave the best of its columns instead of all of them does (the

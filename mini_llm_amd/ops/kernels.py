@@ -286,15 +286,18 @@ def linear_split(x, weight, k_blocks: int):
     return partials
 
 
-def convert(src, dtype, transpose=False):
-    """A 1-D or 2-D float32/bfloat16 tensor in another element type, a 2-D one transposed on request
-    (contiguous result). Load-time work on weights."""
+def convert(src, dtype, transpose=False, out=None):
+    """A 1-D or 2-D float32/bfloat16 tensor in another element type (or the same: a copy), a 2-D one
+    transposed on request (contiguous result, written into ``out`` if one is given). Load-time work on weights."""
     _device_tensor(src, "src")
     _require(src.dim() in (1, 2), "convert takes vectors and matrices")
     rows, cols = (1, src.shape[0]) if src.dim() == 1 else src.shape
     _require(not transpose or src.dim() == 2, "only a matrix can be transposed")
     shape = src.shape if not transpose else (cols, rows)
-    out = torch.empty(tuple(shape), dtype=dtype, device=src.device)
+    if out is None:
+        out = torch.empty(tuple(shape), dtype=dtype, device=src.device)
+    _device_tensor(out, "out", dtype)
+    _require(tuple(out.shape) == tuple(shape), "out has the wrong shape")
     check(library().mllm_convert(_ptr(src), _ptr(out), rows, cols, _code(src.dtype), _code(dtype), int(bool(transpose)), _stream()))
     return out
 

@@ -90,6 +90,14 @@ class Norm(Part):
         """x: [rows, width] float32 -> [rows or len(row_index), width] of out_dtype."""
         raise NotImplementedError
 
+    def forward_into(self, x, out):
+        """The normalised rows of x written into ``out`` ([rows, width], its element type the one asked for): for a
+        caller that gathers the rows of several calls in one tensor. A norm whose kernel can write where it is told
+        overrides this; the default copies."""
+        from ..ops import kernels
+
+        return kernels.convert(self.forward(x, out.dtype), out.dtype, out=out)
+
     def forward_with_sums(self, hidden, out_dtype, packed=False):
         """hidden: float32 rows, or rows whose last sums are pending -> (the normalised rows, the
         rows with their sums taken: what the residual stream goes on with). A norm that can take

@@ -25,6 +25,9 @@ class LayerNorm(Norm):
     def forward(self, x, out_dtype, row_index=None):
         return kernels.layernorm(x, self.weight, self.bias, self.eps, out_dtype=out_dtype, row_index=row_index)
 
+    def forward_into(self, x, out):
+        return kernels.layernorm(x, self.weight, self.bias, self.eps, out_dtype=out.dtype, out=out)
+
     def forward_with_sums(self, hidden, out_dtype, packed=False):
         return kernels.layernorm(hidden, self.weight, self.bias, self.eps, out_dtype=out_dtype, with_sums=True, packed_out=packed)
 

@@ -506,6 +506,47 @@ def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_queued_decoding_of_many_sequences_side_by_side_without_copies(model_dirs, dtype):
+    # 40 sequences decode for 70 steps, queued: the captured step chooses its tokens itself and moves its batch on by
+    # one token on the device, so between two steps nothing is copied to the device unless a sequence has reached a new
+    # page (all prompts have the same length here: every 16th step); from 32 rows on the step's requests go through the
+    # layers in two groups side by side. The tokens must be the plain implementation's.
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+
+    folder, config, weights = model_dirs["A"]
+    engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=40, page_size=16))
+    prompts = [random_tokens(900 + i, 21, config["vocab_size"]) for i in range(40)]
+    handles = [engine.try_take_cache() for _ in prompts]
+    got = [[engine.prefill_greedy(h, p)] for h, p in zip(handles, prompts)]
+    steps = 70
+    engine.decode_batch_enqueue(handles)
+    for _ in range(steps - 1):
+        engine.decode_batch_enqueue(handles)
+        for g, t in zip(got, engine.take()):
+            g.append(t)
+    for g, t in zip(got, engine.take()):
+        g.append(t)
+    graph = engine.runner._graphs[64, True]
+    assert graph.lanes is not None and len(graph.lanes.cuts(64)) == 2
+    assert engine.runner.graph_steps == steps and graph.uploads <= 2 + steps // 16, graph.uploads
+    rounded = plain_gpt2.bf16_weights(weights) if dtype == "bfloat16" else None
+    for i in range(0, 40, 3):
+        if dtype == "float32":
+            assert got[i] == plain_gpt2.greedy(config, weights, prompts[i], steps + 1), i
+        else:
+            plain_check_greedy(config, rounded, prompts[i], got[i], margin=0.03, stored=plain_gpt2.stored_as_bf16)
+    # a sequence leaves and the rest go on: the device's batch no longer stands for them, so it is brought anew
+    engine.release_cache(handles[0])
+    before = graph.uploads
+    engine.decode_batch_enqueue(handles[1:])
+    tokens = engine.take()
+    assert graph.uploads == before + 1 and len(tokens) == 39
+    if dtype == "float32":
+        assert tokens[2] == plain_gpt2.greedy(config, weights, prompts[3], steps + 2)[-1]
+    engine.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_step_ahead_gives_the_tokens_of_step_by_step(model_dirs, engines, dtype):
     # nine requests in a pool that holds about three of them (requests wait, and some are preempted
     # and recomputed), prompts in portions of 24 tokens beside decodes, an end token for every
