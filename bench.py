@@ -155,130 +155,164 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4), "from_graph": engine.runner.portion_graph_steps - replayed_before >= runs}
 
 
-def measure_kernels(engine, batch: int = 8, context: int = 768, reps: int = 7):
-    """What the kernels that a step's time goes to reach of their own roofline, each timed alone
-    between two events over all layers' weights in turn (as a step walks them), median of ``reps``:
-    for a 2,048-token prompt step the four products of a layer and the prompt attention (flops /
-    time / the matrix cores' peak), for a decode step of ``batch`` sequences at ``context`` tokens the
-    two halves of a layer and the head (the bytes each has to read / time / the memory's peak); a time
-    holds the gap to the next kernel, as in a step. The
-    reference prices its kernels the same way, against a pure read of the same bytes
-    (docs/kernels/010_matvec_batch.md:20,108-117)."""
+def kernel_times_inside_a_step(engine, make_entries, choose: bool, reps: int = 5):
+    """(names, microseconds): the kernels of one real step of the engine, in order, and what each takes INSIDE the step.
+
+    The step goes through the engine's own step function and is captured as generation captures it. It is captured once
+    for every n with only its first n kernels really launched (ops.library.first_launches), and the replay of each such
+    graph is timed: kernel n's time is the difference between two of them. So a time holds what the kernel costs where it
+    stands: its start behind the kernel before it, and its first trip to memory for what that one wrote. (The first
+    kernel's figure also holds what a replay costs by itself.) ``make_entries()`` opens the step's requests and returns
+    (entries, handles); they are given back after each capture."""
     import numpy as np
     import torch
 
-    from mini_llm_amd.engine import StepEntry
-    from mini_llm_amd.engine.batch import build_step_batch
-    from mini_llm_amd.ops import kernels
+    from mini_llm_amd.engine.step import ModelRunner
+    from mini_llm_amd.ops.library import first_launches
 
-    model, cache, runner = engine.model, engine.cache, engine.runner
-    config, dtype = engine.config, engine.options.dtype
-    e = element_size(dtype)
-    compute = model.precision.compute
-    d, ff, n_layer, vocab = config.n_embd, config.n_inner, config.n_layer, config.vocab_size
-    rng = np.random.default_rng(SEED + 4)
-    calls = [(model.blocks[call.block], cache.layer_context, call) for call in model.schedule]
+    model, cache, device = engine.model, engine.cache, engine.options.device
 
-    def timed(per_layer) -> float:
-        """Seconds of one call of per_layer(block, ctx), averaged over the layers. The calls over the layers are captured into
-        a graph and the replay is timed, as a step runs them: launched one by one the host's path through Python would count."""
-        def over_the_layers():
-            for block, context_of, call in calls:
-                per_layer(block, context_of(batch_of_step, call))
+    def captured(limit, period=None):
+        runner = ModelRunner(model, cache, device, portion_graph_after=1, lanes_from=engine.runner.lanes_from)
+        entries, handles = make_entries()
+        with first_launches(limit, period) as seen:
+            runner.step(entries, choose=choose)
+        graphs = list(runner._graphs.values()) + list(runner._portion_graphs.values())
+        assert len(graphs) == 1 and graphs[0].graph is not None, "the step was not captured"
+        # the eager run before the capture and the capture itself ask for the same launches
+        names = seen.asked[: len(seen.asked) // 2]
+        assert names == seen.asked[len(names):], "the captured step is not the step that ran"
+        return runner, graphs[0].graph, names, handles
 
-        over_the_layers()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            over_the_layers()
+    def replay_us(graph):
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        samples = []
-        for rep in range(reps + 2):
+        graph.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
             start.record()
-            graph.replay()
+            for _ in range(reps):
+                graph.replay()
             stop.record()
             torch.cuda.synchronize()
-            samples.append(start.elapsed_time(stop) / 1e3 / len(calls))
-        return float(np.median(samples[2:]))
+            best = min(best, start.elapsed_time(stop) * 1e3 / reps)
+        return best
 
-    def staged(entries):
-        """The batch of a step whose pages are reserved but which is never committed."""
-        for entry in entries:
-            cache.reserve(entry.request_id, len(entry.tokens))
-        return build_step_batch(entries, cache, runner.staging, vocab_size=vocab, short_portion=model.short_portion())
+    runner, graph, names, handles = captured(None)
+    whole = replay_us(graph)
+    runner.drop_graphs()
+    for h in handles:
+        engine.release_cache(h)
+    upto = []
+    for n in range(1, len(names)):
+        runner, graph, _, handles = captured(n, len(names))   # the step runs once before its capture: the first n of each run
+        upto.append(replay_us(graph))
+        runner.drop_graphs()
+        for h in handles:
+            engine.release_cache(h)
+    upto.append(whole)
+    each = [upto[0]] + [max(0.0, upto[i] - upto[i - 1]) for i in range(1, len(upto))]
+    return names, each
 
+
+def measure_kernels(engine, batch: int = 8, context: int = 768):
+    """What the kernels that a step's time goes to take inside the step and reach of their own roofline
+    (``kernel_times_inside_a_step``): for a 2,048-token prompt step the four products of a layer and the prompt
+    attention (flops / time / the matrix cores' peak), for a greedy decode step of ``batch`` sequences at ``context``
+    tokens the kernels of a layer, the head and the choice of the tokens (the bytes each has to read / time / the
+    memory's peak); a layer's kernel is the mean over the layers. The reference prices its kernels against a pure read
+    of the same bytes (docs/kernels/010_matvec_batch.md:20,108-117) and times the stages of its steps with event pairs
+    (engine/src/gpu_timer.cu:13-120)."""
+    import numpy as np
+
+    from mini_llm_amd.engine import StepEntry
+
+    config, dtype = engine.config, engine.options.dtype
+    e = element_size(dtype)
+    d, ff, n_layer, vocab = config.n_embd, config.n_inner, config.n_layer, config.vocab_size
+    rng = np.random.default_rng(SEED + 4)
     out = {}
 
-    def note(name, seconds, work, peak, unit):
-        out[name] = {"us": round(seconds * 1e6, 2), "frac": round(work / seconds / peak, 4), "of": unit}
+    def note(name, us, work, peak, unit):
+        out[name] = {"us": round(us, 2), "frac": round(work / (us * 1e-6) / peak, 4) if us > 0 else None, "of": unit}
+
+    def by_layer(names, each, tail):
+        """The step's kernels as (first, [per layer: the mean over the layers of each kernel of a layer], last ``tail``), if
+        the kernels between the first and the last ones fall into n_layer equal runs; else None."""
+        middle = len(names) - 1 - tail
+        if middle <= 0 or middle % n_layer:
+            return None
+        per = middle // n_layer
+        layers = [(names[1 + k], float(np.mean([each[1 + layer * per + k] for layer in range(n_layer)]))) for k in range(per)]
+        return (names[0], each[0]), layers, list(zip(names[-tail:], each[-tail:]))
 
     # --- a prompt step of two 1,024-token prompts
     lengths = [CONTEXT, CONTEXT]
-    handles = [engine.try_take_cache() for _ in lengths]
-    entries = [StepEntry(h, rng.integers(0, vocab, n).tolist(), [n - 1]) for h, n in zip(handles, lengths)]
-    batch_of_step = staged(entries)
+    prompts = [rng.integers(0, vocab, n).astype(np.int32) for n in lengths]
+
+    def prompt_step():
+        handles = [engine.try_take_cache() for _ in lengths]
+        return [StepEntry(h, p, [len(p) - 1]) for h, p in zip(handles, prompts)], handles
+
+    names, each = kernel_times_inside_a_step(engine, prompt_step, choose=False)
     rows = sum(lengths)
-    hidden = model.embedding.forward(batch_of_step.tokens, batch_of_step.positions, model.position_encoding)
-    block0 = model.blocks[0]
-    mixer, feed = block0.mixer_part(), block0.feed_forward
-    x = block0.norm_1.forward(hidden, compute)
     peak, unit = PEAK_FLOPS[dtype], f"{'bf16' if dtype == 'bfloat16' else 'fp32'} matrix peak"
-    kept = {}
+    cut = by_layer(names, each, tail=2)   # the final norm and the head
+    out["prefill_step"] = {"us": round(sum(each), 1), "kernels": len(names)}
+    if cut is not None and len(cut[1]) == 7:
+        (_, norm_1), (_, qkv), (_, attention), (_, proj), (_, norm_2), (_, up), (_, down) = cut[1]
+        note("prefill_qkv_product", qkv, 2.0 * rows * d * 3 * d, peak, unit)
+        note("prefill_attention", attention, sum(4.0 * (n * (n + 1) / 2) * d for n in lengths), peak, unit)
+        note("prefill_out_product", proj, 2.0 * rows * d * d, peak, unit)
+        note("prefill_up_product", up, 2.0 * rows * d * ff, peak, unit)
+        note("prefill_down_product", down, 2.0 * rows * d * ff, peak, unit)
+        out["prefill_norms"] = {"us": round(norm_1 + norm_2, 2)}
+    else:
+        out["prefill_step"]["by_entry_point"] = _by_entry_point(names, each)
 
-    def qkv(block, ctx):
-        m = block.mixer_part()
-        kept["q"] = kernels.linear_qkv_cache(x, m.qkv.weight, m.qkv.bias, ctx.k_pages, ctx.v_pages, ctx.group.slots, m.n_heads, m.n_kv_heads, m.head_size)
+    # --- a greedy decode step: ``batch`` sequences that hold ``context`` tokens each (a whole number of pages: the replays
+    # of the whole step move the sequences on by a token each, and must stay on the page the step has reserved)
+    page = engine.cache.page_size
+    assert context % page == 0 and page >= 64, "the decode step's replays need room on the sequences' newest page"
+    stored = [rng.integers(0, vocab, context).tolist() for _ in range(batch)]
 
-    note("prefill_qkv_product", timed(qkv), 2.0 * rows * d * 3 * d, peak, unit)
+    def decode_step():
+        handles = [engine.try_take_cache() for _ in range(batch)]
+        for i in range(0, batch, 4):
+            engine.runner.step([StepEntry(h, tokens, []) for h, tokens in zip(handles[i : i + 4], stored[i : i + 4])])
+        return [StepEntry(h, [int(rng.integers(0, vocab))], [0]) for h in handles], handles
 
-    def attention(block, ctx):
-        m, b = block.mixer_part(), ctx.batch
-        kept["mixed"] = kernels.paged_attention(kept["q"], ctx.k_pages, ctx.v_pages, b.token_request, b.positions, ctx.group.block_tables, m.n_heads,
-                                                m.n_kv_heads, m.head_size, m.scale, max_q_len=b.max_q_len, max_len=b.max_total_len,
-                                                q_starts=b.q_starts, context_lens=b.context_lens)
-
-    note("prefill_attention", timed(attention), sum(4.0 * (n * (n + 1) / 2) * d for n in lengths), peak, unit)
-    note("prefill_out_product", timed(lambda block, ctx: block.mixer_part().out.forward_pending(kept["mixed"], hidden)), 2.0 * rows * d * d, peak, unit)
-
-    def up(block, ctx):
-        kept["u"] = block.feed_forward.up.forward(x, activation=block.feed_forward.activation)
-
-    note("prefill_up_product", timed(up), 2.0 * rows * d * ff, peak, unit)
-    note("prefill_down_product", timed(lambda block, ctx: block.feed_forward.down.forward_pending(kept["u"], hidden)), 2.0 * rows * d * ff, peak, unit)
-    kept.clear()
-    for h in handles:
-        cache.rollback(h)
-        engine.release_cache(h)
-
-    # --- a decode step: ``batch`` sequences that hold ``context`` tokens each
-    handles = [engine.try_take_cache() for _ in range(batch)]
-    for i in range(0, batch, 4):
-        runner.step([StepEntry(h, rng.integers(0, vocab, context - 1).tolist(), []) for h in handles[i : i + 4]])
-    entries = [StepEntry(h, [int(rng.integers(0, vocab))], [0]) for h in handles]
-    batch_of_step = staged(entries)
-    hidden = model.embedding.forward(batch_of_step.tokens, batch_of_step.positions, model.position_encoding)
+    names, each = kernel_times_inside_a_step(engine, decode_step, choose=True)
     hbm = HBM_GBS * 1e9
-    # each half takes the stream as the other half leaves it (with its last sums pending, where the parts do that)
-    context_0 = cache.layer_context(batch_of_step, model.schedule[0])
-    after_mlp = feed.forward_normed(hidden, block0.norm_2, compute, context_0)
-    after_attention = mixer.forward_normed(after_mlp, block0.norm_1, compute, context_0)
-    note("decode_attention_half", timed(lambda block, ctx: block.mixer_part().forward_normed(after_mlp, block.norm_1, compute, ctx)),
-         (4.0 * d * d + batch * context * 2.0 * d) * e, hbm, "HBM peak")
-    note("decode_mlp_half", timed(lambda block, ctx: block.feed_forward.forward_normed(after_attention, block.norm_2, compute, ctx)),
-         2.0 * d * ff * e, hbm, "HBM peak")
-    normed = model.final_norm.forward(kernels.settle(hidden), compute, row_index=batch_of_step.logit_rows)
-    logits = {}
-
-    def head(block, ctx):
-        logits["rows"] = model.head.forward(normed)
-
-    note("decode_head", timed(head), float(vocab) * d * e, hbm, "HBM peak")
-    note("decode_sampler", timed(lambda block, ctx: kernels.sample(logits["rows"])), batch * vocab * 4.0, hbm, "HBM peak")
-    for h in handles:
-        cache.rollback(h)
-        engine.release_cache(h)
-    torch.cuda.synchronize()
+    out["decode_step"] = {"us": round(sum(each), 1), "kernels": len(names)}
+    cut = by_layer(names, each, tail=3)   # the final norm, the head and the choice
+    cache_bytes = batch * context * 2.0 * d * e
+    if cut is not None and [name for name, _ in cut[1]] == ["decode_attention_half", "decode_mlp_half"]:
+        note("decode_attention_half", cut[1][0][1], 4.0 * d * d * e + cache_bytes, hbm, "HBM peak")
+        note("decode_mlp_half", cut[1][1][1], 2.0 * d * ff * e, hbm, "HBM peak")
+    elif cut is not None:
+        layer_us = sum(us for _, us in cut[1])
+        note("decode_layer", layer_us, (4.0 * d * d + 2.0 * d * ff) * e + cache_bytes, hbm, "HBM peak")
+        out["decode_layer"]["by_entry_point"] = _by_entry_point([name for name, _ in cut[1]], [us for _, us in cut[1]])
+    if cut is not None:
+        out["decode_embed"] = {"us": round(cut[0][1], 2), "holds": "what a replay costs by itself"}
+        (_, final_norm), (_, head), (_, choice) = cut[2]
+        out["decode_final_norm"] = {"us": round(final_norm, 2)}
+        note("decode_head", head, float(vocab) * d * e, hbm, "HBM peak")
+        out["decode_choice"] = {"us": round(choice, 2)}
+    else:
+        out["decode_step"]["by_entry_point"] = _by_entry_point(names, each)
     return out
+
+
+def _by_entry_point(names, each):
+    """entry point -> [launches, microseconds in sum], for a step whose kernels do not fall into the pattern looked for."""
+    table = {}
+    for name, us in zip(names, each):
+        entry = table.setdefault(name, [0, 0.0])
+        entry[0] += 1
+        entry[1] = round(entry[1] + us, 2)
+    return table
 
 
 def check_before_timing(engine, host_weights=None, n_new: int = 8):

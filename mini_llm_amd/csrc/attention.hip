@@ -736,8 +736,10 @@ MLLM_API int mllm_attention_prefill_supported(int head_size, int page_size) {
 MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out,
                                     int out_stride, const int* q_starts, const int* context_lens,
                                     const int* block_tables, int max_blocks, int n_requests, int max_q_len,
-                                    int n_heads, int n_kv_heads, int head_size, int page_size, int window,
+                                    int max_len, int n_heads, int n_kv_heads, int head_size, int page_size, int window,
                                     float scale, int dtype, hipStream_t stream) {
+    // max_len: the longest sequence after this step, or a bound on it (0 or less: what the block tables can hold); it only
+    // decides how many waves share a block's keys
     MLLM_REQUIRE(n_requests >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_prefill: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_prefill: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_prefill_supported(head_size, page_size),
@@ -756,7 +758,9 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
         // long portions in bfloat16, heads of 32 / 64 / 128, pages of 32 keys or more: keys and values stream from the pages straight into LDS
 #define MLLM_STREAM_CASE(HD)                                                                                            \
     prefill_stream::launch<HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
-                               max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
+                               max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, stream)
+        const long table_reach = (long)max_blocks * page_size;
+        const int reach = (int)(max_len > 0 && max_len < table_reach ? max_len : (table_reach < (1 << 30) ? table_reach : (1 << 30)));
         if (head_size == 32) MLLM_STREAM_CASE(32);
         else if (head_size == 64) MLLM_STREAM_CASE(64);
         else MLLM_STREAM_CASE(128);

@@ -26,7 +26,7 @@
 namespace prefill_stream {
 
 constexpr int KEYS = 32;      // keys per tile
-constexpr int SPLITS = 4;     // waves per block; wave w takes tiles w, w + 4, ...
+// SPLITS (a parameter of the kernel): waves per block, 4 or 8; wave w takes tiles w, w + SPLITS, ...
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -113,7 +113,7 @@ __device__ __forceinline__ void read_transposed<4, 256>(const unsigned (&address
         : "memory");
 }
 
-template <int HD>
+template <int HD, int SPLITS>
 struct Layout {
     static constexpr int PPR = HD / 8;              // 16-byte pieces per row
     static constexpr int ROW_BYTES = HD * 2;
@@ -132,12 +132,14 @@ struct Layout {
 
 // QUERIES: 64 queries a block (two sub-tiles of 32, both held by every wave), or 32 where that would leave compute units
 // without a block: what the kernel waits for is the wave with the most tiles, and a tile of 32 queries takes it half as long.
-template <int HD, int QUERIES>
-__global__ __launch_bounds__(64 * SPLITS, HD <= 64 ? 2 : 1) void attention_prefill_stream_kernel(
+// SPLITS: four waves a block, or eight where the portions reach far back: the kernel's time is the time of the wave with
+// the most tiles (it pays every tile's chain in full), which eight waves halve; a block then has a compute unit to itself.
+template <int HD, int QUERIES, int SPLITS>
+__global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) void attention_prefill_stream_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
     bf16_t* __restrict__ out, int out_stride, const int* __restrict__ q_starts, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads, int page_shift, int window, float scale) {
-    typedef Layout<HD> L;
+    typedef Layout<HD, SPLITS> L;
     constexpr int QSUB = QUERIES / 32;
     static_assert(QUERIES == 32 || QUERIES == 64, "one or two sub-tiles of queries");
     constexpr int QSTEPS = HD / 16;  // k-steps of the score product
@@ -438,34 +440,48 @@ inline bool takes(int head_size, int page_size, int max_q_len, float scale, int 
     return q_stride % 8 == 0 && out_stride % 4 == 0 && ((size_t)q) % 16 == 0 && ((size_t)out) % 8 == 0;
 }
 
-template <int HD, int QUERIES>
+template <int HD, int QUERIES, int SPLITS>
 void launch_queries(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
                     const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
                     int page_shift, int window, float scale, hipStream_t stream) {
-    constexpr int LDS_BYTES = Layout<HD>::LDS_BYTES;
+    constexpr int LDS_BYTES = Layout<HD, SPLITS>::LDS_BYTES;
     static bool raised = false;  // per instantiation: the limit on dynamic LDS is a property of the kernel
     if (!raised && LDS_BYTES > 60 * 1024)  // (if this fails the launch below fails too, and the entry point reports that)
-        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD, QUERIES>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
+        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD, QUERIES, SPLITS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
     // x: (request, head), so that with a multiple of eight heads the blocks of one head share an XCD's L2; y: tiles of queries
     dim3 grid(n_heads * n_requests, ceil_div(max_q_len, QUERIES));
     mllm_count_kernel(MLLM_K_ATTENTION_PREFILL_STREAM);
-    attention_prefill_stream_kernel<HD, QUERIES><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
+    attention_prefill_stream_kernel<HD, QUERIES, SPLITS><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, out_stride, q_starts, context_lens,
         block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);
 }
 
 template <int HD>
 void launch(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
-            const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
-            int page_shift, int window, float scale, hipStream_t stream) {
+            const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int max_len, int n_heads,
+            int n_kv_heads, int page_shift, int window, float scale, hipStream_t stream) {
+#define MLLM_STREAM_LAUNCH(QUERIES, SPLITS)                                                                                              \
+    launch_queries<HD, QUERIES, SPLITS>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, \
+                                        n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
     // blocks of 64 queries where they give every compute unit a block (measured: 2 x 1,024 tokens x 12 heads 15.9 against 17.2 us),
     // else of 32 (4 x 128 tokens on 896 cached: 9.7 against 13.0 us; 512 on 7,680: 46.7 against 66.0 us)
-    if ((long)n_heads * n_requests * ceil_div(max_q_len, 64) >= 256)
-        launch_queries<HD, 64>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, n_requests, max_q_len,
-                               n_heads, n_kv_heads, page_shift, window, scale, stream);
-    else
-        launch_queries<HD, 32>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, n_requests, max_q_len,
-                               n_heads, n_kv_heads, page_shift, window, scale, stream);
+    const bool wide = (long)n_heads * n_requests * ceil_div(max_q_len, 64) >= 256;
+    // Eight waves a block where the block of the last queries has sixteen tiles of keys or more to walk (max_len: the longest
+    // sequence after this step, or what bounds it; a window bounds the keys too) AND every block still finds a compute
+    // unit of its own at once (eight waves' tiles leave room for one block a unit): a long context with few queries.
+    // Measured, heads of 64: 512 queries on 7,680 cached keys 38.2 against 46.7 us with four waves; but two prompts of 1,024
+    // tokens (384 blocks: a second round) 19.1 against 15.9 us, one of 4,096 64.8 against 57 us.
+    const int reach = window > 0 ? min(max_len, window + 64) : max_len;
+    const long blocks = (long)n_heads * n_requests * ceil_div(max_q_len, wide ? 64 : 32);
+    bool eight = false;
+    if constexpr (HD <= 64) {  // (eight waves' tiles of a head of 128 do not fit a compute unit's LDS)
+        eight = reach >= 16 * KEYS && blocks <= 256;
+        if (wide && eight) MLLM_STREAM_LAUNCH(64, 8);
+        else if (eight) MLLM_STREAM_LAUNCH(32, 8);
+    }
+    if (wide && !eight) MLLM_STREAM_LAUNCH(64, 4);
+    else if (!eight) MLLM_STREAM_LAUNCH(32, 4);
+#undef MLLM_STREAM_LAUNCH
 }
 
 }  // namespace prefill_stream

@@ -431,7 +431,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         n_requests = context_lens.shape[0]
         _require(q_starts.shape[0] == n_requests + 1, "q_starts must have one entry more than context_lens")
         _require(block_tables.shape[0] >= n_requests, "fewer block tables than requests")
-        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
+        check(lib.mllm_attention_prefill(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_starts), _ptr(context_lens), _ptr(block_tables), block_tables.shape[1], n_requests, int(max_q_len), int(max_len or 0), n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
         return out
     check(lib.mllm_attention(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads, head_size, page_size, int(window), float(scale), _code(q.dtype), _stream()))
     return out

@@ -32,7 +32,7 @@ _SIGNATURES = {
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
-    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
+    "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
     "mllm_gemm_best_per_row": [c_int, c_int, c_int, c_int],
@@ -56,6 +56,8 @@ class KernelLibraryError(RuntimeError):
 
 def library() -> ctypes.CDLL:
     global _library
+    if _standing_in is not None:
+        return _standing_in
     if _library is None:
         path = os.environ.get("MINI_LLM_LIBRARY")
         if path:
@@ -84,6 +86,57 @@ def library() -> ctypes.CDLL:
         lib.path = path
         _library = lib
     return _library
+
+
+class _FirstLaunches:
+    """Stands in for the library while ``first_launches`` is active: lets the first so many kernel launches through,
+    answers every later one with "launched" without launching, and keeps the names of all that were asked for."""
+
+    def __init__(self, lib, limit, period):
+        self._lib, self._limit, self._period = lib, limit, period
+        self.asked = []
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        argtypes = _SIGNATURES.get(name)
+        if not argtypes or argtypes[-1] is not P or name.startswith("mllm_probe"):
+            return fn   # a question about sizes, not a launch (every launching entry point ends with its stream)
+
+        def launch(*args):
+            at = len(self.asked)
+            self.asked.append(name[len("mllm_"):])
+            if self._limit is not None and (at % self._period if self._period else at) >= self._limit:
+                return 0
+            return fn(*args)
+
+        return launch
+
+
+_standing_in: _FirstLaunches | None = None
+
+
+class first_launches:
+    """``with first_launches(n) as seen:`` - inside, only the first ``n`` kernel launches of this process's calls into the
+    library really happen (``n`` None: all of them; with ``period`` p: the first n of every p, for work that is run
+    several times over, as a step is before and during its capture); ``seen.asked`` lists the entry points of all
+    launches that were asked for, in order. For measuring: a step captured under it is the first n kernels of that step, so the time of kernel n
+    inside the step is the difference between two such graphs' replays (the reference times the stages of its steps with
+    event pairs instead, engine/src/gpu_timer.cu:13-120; a replayed graph has no place for those). Whatever the skipped
+    kernels would have written is left as it was: nothing computed inside may be used."""
+
+    def __init__(self, limit: int | None, period: int | None = None):
+        self._limit, self._period = limit, period
+
+    def __enter__(self):
+        global _standing_in
+        if _standing_in is not None:
+            raise RuntimeError("first_launches is already active")
+        _standing_in = _FirstLaunches(library(), self._limit, self._period)
+        return _standing_in
+
+    def __exit__(self, *_):
+        global _standing_in
+        _standing_in = None
 
 
 def check(status: int) -> None:

@@ -406,14 +406,16 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
     [(3, 3, 32, 16, 0), (2, 2, 64, 64, 0), (4, 2, 64, 16, 150), (2, 1, 128, 8, 0), (2, 2, 128, 256, 0), (3, 3, 32, 32, 70),
      (2, 2, 48, 32, 0), (5, 5, 64, 4, 0)],
 )
-@pytest.mark.parametrize("copies", [1, 12])
-def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head_size, page_size, window, copies):
+@pytest.mark.parametrize("copies,reach", [(1, None), (12, None), (1, 100), (12, 100)])
+def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head_size, page_size, window, copies, reach):
     # portions of several query tiles over several key tiles, requests of different lengths in one call (one
     # with a single token, one that starts at position 0, one whose portion ends one past a tile), pages
     # scrambled and unwritten places holding NaN. In the longest request some queries look hard at one far
     # key each (the first key, keys at the two sides of tile and page edges), so that a tile that is
     # skipped, read twice or read from a wrong page shows in those rows. Once as they are (few blocks: the
-    # bfloat16 kernel takes 32 queries a block) and once twelve times over (64 queries a block).
+    # bfloat16 kernel takes 32 queries a block) and once twelve times over (64 queries a block); with the reach of the
+    # longest sequence as the block tables give it (eight waves share a block's keys where heads are 64 or less) and
+    # named short (four waves: the number only decides how a block's keys are shared out).
     rng = np.random.default_rng(head_size * 10 + page_size)
     shapes = [(0, 300), (200, 129), (500, 1), (70, 65), (0, 2)] * copies
     need = sum((c + n + page_size - 1) // page_size for c, n in shapes)
@@ -449,7 +451,7 @@ def test_prompt_attention_over_long_portions(K, dtype, n_heads, n_kv_heads, head
     starts = np.cumsum([0] + [new for _, new in shapes])
     out = K.paged_attention(
         dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
-        n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=300,
+        n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=300, max_len=reach,
         q_starts=dev(starts, torch.int32), context_lens=dev([c for c, _ in shapes], torch.int32))
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     np.testing.assert_allclose(host(out), np.concatenate(refs), rtol=tol, atol=tol)
