@@ -155,20 +155,22 @@ def measure_prefill(engine, runs: int = 5):
             "frac": round(flops / seconds / PEAK_FLOPS[engine.options.dtype], 4), "from_graph": engine.runner.portion_graph_steps - replayed_before >= runs}
 
 
-def kernel_times_inside_a_step(engine, make_entries, choose: bool, reps: int = 5):
+def kernel_times_inside_a_step(engine, make_entries, choose: bool, reps: int = 5):   # (reps_of_a_step: what callers plan room for)
     """(names, microseconds): the kernels of one real step of the engine, in order, and what each takes INSIDE the step.
 
     The step goes through the engine's own step function and is captured as generation captures it. It is captured once
     for every n with only its first n kernels really launched (ops.library.first_launches), and the replay of each such
     graph is timed: kernel n's time is the difference between two of them. So a time holds what the kernel costs where it
     stands: its start behind the kernel before it, and its first trip to memory for what that one wrote. (The first
-    kernel's figure also holds what a replay costs by itself.) ``make_entries()`` opens the step's requests and returns
+    kernel's figure also holds what a replay and the two events around it cost by themselves.) ``make_entries()`` opens the step's requests and returns
     (entries, handles); they are given back after each capture."""
     import numpy as np
     import torch
 
+    import ctypes
+
     from mini_llm_amd.engine.step import ModelRunner
-    from mini_llm_amd.ops.library import first_launches
+    from mini_llm_amd.ops.library import check, first_launches, library
 
     model, cache, device = engine.model, engine.cache, engine.options.device
 
@@ -184,38 +186,48 @@ def kernel_times_inside_a_step(engine, make_entries, choose: bool, reps: int = 5
         assert names == seen.asked[len(names):], "the captured step is not the step that ran"
         return runner, graphs[0].graph, names, handles
 
+    # Between two timed replays the caches are emptied by a read of 512 MiB of other memory: in generation a step's weights and
+    # cache rows have been pushed out by the rest of the step before they are read again, but a short graph replayed by
+    # itself would find everything still in the 256 MB memory-side cache.
+    lib = library()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    other = torch.zeros((512 << 20) // 4, dtype=torch.float32, device=device)
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+
     def replay_us(graph):
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         graph.replay()
-        torch.cuda.synchronize()
-        best = float("inf")
-        for _ in range(3):
+        samples = []
+        for _ in range(reps):
+            check(lib.mllm_probe_read(ctypes.c_void_p(other.data_ptr()), other.numel() * 4, ctypes.c_void_p(sink.data_ptr()), 2048, stream))
             start.record()
-            for _ in range(reps):
-                graph.replay()
+            graph.replay()
             stop.record()
             torch.cuda.synchronize()
-            best = min(best, start.elapsed_time(stop) * 1e3 / reps)
-        return best
+            samples.append(start.elapsed_time(stop) * 1e3)
+        return float(np.median(samples))
 
-    runner, graph, names, handles = captured(None)
-    whole = replay_us(graph)
-    runner.drop_graphs()
-    for h in handles:
-        engine.release_cache(h)
-    upto = []
-    for n in range(1, len(names)):
-        runner, graph, _, handles = captured(n, len(names))   # the step runs once before its capture: the first n of each run
-        upto.append(replay_us(graph))
+    def forget(runner, handles):
         runner.drop_graphs()
         for h in handles:
             engine.release_cache(h)
-    upto.append(whole)
+
+    runner, graph, names, handles = captured(None)   # for the names and their number
+    forget(runner, handles)
+    upto = []
+    for n in range(1, len(names) + 1):
+        runner, graph, _, handles = captured(n, len(names))   # the step runs once before its capture: the first n of each run
+        upto.append(replay_us(graph))
+        forget(runner, handles)
     each = [upto[0]] + [max(0.0, upto[i] - upto[i - 1]) for i in range(1, len(upto))]
     return names, each
 
 
-def measure_kernels(engine, batch: int = 8, context: int = 768):
+def reps_of_a_step() -> int:
+    return 5
+
+
+def measure_kernels(engine, batch: int = 8, context: int = 776):
     """What the kernels that a step's time goes to take inside the step and reach of their own roofline
     (``kernel_times_inside_a_step``): for a 2,048-token prompt step the four products of a layer and the prompt
     attention (flops / time / the matrix cores' peak), for a greedy decode step of ``batch`` sequences at ``context``
@@ -270,10 +282,10 @@ def measure_kernels(engine, batch: int = 8, context: int = 768):
     else:
         out["prefill_step"]["by_entry_point"] = _by_entry_point(names, each)
 
-    # --- a greedy decode step: ``batch`` sequences that hold ``context`` tokens each (a whole number of pages: the replays
-    # of the whole step move the sequences on by a token each, and must stay on the page the step has reserved)
+    # --- a greedy decode step: ``batch`` sequences that hold ``context`` tokens each (the replays of the whole step move
+    # the sequences on by a token each, and must stay on the page the step has reserved)
     page = engine.cache.page_size
-    assert context % page == 0 and page >= 64, "the decode step's replays need room on the sequences' newest page"
+    assert page - context % page > reps_of_a_step() + 8, "the decode step's replays need room on the sequences' newest page"
     stored = [rng.integers(0, vocab, context).tolist() for _ in range(batch)]
 
     def decode_step():
@@ -484,6 +496,8 @@ def main() -> int:
     parser.add_argument("--shape", default="small", choices=("small", "medium", "xl"), help="the GPT-2 shape that is run (the headline is small)")
     parser.add_argument("--prompt-len", "--prompt-tokens", dest="prompt_len", type=int, default=PROMPT_LEN,
                         help="tokens of each sequence's prompt before decoding is timed (--prompt-tokens is the reference's name: engine/bench/bench_options.c:25-94)")
+    parser.add_argument("--context", type=int, default=CONTEXT, help="the model's positions: sequences decode towards this length, and the prompt step is two prompts of this length "
+                        "(the headline is 1024; a longer one runs the same layer sizes with a longer position table)")
     parser.add_argument("--json", default=None, metavar="PATH", help="also write the printed record to this file (the reference's option)")
     parser.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     parser.add_argument("--no-check", action="store_true", help="skip the comparison of decoding with a whole-prompt step before timing")
@@ -513,6 +527,13 @@ def main() -> int:
     from mini_llm_amd.weights import bind_tensors, random_tensors
 
     shape, seed = SHAPES[args.shape]
+    if args.context != CONTEXT:
+        if args.context < 64:
+            parser.error("--context must be at least 64")
+        if args.prompt_len == PROMPT_LEN:
+            args.prompt_len = args.context // 2
+        globals()["CONTEXT"] = args.context
+        shape = dict(shape, n_positions=args.context)
     if not 1 <= args.prompt_len < CONTEXT:
         parser.error(f"--prompt-len must be in 1..{CONTEXT - 1}")
     layers = args.layers or shape["n_layer"]
@@ -578,7 +599,7 @@ def main() -> int:
             s, _ = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
             points[f"decode_b{batch}"] = round(batch * steps / s, 1)
         record["points"] = points
-        record["kernels"] = measure_kernels(engine)
+        record["kernels"] = measure_kernels(engine, context=(3 * CONTEXT // 4) // 64 * 64 + 8)
         if not args.one_dtype:
             # the same figures in the other precision (the headline names both): one record for the two
             other = "float32" if args.dtype == "bfloat16" else "bfloat16"
