@@ -251,7 +251,8 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
         for (int base = begin; base < end; base += KPI) {
             const int next = base + KPI;
             if (PAGES_AHEAD && next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
-            sweep.consume(f, qf, base, end, lane);
+            if constexpr (sizeof(T) == 2) sweep.consume(f, raw, scale, base, end, lane);  // bfloat16: the query as it is stored
+            else sweep.consume(f, qf, base, end, lane);
             if (!PAGES_AHEAD && next < end) sweep.look_up(page, table, page_shift, next, end, spare_key, lane);
             if (next < end) sweep.fetch_rows(f, page, k_pages, v_pages, kv_head, n_kv_heads, page_shift, next, end, spare_key, lane);
         }

@@ -288,12 +288,16 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         lds_barrier();  // 4
         lds_barrier();  // 5: q, k, v of this token are in LDS
         float qf[VEC];
+        bf16x8 q_stored;  // the query as a kernel of its own would have stored it: the cached keys meet it in pairs
 #pragma unroll
-        for (int i = 0; i < VEC; i++) qf[i] = qkv_row[0][sub * VEC + i] * scale;
+        for (int i = 0; i < VEC; i++) {
+            qf[i] = qkv_row[0][sub * VEC + i] * scale;
+            q_stored[i] = static_cast<bf16_t>(qkv_row[0][sub * VEC + i]);
+        }
         sweep.init();
         // not under a condition (a wave without keys counts none): the compiler would move the loads
         // above down into a conditional block, behind the meetings of the waves
-        sweep.template consume<true>(fetched, qf, begin, end, lane);
+        sweep.template consume<true>(fetched, q_stored, scale, begin, end, lane);
         if (wave == DL_PROJECT_WAVES) sweep.one_key(qf, qkv_row[1], qkv_row[2], lane);  // the token's own key and value, from LDS
         sweep.merge_inside_rows();
         {
@@ -398,13 +402,13 @@ __global__ __launch_bounds__(DL_THREADS) void decode_attention_half_kernel(
         lds_barrier();  // 4: the shares of the q/k/v product are in LDS
         finish_qkv_rows();
         lds_barrier();  // 5: q, k, v of this token are in LDS
-        float qf[VEC];
+        bf16x8 q_stored;
 #pragma unroll
-        for (int i = 0; i < VEC; i++) qf[i] = qkv_row[0][sub * VEC + i] * scale;
+        for (int i = 0; i < VEC; i++) q_stored[i] = static_cast<bf16_t>(qkv_row[0][sub * VEC + i]);
         sweep.init();
-        sweep.template consume<true>(fetched, qf, begin, end, lane);  // not under a further condition, as above
+        sweep.template consume<true>(fetched, q_stored, scale, begin, end, lane);  // not under a further condition, as above
         if (begin + KPI < end)  // a context longer than one round of every wave of the block covers
-            sweep.keys(qf, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin + KPI, end, lane);
+            sweep.keys(q_stored, scale, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, begin + KPI, end, lane);
         sweep.merge_inside_rows();
     } else {
         lds_barrier();  // 4

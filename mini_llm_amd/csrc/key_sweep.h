@@ -25,6 +25,15 @@ struct Chunk<bf16_t> {
     static __device__ __forceinline__ float get(const Raw& r, int i) { return static_cast<float>(r[i]); }
 };
 
+// e^x for the softmax weights of a sweep. In 32-bit the library's expf; where keys and values are bfloat16 (eight bits
+// of fraction) the hardware's 2^x of x log2(e), three instructions instead of a score of them and one unit in the last
+// place of a 32-bit result: the sweep's arithmetic is what a decode step's attention waits for once its rows are there.
+template <typename T>
+__device__ __forceinline__ float sweep_exp(float x) {
+    if constexpr (sizeof(T) == 2) return __builtin_amdgcn_exp2f(x * 1.4426950408889634f);
+    else return expf(x);
+}
+
 template <typename T, int HD>
 struct KeySweep {
     static constexpr int VEC = Chunk<T>::VEC;
@@ -99,29 +108,59 @@ struct KeySweep {
     // a weight of zero silences a NaN.
     template <bool CLEAN_VALUES = false>
     __device__ __forceinline__ void consume(const Fetched& f, const float (&qf)[VEC], int base, int end, int lane) {
-        const int group = lane / LPR;
-        float score[UNROLL];
-        float tile_max = -INFINITY;
+        float dots[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             float dot = 0.0f;
 #pragma unroll
             for (int i = 0; i < VEC; i++) dot += qf[i] * Chunk<T>::get(f.kf[u], i);
-            dot = lanes_sum<LPR>(dot);
+            dots[u] = dot;
+        }
+        take<CLEAN_VALUES>(f, dots, base, end, lane);
+    }
+
+    // The same for a query kept as it is stored, in bfloat16 (the lane's VEC dimensions), and the factor its scores are
+    // scaled by: the products of two bfloat16 numbers are exact in 32-bit, so a dot product over pairs (v_dot2c_f32_bf16)
+    // gives what the converted numbers would, in a quarter of the instructions.
+    template <bool CLEAN_VALUES = false>
+    __device__ __forceinline__ void consume(const Fetched& f, const Raw& q, float scale, int base, int end, int lane) {
+        static_assert(sizeof(T) == 2, "a query in bfloat16 meets keys in bfloat16");
+        float dots[UNROLL];
+        const bf16x2* q_pairs = reinterpret_cast<const bf16x2*>(&q);
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const bf16x2* k_pairs = reinterpret_cast<const bf16x2*>(&f.kf[u]);
+            float dot = 0.0f;
+#pragma unroll
+            for (int i = 0; i < VEC / 2; i++) dot = __builtin_amdgcn_fdot2_f32_bf16(q_pairs[i], k_pairs[i], dot, false);
+            dots[u] = dot * scale;
+        }
+        take<CLEAN_VALUES>(f, dots, base, end, lane);
+    }
+
+    // dots: this lane's share of the scaled dot products of the fetched keys with the query.
+    template <bool CLEAN_VALUES>
+    __device__ __forceinline__ void take(const Fetched& f, const float (&dots)[UNROLL], int base, int end, int lane) {
+        const int group = lane / LPR;
+        float score[UNROLL];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            float dot = lanes_sum<LPR>(dots[u]);
             score[u] = base + u * RPI + group < end ? dot : -INFINITY;
             tile_max = fmaxf(tile_max, score[u]);
         }
         tile_max = wave_max_total(tile_max);
         float new_max = fmaxf(running_max, tile_max);
         float reference = new_max == -INFINITY ? 0.0f : new_max;  // no key so far (base >= end is allowed): nothing to rescale
-        float rescale = expf(running_max - reference);
+        float rescale = sweep_exp<T>(running_max - reference);
         running_sum *= rescale;
 #pragma unroll
         for (int i = 0; i < VEC; i++) o[i] *= rescale;
 #pragma unroll
         for (int u = 0; u < UNROLL; u++) {
             const bool counts = base + u * RPI + group < end;
-            float p = counts ? expf(score[u] - reference) : 0.0f;
+            float p = counts ? sweep_exp<T>(score[u] - reference) : 0.0f;
             running_sum += p;
 #pragma unroll
             for (int i = 0; i < VEC; i++) {
@@ -144,6 +183,17 @@ struct KeySweep {
         }
     }
 
+    // The same with the query as it is stored (bfloat16).
+    __device__ __forceinline__ void keys(const Raw& q, float scale, const T* __restrict__ k_pages,
+                                         const T* __restrict__ v_pages, const int* __restrict__ table,
+                                         int kv_head, int n_kv_heads, int page_shift, int begin, int end, int lane) {
+        for (int base = begin; base < end; base += KPI) {
+            Fetched f;
+            fetch(f, k_pages, v_pages, table, kv_head, n_kv_heads, page_shift, base, end, end - 1, lane);
+            consume(f, q, scale, base, end, lane);
+        }
+    }
+
     // One more key that is not in the cache: key_row and value_row hold its HD dimensions in
     // 32-bit (LDS or memory). Counted once, by the lanes of row group 0.
     __device__ __forceinline__ void one_key(const float (&qf)[VEC], const float* key_row, const float* value_row, int lane) {
@@ -153,9 +203,9 @@ struct KeySweep {
         for (int i = 0; i < VEC; i++) dot += qf[i] * key_row[sub * VEC + i];
         dot = lanes_sum<LPR>(dot);
         float new_max = fmaxf(running_max, dot);
-        float rescale = expf(running_max - new_max);
+        float rescale = sweep_exp<T>(running_max - new_max);
         running_sum *= rescale;
-        float p = group == 0 ? expf(dot - new_max) : 0.0f;
+        float p = group == 0 ? sweep_exp<T>(dot - new_max) : 0.0f;
         running_sum += p;
 #pragma unroll
         for (int i = 0; i < VEC; i++) o[i] = o[i] * rescale + p * value_row[sub * VEC + i];
