@@ -249,55 +249,55 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const T* _
 
     // A lane holds column lane%32 and rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile.
     if constexpr (BEST) {
-        // Per row the best of this block's columns: first among the lane's own (one per tile along N), then among the
-        // 32 lanes that hold the row (xor steps below 32 stay inside a half of the wave), then among the waves that
-        // share the row, through LDS (the tiles' memory: every wave has left the loop behind the last barrier).
-        float* shared_values = reinterpret_cast<float*>(&a_tiles[0][0]);   // [WAVES_N][BM]
-        int* shared_indices = reinterpret_cast<int*>(&w_tiles[0][0]);
-        static_assert(sizeof(a_tiles) >= WAVES_N * BM * 4 && sizeof(w_tiles) >= WAVES_N * BM * 4, "room for the waves' best columns");
+        // Per row the best of this block's columns. The sums go to LDS as a [BM, BN] matrix (the tiles' memory: every
+        // wave has left the loop behind the last barrier); then the THREADS / BM threads next to each other that share
+        // a row take BN / that many columns each and settle the rest among themselves with data-parallel steps
+        // inside a row of 16 lanes. (Reducing in the layout of the accumulators, where a row's 32 columns lie in 32
+        // lanes, took 160 trips through the LDS crossbar a tile: the head got slower than with its logits written.)
+        constexpr int SHARE = THREADS / BM, COLS = BN / SHARE;   // threads a row, columns a thread
+        static_assert(SHARE >= 1 && SHARE <= 16 && (SHARE & (SHARE - 1)) == 0 && BN % SHARE == 0 && COLS % 4 == 0, "a row's threads lie in one row of 16 lanes");
+        constexpr bool IN_W = sizeof(w_tiles) >= sizeof(float) * BM * BN;
+        static_assert(IN_W || sizeof(a_tiles) >= sizeof(float) * BM * BN, "room for the block's sums");
+        float* sums = IN_W ? reinterpret_cast<float*>(&w_tiles[0][0]) : reinterpret_cast<float*>(&a_tiles[0][0]);
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
+        for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int local_from = wave_m * TM * 32 + i * 32 + 8 * (v / 4);  // the same for the whole wave
                 if (m0 + local_from >= M) continue;
                 const int local_row = local_from + 4 * half + (v % 4);
-                float best = -INFINITY;
-                int best_index = 0x7fffffff;
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    int col = n0 + wave_n * TN * 32 + j * 32 + lane32;
-                    float value = acc[i][j][v] + early_bias[j];
-                    if (col < N && beats(value, col, best, best_index)) {
-                        best = value;
+                for (int j = 0; j < TN; j++) sums[local_row * BN + wave_n * TN * 32 + j * 32 + lane32] = acc[i][j][v] + early_bias[j];
+            }
+        __syncthreads();
+        const int local_row = tid / SHARE, share = tid % SHARE;
+        float best = -INFINITY;
+        int best_index = 0x7fffffff;
+        if (m0 + local_row < M) {   // (whole rows of 16 lanes go one way: SHARE divides 16)
+#pragma unroll
+            for (int c0 = 0; c0 < COLS; c0 += 4) {
+                const f32x4 four = *reinterpret_cast<const f32x4*>(&sums[local_row * BN + share * COLS + c0]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int col = n0 + share * COLS + c0 + e;
+                    if (col < N && beats(four[e], col, best, best_index)) {
+                        best = four[e];
                         best_index = col;
                     }
                 }
-#pragma unroll
-                for (int offset = 16; offset > 0; offset >>= 1) {
-                    float other = __shfl_xor(best, offset, WAVE);
-                    int other_index = __shfl_xor(best_index, offset, WAVE);
-                    if (beats(other, other_index, best, best_index)) {
-                        best = other;
-                        best_index = other_index;
-                    }
-                }
-                if (lane32 == 0) {
-                    shared_values[wave_n * BM + local_row] = best;
-                    shared_indices[wave_n * BM + local_row] = best_index;
-                }
             }
         }
-        __syncthreads();
-        for (int local_row = tid; local_row < BM && m0 + local_row < M; local_row += THREADS) {
-            float best = shared_values[local_row];
-            int best_index = shared_indices[local_row];
-#pragma unroll
-            for (int w = 1; w < WAVES_N; w++)
-                if (beats(shared_values[w * BM + local_row], shared_indices[w * BM + local_row], best, best_index)) {
-                    best = shared_values[w * BM + local_row];
-                    best_index = shared_indices[w * BM + local_row];
-                }
+        auto meet = [&](float other, int other_index) {
+            if (beats(other, other_index, best, best_index)) {
+                best = other;
+                best_index = other_index;
+            }
+        };
+        if constexpr (SHARE >= 2) meet(dpp_moved<0xB1>(best), __builtin_amdgcn_update_dpp(0, best_index, 0xB1, 0xf, 0xf, false));
+        if constexpr (SHARE >= 4) meet(dpp_moved<0x4E>(best), __builtin_amdgcn_update_dpp(0, best_index, 0x4E, 0xf, 0xf, false));
+        if constexpr (SHARE >= 8) meet(dpp_moved<0x141>(best), __builtin_amdgcn_update_dpp(0, best_index, 0x141, 0xf, 0xf, false));
+        if constexpr (SHARE >= 16) meet(dpp_moved<0x140>(best), __builtin_amdgcn_update_dpp(0, best_index, 0x140, 0xf, 0xf, false));
+        if (share == 0 && m0 + local_row < M) {
             size_t at = (size_t)(m0 + local_row) * best_out.per_row + blockIdx.x;
             best_out.values[at] = best;
             best_out.indices[at] = best_index;
