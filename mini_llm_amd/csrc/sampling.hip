@@ -178,7 +178,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 // follows the step). With `advance` the row's position and stored length grow by one, its cache row
 // of every group is looked up in the block table for the new position (-1 where the table has no page
 // there yet: the host brings the table before that step runs), and its token source becomes its own
-// slot. One block.
+// slot. A block takes 16 rows, a wave a row.
 struct StepGroups {
     const int* tables[4];
     int* slots[4];
@@ -186,6 +186,7 @@ struct StepGroups {
 };
 
 constexpr int CHOOSE_THREADS = 1024;
+constexpr int CHOOSE_ROWS = CHOOSE_THREADS / WAVE;  // rows a block takes: a wave a row
 
 __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
     const float* __restrict__ values, const int* __restrict__ indices, int per_row, int n_rows,
@@ -193,38 +194,36 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
     int* __restrict__ out_tokens, int* __restrict__ host_ring, int ring_rows, int ring_stride, int* __restrict__ cursor,
     int advance, int* __restrict__ positions, int* __restrict__ context_lens, int* __restrict__ token_sources,
     StepGroups groups) {
-    extern __shared__ int chosen[];  // [n_rows]
-    const int tid = threadIdx.x;
+    __shared__ int chosen[CHOOSE_ROWS];
+    const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int ring_row = cursor ? cursor[0] : 0;
     const int sequence = cursor ? cursor[1] : 0;
-    // A row's candidates are shared among the `group` lanes next to each other that take the row (a whole wave for
-    // few rows, down to four lanes for hundreds), and asked for eight at a time before any is compared: a candidate
-    // was written by some other compute unit and comes from memory.
-    int group = WAVE;
-    while (group > 4 && (CHOOSE_THREADS / group) < n_rows) group >>= 1;
-    const int in_group = tid % group, groups_in_block = CHOOSE_THREADS / group;
+    // A wave takes a row; its candidates are asked for eight a lane at a time before any is compared: a candidate was
+    // written by some other compute unit and comes from memory.
+    const int row = blockIdx.x * CHOOSE_ROWS + wave;
     constexpr int BATCH = 8;
-    for (int row = tid / group; row < n_rows; row += groups_in_block) {
+    if (row < n_rows) {
         float best = -INFINITY;
         int best_index = 0x7fffffff;
         const size_t base = (size_t)row * per_row;
-        for (int c0 = in_group; c0 < per_row; c0 += group * BATCH) {
+        for (int c0 = lane; c0 < per_row; c0 += WAVE * BATCH) {
             float value[BATCH];
             int index[BATCH];
 #pragma unroll
             for (int u = 0; u < BATCH; u++) {
-                int c = min(c0 + u * group, per_row - 1);
+                int c = min(c0 + u * WAVE, per_row - 1);
                 value[u] = values ? values[base + c] : 0.0f;
                 index[u] = indices[base + c];
             }
 #pragma unroll
             for (int u = 0; u < BATCH; u++)
-                if (c0 + u * group < per_row && beats(value[u], index[u], best, best_index)) {
+                if (c0 + u * WAVE < per_row && beats(value[u], index[u], best, best_index)) {
                     best = value[u];
                     best_index = index[u];
                 }
         }
-        for (int offset = group / 2; offset > 0; offset >>= 1) {
+#pragma unroll
+        for (int offset = WAVE / 2; offset > 0; offset >>= 1) {
             float other = __shfl_xor(best, offset, WAVE);
             int other_index = __shfl_xor(best_index, offset, WAVE);
             if (beats(other, other_index, best, best_index)) {
@@ -232,40 +231,47 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
                 best_index = other_index;
             }
         }
-        if (in_group == 0) chosen[row] = best_index;
+        if (lane == 0) chosen[wave] = best_index;
     }
     __syncthreads();
-    for (int row = tid; row < n_rows; row += CHOOSE_THREADS) {
+    if (tid < CHOOSE_ROWS && blockIdx.x * CHOOSE_ROWS + tid < n_rows) {   // the block's rows, a lane each: one store of their tokens
+        const int row = blockIdx.x * CHOOSE_ROWS + tid;
         const int slot = state_slots[row];
         const bool live = slot >= 0;
-        const int token = live ? chosen[row] : -1;
+        const int token = live ? chosen[tid] : -1;
         out_tokens[row] = token;
         if (host_ring) {
             host_ring[(size_t)ring_row * ring_stride + row] = token;
-            __threadfence_system();   // the token is in host memory before the row's number (below) can be
+            __threadfence_system();   // the token is in host memory before the block's number (below) can be
         }
-        if (!live) continue;
-        token_slots[slot] = token;
-        if (advance) {
-            const int position = positions[row] + 1;
-            positions[row] = position;
-            context_lens[row] = position;
-            token_sources[row] = slot;
-            const int block = position >> groups.page_shift, offset = position & ((1 << groups.page_shift) - 1);
-            for (int g = 0; g < groups.count; g++) {
-                int page = block < groups.table_width ? groups.tables[g][(size_t)row * groups.table_width + block] : -1;
-                groups.slots[g][row] = page >= 0 ? (page << groups.page_shift) + offset : -1;
+        if (live) {
+            token_slots[slot] = token;
+            if (advance) {
+                const int position = positions[row] + 1;
+                positions[row] = position;
+                context_lens[row] = position;
+                token_sources[row] = slot;
+                const int block = position >> groups.page_shift, offset = position & ((1 << groups.page_shift) - 1);
+                for (int g = 0; g < groups.count; g++) {
+                    int page = block < groups.table_width ? groups.tables[g][(size_t)row * groups.table_width + block] : -1;
+                    groups.slots[g][row] = page >= 0 ? (page << groups.page_shift) + offset : -1;
+                }
             }
         }
     }
     if (cursor) {
-        // The row's last entry says which step's tokens the row holds: whoever reads the ring on the host waits for
-        // that number instead of an event behind the step (which costs the device about 6 us between two steps).
+        // The row's last entries, one a block, say which step's tokens the row holds: whoever reads the ring on the
+        // host waits for that number in all of them instead of an event behind the step (which costs the device about
+        // 6 us between two steps). The block that finishes last moves the cursor on: every block has read it by then.
         __syncthreads();
         if (tid == 0) {
-            host_ring[(size_t)ring_row * ring_stride + ring_stride - 1] = sequence;
-            cursor[0] = (ring_row + 1) % ring_rows;   // every thread has read both before the first barrier
-            cursor[1] = (sequence + 1) & 0x3fffffff;
+            host_ring[(size_t)ring_row * ring_stride + ring_stride - 1 - blockIdx.x] = sequence;
+            const int arrived = atomicAdd(&cursor[2], 1);
+            if (arrived == (int)gridDim.x - 1) {
+                cursor[2] = 0;
+                cursor[0] = (ring_row + 1) % ring_rows;
+                cursor[1] = (sequence + 1) & 0x3fffffff;
+            }
         }
     }
 }
@@ -293,7 +299,8 @@ MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, i
                          int page_size, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_rows <= 8192 && per_row >= 1, "choose: bad sizes rows=%d candidates=%d", n_rows, per_row);
     MLLM_REQUIRE(indices && state_slots && token_slots && out_tokens, "choose: an operand is missing");
-    MLLM_REQUIRE(!host_ring || (ring_rows >= 1 && ring_stride >= n_rows + (cursor ? 1 : 0)), "choose: the ring's rows are shorter than the batch (and, with a cursor, one entry for the step's number)");
+    const int n_blocks = ceil_div(n_rows, CHOOSE_ROWS);
+    MLLM_REQUIRE(!host_ring || (ring_rows >= 1 && ring_stride >= n_rows + (cursor ? n_blocks : 0)), "choose: the ring's rows are shorter than the batch (and, with a cursor, an entry for each 16 rows' step number)");
     MLLM_REQUIRE(!cursor || host_ring, "choose: a cursor without a ring");
     StepGroups groups{};
     if (advance) {
@@ -311,7 +318,7 @@ MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, i
     }
     if (n_rows == 0) return 0;
     mllm_count_kernel(MLLM_K_CHOOSE);
-    choose_kernel<<<1, CHOOSE_THREADS, (size_t)n_rows * sizeof(int), stream>>>(
+    choose_kernel<<<n_blocks, CHOOSE_THREADS, 0, stream>>>(
         values, indices, per_row, n_rows, state_slots, token_slots, out_tokens, host_ring, ring_rows, ring_stride,
         cursor, advance, positions, context_lens, token_sources, groups);
     return mllm_check_launch("choose");

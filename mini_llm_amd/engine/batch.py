@@ -292,7 +292,7 @@ class DecodeBatchBuilder:
         lengths = [capacity] * 3 + [capacity + 1] + [capacity] * 4
         for _ in range(n_groups):
             lengths += [capacity * self.table_width, capacity]
-        lengths.append(2)   # for a step that chooses its tokens on the device: the row of the token ring it writes next, and its number
+        lengths.append(3)   # for a step that chooses its tokens on the device: the row of the token ring it writes next, its number, and a count that is zero between steps
         self.offsets, total = [], 0
         for n in lengths:
             self.offsets.append(total)
@@ -355,4 +355,4 @@ class DecodeBatchBuilder:
 
     def cursor_view(self, device_flat):
         at = self.offsets[8 + 2 * len(self.tables)]
-        return device_flat[at : at + 2]
+        return device_flat[at : at + 3]

@@ -45,9 +45,12 @@ class StepError(ValueError):
 
 
 # A decode step of many requests is one kernel bound by memory (attention over the cache) among six that wait for trips
-# to memory with most compute units idle. From so many requests on the captured step runs two halves of the requests
-# side by side (graph branches), so that one half's small kernels run under the other half's attention.
-DECODE_LANES_FROM = 32
+# to memory with most compute units idle. From so many requests on (0: never) the captured step runs groups of its
+# requests side by side, as branches of the graph, so that one group's small kernels run under another's attention.
+# Off by default: the branches do overlap on the device (128 rows: 0.98 against 1.06 ms a step), but launching a graph
+# with branches costs the host 4 to 5 us a kernel (0.78 ms for the 170 kernels of two groups), which at 64 and at 256
+# rows is more than the device needs for the step, and a host that also schedules has less to spare than that.
+DECODE_LANES_FROM = 0
 DECODE_LANE_ROWS = 64    # the most requests of a group (the kernels for few rows take up to 64)
 TOKEN_RING_ROWS = 8   # steps whose chosen tokens stay readable on the host after they were launched
 
@@ -58,11 +61,11 @@ class ChosenTokens:
     kernel writes the row itself, once the row's last entry shows the step's ``number`` (``tolist`` waits for either).
     A row is used again ``TOKEN_RING_ROWS`` steps later."""
 
-    __slots__ = ("device", "_host", "_n", "_event", "_number")
+    __slots__ = ("device", "_host", "_n", "_event", "_number", "_flags")
     WAIT_SECONDS = 30.0
 
-    def __init__(self, device, host, n, event=None, number=None):
-        self.device, self._host, self._n, self._event, self._number = device, host, n, event, number
+    def __init__(self, device, host, n, event=None, number=None, flags=1):
+        self.device, self._host, self._n, self._event, self._number, self._flags = device, host, n, event, number, flags
 
     def __len__(self):
         return self._n
@@ -75,11 +78,12 @@ class ChosenTokens:
         return self._host[: self._n].tolist()
 
     def _await_number(self) -> None:
-        """Spins on the row's last entry (written by the device behind the tokens, with a fence between); gives the
-        processor away between looks once the first few thousand have found nothing."""
+        """Spins on the row's last entries (each written by the device behind a share of the tokens, with a fence between);
+        gives the processor away between looks once the first few thousand have found nothing."""
         row, number = self._host, self._number
         looks, deadline = 0, None
-        while row[-1] != number:
+        flags = row[-self._flags:]
+        while (flags != number).any():
             looks += 1
             if looks > 2000:
                 time.sleep(0)
@@ -145,7 +149,10 @@ class _DecodeGraph:
         # from so many rows on the requests go through the layers in two groups side by side
         self.lanes = _Lanes(runner.device, max(2, capacity // DECODE_LANE_ROWS)) if runner.lanes_from and capacity >= runner.lanes_from else None
         if chooses:
-            self.ring = torch.full((TOKEN_RING_ROWS, capacity + 1), -1, dtype=torch.int32).pin_memory()
+            from ..ops import kernels
+
+            self.flags = kernels.choose_flags(capacity)
+            self.ring = torch.full((TOKEN_RING_ROWS, capacity + self.flags), -1, dtype=torch.int32).pin_memory()
             self.ring_rows = self.ring.numpy()   # the same memory, for the host's reads
             self.ring_at = 0        # the ring row the next step writes and that step's number: the host's count of the
             self.number = 0         # device's cursor
@@ -179,7 +186,7 @@ class _DecodeGraph:
                       and all(r is at[0] and r.table_changes == at[1] and r.length == at[2] for r, at in zip(records, stands)))
         if not carried_on:
             flat = self.builder.fill(entries)
-            self.builder.cursor[:] = (self.ring_at, self.number)
+            self.builder.cursor[:] = (self.ring_at, self.number, 0)
             runner.staging.upload(flat, into=self.buffer)
             self.uploads += 1
         batch = self.static_batch
@@ -188,7 +195,7 @@ class _DecodeGraph:
             choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True)
             self.graph, self.logits = _capture(runner, batch, choice, self.lanes)
         self.graph.replay()
-        chosen = ChosenTokens(self.logits[: len(entries)], self.ring_rows[self.ring_at], len(entries), number=self.number)
+        chosen = ChosenTokens(self.logits[: len(entries)], self.ring_rows[self.ring_at], len(entries), number=self.number, flags=self.flags)
         self.ring_at = (self.ring_at + 1) % TOKEN_RING_ROWS
         self.number = (self.number + 1) & 0x3FFFFFFF
         self.on_device = [(r, r.table_changes, r.length + 1) for r in records]

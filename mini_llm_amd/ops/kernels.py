@@ -504,13 +504,21 @@ class StepAdvance:
     page_size: int
 
 
+def choose_flags(rows: int) -> int:
+    """How many of a ring row's last entries ``choose`` sets to the step's number for a batch of so many rows (one for
+    every 16 rows: a block of the kernel)."""
+    return -(-int(rows) // 16)
+
+
 def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, cursor=None, advance: StepAdvance | None = None):
     """One token per row from its candidates: the best (value, index) pair by numpy's argmax rules (``values`` None: the
     smallest index; one candidate a row: that one). Rows whose ``state_slots`` entry is negative are padding and give -1. The
-    token of a live row also goes to token_slots[state_slots[row]] and, with ``host_ring`` (int32 [ring rows, > rows] in
-    page-locked host memory) to the ring row that ``cursor[0]`` names (``cursor``: int32 [2] on the device); the row's last
-    entry then gets the step's number ``cursor[1]``, and both move on by one (the row modulo the ring's rows, the number
-    modulo 2^30): a reader on the host that knows the number waits for it to appear, and needs no event.
+    token of a live row also goes to token_slots[state_slots[row]] and, with ``host_ring`` (int32 [ring rows, >= rows +
+    ``choose_flags(rows)``] in page-locked host memory) to the ring row that ``cursor[0]`` names (``cursor``: int32 [3] on
+    the device, its third entry zero); the row's last ``choose_flags(rows)`` entries then get the step's number
+    ``cursor[1]`` (one from each block of the kernel), and row and number move on by one (the row modulo the ring's
+    rows, the number modulo 2^30): a reader on the host that knows the number waits for it to appear in all of them,
+    and needs no event.
     ``advance``: see StepAdvance. Returns the tokens (int32 [rows], on the device)."""
     _device_tensor(indices, "indices", torch.int32, 2)
     rows, per_row = indices.shape
@@ -530,9 +538,9 @@ def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, 
         _require(isinstance(host_ring, torch.Tensor) and host_ring.dtype == torch.int32 and host_ring.dim() == 2 and host_ring.is_contiguous()
                  and host_ring.is_pinned(), "the ring must be a contiguous int32 matrix in page-locked host memory")
         ring_rows, ring_stride = host_ring.shape
-        _require(ring_stride >= rows + 1, "the ring's rows need an entry per row of the batch and one for the step's number")
+        _require(ring_stride >= rows + choose_flags(rows), "the ring's rows need an entry per row of the batch and choose_flags(rows) for the step's number")
         _device_tensor(cursor, "cursor", torch.int32, 1)
-        _require(cursor.shape[0] == 2, "the cursor is (ring row, step number)")
+        _require(cursor.shape[0] == 3, "the cursor is (ring row, step number, blocks that are through)")
     else:
         _require(cursor is None, "a cursor without a ring")
     tables = slots = None

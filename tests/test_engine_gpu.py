@@ -509,12 +509,12 @@ def test_queued_decoding_gives_the_same_tokens(model_dirs, engines):
 def test_queued_decoding_of_many_sequences_side_by_side_without_copies(model_dirs, dtype):
     # 40 sequences decode for 70 steps, queued: the captured step chooses its tokens itself and moves its batch on by
     # one token on the device, so between two steps nothing is copied to the device unless a sequence has reached a new
-    # page (all prompts have the same length here: every 16th step); from 32 rows on the step's requests go through the
-    # layers in two groups side by side. The tokens must be the plain implementation's.
+    # page (all prompts have the same length here: every 16th step); by option the step's requests go through the layers
+    # in two groups side by side (branches of the captured graph). The tokens must be the plain implementation's.
     from mini_llm_amd.engine.engine import Engine, EngineOptions
 
     folder, config, weights = model_dirs["A"]
-    engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=40, page_size=16))
+    engine = Engine(folder, EngineOptions(dtype=dtype, max_sessions=40, page_size=16, decode_lanes_from=32))
     prompts = [random_tokens(900 + i, 21, config["vocab_size"]) for i in range(40)]
     handles = [engine.try_take_cache() for _ in prompts]
     got = [[engine.prefill_greedy(h, p)] for h, p in zip(handles, prompts)]

@@ -1028,7 +1028,7 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
     tab_d, slot_d = [d(t) for t in tables], [d(np.full(rows, -5)) for _ in tables]
     last = torch.full((9,), -1, dtype=torch.int32, device=DEV)
     ring = torch.full((3, 8), -9, dtype=torch.int32).pin_memory()
-    cursor = d([2, 41])
+    cursor = d([2, 41, 0])
     advance = K.StepAdvance(pos_d, ctx_d, src_d, tab_d, slot_d, page)
     for turn in range(2):
         tokens = K.choose(None, d(indices), d(live), last, host_ring=ring, cursor=cursor, advance=advance)
@@ -1036,7 +1036,7 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
         want = np.where(live >= 0, indices[:, 0], -1)
         assert tokens.cpu().numpy().tolist() == want.tolist()
         ring_row = (2 + turn) % 3
-        assert ring[ring_row, :rows].tolist() == want.tolist() and cursor.cpu().tolist() == [(ring_row + 1) % 3, 42 + turn]
+        assert ring[ring_row, :rows].tolist() == want.tolist() and cursor.cpu().tolist() == [(ring_row + 1) % 3, 42 + turn, 0]
         assert ring[ring_row, 7].item() == 41 + turn          # the step's number, behind its tokens
         now = positions + (turn + 1) * (live >= 0)
         assert pos_d.cpu().numpy().tolist() == now.tolist() and ctx_d.cpu().numpy().tolist() == now.tolist()
@@ -1054,3 +1054,34 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
             assert slots.cpu().numpy().tolist() == expect
     assert last.cpu().numpy().tolist() == [indices[1, 0], -1, indices[3, 0], indices[0, 0], -1, -1, -1, indices[4, 0], -1]
     assert (ring[:, rows:7] == -9).all() and ring[1, 7].item() == -9
+
+
+def test_choose_over_several_blocks(K):
+    # more than 16 rows: a block of the kernel takes 16; each leaves the step's number in an entry of its own at the end
+    # of the ring row, and the block that finishes last moves the cursor
+    rng = np.random.default_rng(6)
+    rows, per_row, page = 40, 700, 16
+    values = rng.standard_normal((rows, per_row)).astype(np.float32)
+    indices = rng.permutation(rows * per_row).reshape(rows, per_row).astype(np.int32)
+    live = rng.permutation(64)[:rows].astype(np.int32)
+    live[[3, 17, 39]] = -1
+    positions = rng.integers(0, 60, rows).astype(np.int32)
+    table = rng.integers(0, 50, (rows, 4)).astype(np.int32)
+    d = lambda a: dev(a, torch.int32)
+    pos_d, ctx_d, src_d, slot_d = d(positions), d(positions), d(np.full(rows, -1)), d(np.full(rows, -5))
+    last = torch.full((64,), -1, dtype=torch.int32, device=DEV)
+    flags = K.choose_flags(rows)
+    assert flags == 3
+    ring = torch.full((4, rows + flags), -9, dtype=torch.int32).pin_memory()
+    cursor = d([1, 1000, 0])
+    want = np.where(live >= 0, indices[np.arange(rows), values.argmax(axis=1)], -1)
+    for turn in range(3):
+        tokens = K.choose(dev(values), d(indices), d(live), last, host_ring=ring, cursor=cursor,
+                          advance=K.StepAdvance(pos_d, ctx_d, src_d, [d(table)], [slot_d], page))
+        torch.cuda.synchronize()
+        assert tokens.cpu().numpy().tolist() == want.tolist()
+        ring_row = (1 + turn) % 4
+        assert ring[ring_row, :rows].tolist() == want.tolist() and ring[ring_row, rows:].tolist() == [1000 + turn] * 3
+        assert cursor.cpu().tolist() == [(ring_row + 1) % 4, 1001 + turn, 0]
+        assert pos_d.cpu().numpy().tolist() == (positions + (turn + 1) * (live >= 0)).tolist()
+    assert last.cpu().numpy()[live[live >= 0]].tolist() == want[live >= 0].tolist()
