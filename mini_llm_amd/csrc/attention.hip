@@ -755,19 +755,24 @@ MLLM_API int mllm_attention_prefill(const void* q, int q_stride, const void* k_p
 #define MLLM_PREFILL_CASE(T, PAD)                                                                                      \
     launch_prefill<T, PAD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,      \
                            max_blocks, n_requests, max_q_len, n_heads, n_kv_heads, head_size, page_shift, window, scale, stream)
-    if (dtype == MLLM_BF16 && prefill_stream::takes(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
-        // long portions in bfloat16, heads of 32 / 64 / 128, pages of 32 keys or more: keys and values stream from the pages straight into LDS
-#define MLLM_STREAM_CASE(HD)                                                                                            \
-    prefill_stream::launch<HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
-                               max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, stream)
-        const long table_reach = (long)max_blocks * page_size;
-        const int reach = (int)(max_len > 0 && max_len < table_reach ? max_len : (table_reach < (1 << 30) ? table_reach : (1 << 30)));
-        if (head_size == 32) MLLM_STREAM_CASE(32);
-        else if (head_size == 64) MLLM_STREAM_CASE(64);
-        else MLLM_STREAM_CASE(128);
-#undef MLLM_STREAM_CASE
+    const long table_reach = (long)max_blocks * page_size;
+    const int reach = (int)(max_len > 0 && max_len < table_reach ? max_len : (table_reach < (1 << 30) ? table_reach : (1 << 30)));
+#define MLLM_STREAM_CASE(T, HD)                                                                                            \
+    prefill_stream::launch<T, HD>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables,    \
+                                  max_blocks, n_requests, max_q_len, reach, n_heads, n_kv_heads, page_shift, window, scale, stream)
+    if (dtype == MLLM_BF16 && prefill_stream::takes<bf16_t>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+        // long portions, rows of 64 / 128 / 256 bytes, pages of 32 keys or more: keys and values stream from the pages straight into LDS
+        if (head_size == 32) MLLM_STREAM_CASE(bf16_t, 32);
+        else if (head_size == 64) MLLM_STREAM_CASE(bf16_t, 64);
+        else MLLM_STREAM_CASE(bf16_t, 128);
         return mllm_check_launch("attention_prefill");
     }
+    if (dtype == MLLM_F32 && prefill_stream::takes<float>(head_size, page_size, max_q_len, scale, q_stride, out_stride, q, out)) {
+        if (head_size == 32) MLLM_STREAM_CASE(float, 32);
+        else MLLM_STREAM_CASE(float, 64);
+        return mllm_check_launch("attention_prefill");
+    }
+#undef MLLM_STREAM_CASE
     if (dtype == MLLM_F32) {
         if (padded == 32) MLLM_PREFILL_CASE(float, 32);
         else if (padded == 64) MLLM_PREFILL_CASE(float, 64);

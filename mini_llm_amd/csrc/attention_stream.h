@@ -1,6 +1,9 @@
-// Prompt attention in bfloat16 for heads of 32, 64 or 128 over pages of at least 32 keys: key and value tiles stream
-// from the cache pages straight into LDS (global_load_lds_dwordx4), and a block's keys are divided among its waves.
-// Included by attention.hip.
+// Prompt attention for rows of 64, 128 or 256 bytes (bfloat16 heads of 32, 64 or 128; 32-bit heads of 32 or 64)
+// over pages of at least 32 keys: key and value tiles stream from the cache pages straight into LDS
+// (global_load_lds_dwordx4), and a block's keys are divided among its waves. Included by attention.hip.
+// The text below describes the bfloat16 kernel; what the 32-bit one does differently stands where it does it: the
+// 32-bit matrix instruction (32 x 32 x 2, four to a 16-byte piece of a key), the library's expf, and values read as
+// they are stored (the instruction takes single elements, so nothing has to be transposed).
 //
 // A block owns 64 queries of one (request, head). Each of its four waves holds all 64 queries and walks every fourth
 // tile of 32 keys with softmax statistics of its own; at the end the four partial results are combined through LDS.
@@ -113,36 +116,62 @@ __device__ __forceinline__ void read_transposed<4, 256>(const unsigned (&address
         : "memory");
 }
 
-template <int HD, int SPLITS>
+// Eight 4-byte LDS reads from one address with the offsets the 32-bit value product needs (keys 0-3 and 8-11 of a
+// lane's sixteen, ROW_BYTES apart; `FROM` 0: those, 1: keys 16-19 and 24-27), as instructions, for the reason above.
+// Returns when the values are in registers.
+template <int ROW_BYTES, int FROM>
+__device__ __forceinline__ void read_eight(unsigned address, float (&out)[8]) {
+    asm volatile(
+        "ds_read_b32 %0, %8 offset:%9\n\t"
+        "ds_read_b32 %1, %8 offset:%10\n\t"
+        "ds_read_b32 %2, %8 offset:%11\n\t"
+        "ds_read_b32 %3, %8 offset:%12\n\t"
+        "ds_read_b32 %4, %8 offset:%13\n\t"
+        "ds_read_b32 %5, %8 offset:%14\n\t"
+        "ds_read_b32 %6, %8 offset:%15\n\t"
+        "ds_read_b32 %7, %8 offset:%16\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(out[0]), "=&v"(out[1]), "=&v"(out[2]), "=&v"(out[3]), "=&v"(out[4]), "=&v"(out[5]), "=&v"(out[6]), "=&v"(out[7])
+        : "v"(address), "n"((16 * FROM + 0) * ROW_BYTES), "n"((16 * FROM + 1) * ROW_BYTES), "n"((16 * FROM + 2) * ROW_BYTES), "n"((16 * FROM + 3) * ROW_BYTES),
+          "n"((16 * FROM + 8) * ROW_BYTES), "n"((16 * FROM + 9) * ROW_BYTES), "n"((16 * FROM + 10) * ROW_BYTES), "n"((16 * FROM + 11) * ROW_BYTES)
+        : "memory");
+}
+
+template <typename T, int HD, int SPLITS>
 struct Layout {
-    static constexpr int PPR = HD / 8;              // 16-byte pieces per row
-    static constexpr int ROW_BYTES = HD * 2;
-    static constexpr int ROWS_PER_LOAD = 512 / HD;  // rows a wave's 1 KiB load covers
+    static constexpr bool FP32 = sizeof(T) == 4;
+    static constexpr int ROW_BYTES = HD * (int)sizeof(T);
+    static constexpr int PPR = ROW_BYTES / 16;      // 16-byte pieces per row
+    static constexpr int ROWS_PER_LOAD = 1024 / ROW_BYTES;  // rows a wave's 1 KiB load covers
     static constexpr int LOADS = KEYS / ROWS_PER_LOAD;  // loads per tile of keys (as many again for the values)
     static constexpr int TILE_BYTES = KEYS * ROW_BYTES;
     static constexpr int WAVE_BYTES = 4 * TILE_BYTES;   // two key tiles, two value tiles
     static constexpr int LDS_BYTES = SPLITS * WAVE_BYTES;
-    static_assert(HD == 32 || HD == 64 || HD == 128, "rows of 64, 128 or 256 bytes");
+    static_assert(ROW_BYTES == 64 || ROW_BYTES == 128 || ROW_BYTES == 256, "rows of 64, 128 or 256 bytes");
     static_assert(WAVE_BYTES >= 64 * HD * 4, "a wave's partial result (of up to 64 queries) takes the place of its tiles");
     // K: sixteen consecutive keys, the same piece: their 16-byte slots must differ modulo 256 bytes.
     static __device__ __forceinline__ int k_turn(int key) { return (key / (16 / PPR)) % PPR; }
     // V: four consecutive keys, the same 64 bytes of columns: their 64-byte slots must differ modulo 256 bytes.
-    static __device__ __forceinline__ int v_turn(int key) { return HD == 32 ? 0 : (HD == 64 ? ((key >> 1) & 1) * 4 : (key & 3) * 4); }
+    // (32-bit values are read a row's 128 consecutive bytes at a time: no turn needed)
+    static __device__ __forceinline__ int v_turn(int key) { return FP32 || ROW_BYTES == 64 ? 0 : (ROW_BYTES == 128 ? ((key >> 1) & 1) * 4 : (key & 3) * 4); }
 };
 
 // QUERIES: 64 queries a block (two sub-tiles of 32, both held by every wave), or 32 where that would leave compute units
 // without a block: what the kernel waits for is the wave with the most tiles, and a tile of 32 queries takes it half as long.
 // SPLITS: four waves a block, or eight where the portions reach far back: the kernel's time is the time of the wave with
 // the most tiles (it pays every tile's chain in full), which eight waves halve; a block then has a compute unit to itself.
-template <int HD, int QUERIES, int SPLITS>
-__global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) void attention_prefill_stream_kernel(
-    const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages,
-    bf16_t* __restrict__ out, int out_stride, const int* __restrict__ q_starts, const int* __restrict__ context_lens,
+template <typename T, int HD, int QUERIES, int SPLITS>
+__global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4) ? 2 : 1) void attention_prefill_stream_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    T* __restrict__ out, int out_stride, const int* __restrict__ q_starts, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads, int page_shift, int window, float scale) {
-    typedef Layout<HD, SPLITS> L;
+    typedef Layout<T, HD, SPLITS> L;
+    constexpr bool FP32 = L::FP32;
     constexpr int QSUB = QUERIES / 32;
     static_assert(QUERIES == 32 || QUERIES == 64, "one or two sub-tiles of queries");
-    constexpr int QSTEPS = HD / 16;  // k-steps of the score product
+    static_assert(HD % 32 == 0, "the output is written in tiles of 32 head dimensions");
+    constexpr int QSTEPS = L::PPR / 2;  // k-steps of the score product: a lane takes one 16-byte piece of its key in each
+    constexpr int PIECE = 16 / (int)sizeof(T);  // elements of a 16-byte piece
     constexpr int DT = HD / 32;      // 32-row tiles of the output's head dimension
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ float stats_lds[SPLITS][QUERIES][2];
@@ -169,9 +198,9 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
         // a lane beyond the portion's end takes the portion's first row and position -1: no key is at or before it, so every
         // score of it is masked (nothing waits for the rows here: the tiles are asked for while they are still on their way)
         q_position[qs] = q_local < q_len ? context + q_local : -1;
-        const bf16_t* q_row = q + (size_t)(q_first + (q_local < q_len ? q_local : 0)) * q_stride + head * HD;
+        const T* q_row = q + (size_t)(q_first + (q_local < q_len ? q_local : 0)) * q_stride + head * HD;
 #pragma unroll
-        for (int s = 0; s < QSTEPS; s++) q_reg[qs][s] = *reinterpret_cast<const Vec16*>(q_row + s * 16 + half * 8);
+        for (int s = 0; s < QSTEPS; s++) q_reg[qs][s] = *reinterpret_cast<const Vec16*>(q_row + (2 * s + half) * PIECE);
     }
 
     const int block_last_position = context + min(tile_q0 + QUERIES, q_len) - 1;
@@ -191,8 +220,8 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
 #pragma unroll
     for (int l = 0; l < L::LOADS; l++) {
         const int row = l * L::ROWS_PER_LOAD + lane / L::PPR, slot = lane % L::PPR;
-        k_lane[l] = (row * HD + (slot ^ L::k_turn(row)) * 8) * 2;
-        v_lane[l] = (row * HD + (slot ^ L::v_turn(row)) * 8) * 2;
+        k_lane[l] = row * L::ROW_BYTES + (slot ^ L::k_turn(row)) * 16;
+        v_lane[l] = row * L::ROW_BYTES + (slot ^ L::v_turn(row)) * 16;
     }
     auto issue = [&](int i, int page, bool is_value) {  // page: the one that holds the whole tile
         const int k_base = tile_base(i);
@@ -210,7 +239,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
             for (int l = 0; l < L::LOADS; l++) {
                 const int row = l * L::ROWS_PER_LOAD + lane / L::PPR, slot = lane % L::PPR;
                 const int piece = slot ^ (is_value ? L::v_turn(row) : L::k_turn(row));
-                const unsigned char* src = base + (min(row, last_row) * HD + piece * 8) * 2;
+                const unsigned char* src = base + min(row, last_row) * L::ROW_BYTES + piece * 16;
                 __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
                                                  (void __attribute__((address_space(3)))*)(place + l * 1024), 16, 0, 0);
             }
@@ -228,7 +257,22 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
 #pragma unroll
             for (int v = 0; v < 16; v++) acc_o[qs][i2][v] = 0.0f;
     }
-    const float score_scale = scale * 1.4426950408889634f;  // 2^x of a score prescaled by log2(e); positive, so it commutes with the maximum
+    // bfloat16: 2^x of a score prescaled by log2(e); 32-bit: the library's e^x of the scaled score. Positive either way, so
+    // the scaling commutes with the maximum.
+    const float score_scale = FP32 ? scale : scale * 1.4426950408889634f;
+    auto weight_of = [](float x) { return FP32 ? expf(x) : __builtin_amdgcn_exp2f(x); };
+    // one 16-byte piece of a key against the same piece of the queries: one product in bfloat16 (32 x 32 x 16), four in
+    // 32-bit (32 x 32 x 2: component c of every lane forms the pair of one product, the same pairing on both operands)
+    auto piece_product = [](const Vec16& k_piece, const Vec16& q_piece, f32x16 sums) {
+        if constexpr (FP32) {
+            const f32x4 k4 = *reinterpret_cast<const f32x4*>(&k_piece), q4 = *reinterpret_cast<const f32x4*>(&q_piece);
+#pragma unroll
+            for (int c = 0; c < 4; c++) sums = __builtin_amdgcn_mfma_f32_32x32x2f32(k4[c], q4[c], sums, 0, 0, 0);
+            return sums;
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&k_piece), *reinterpret_cast<const bf16x8*>(&q_piece), sums, 0, 0, 0);
+        }
+    };
 
     // K fragment (32 keys x 16 columns): lane l holds key l % 32, columns 16 s + 8 (l / 32) .. + 8
     // V^T fragment by two transposing reads: the sixteen lanes of group g = l / 16 point at keys k0 + (l % 16) / 4, columns
@@ -244,10 +288,9 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
             for (int v = 0; v < 16; v++) s_acc[qs][v] = 0.0f;
 #pragma unroll
         for (int s = 0; s < QSTEPS; s++) {
-            const bf16x8 k_frag = *reinterpret_cast<const bf16x8*>(k_tile + lane32 * L::ROW_BYTES + (((2 * s + half) ^ L::k_turn(lane32)) * 16));
+            const Vec16 k_frag = *reinterpret_cast<const Vec16*>(k_tile + lane32 * L::ROW_BYTES + (((2 * s + half) ^ L::k_turn(lane32)) * 16));
 #pragma unroll
-            for (int qs = 0; qs < QSUB; qs++)
-                s_acc[qs] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k_frag, *reinterpret_cast<const bf16x8*>(&q_reg[qs][s]), s_acc[qs], 0, 0, 0);
+            for (int qs = 0; qs < QSUB; qs++) s_acc[qs] = piece_product(k_frag, q_reg[qs][s], s_acc[qs]);
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
@@ -306,7 +349,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
             const float new_max = fmaxf(running_max[qs], tile_max);
             const float safe_max = new_max == -INFINITY ? 0.0f : new_max;  // a query with no key yet
             if (__any(new_max > running_max[qs])) {  // some query's maximum rose: what has been summed so far shrinks
-                const float rescale = __builtin_amdgcn_exp2f(running_max[qs] - safe_max);
+                const float rescale = weight_of(running_max[qs] - safe_max);
                 running_sum[qs] *= rescale;
 #pragma unroll
                 for (int i2 = 0; i2 < DT; i2++)
@@ -316,14 +359,16 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
             running_max[qs] = new_max;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qs][v], score_scale, -safe_max));
+                const float p = weight_of(__builtin_fmaf(s_acc[qs][v], score_scale, -safe_max));
                 s_acc[qs][v] = p;
                 running_sum[qs] += p;
             }
+            if constexpr (!FP32) {
 #pragma unroll
-            for (int slab = 0; slab < 2; slab++)
+                for (int slab = 0; slab < 2; slab++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) p[qs][slab][e] = static_cast<bf16_t>(s_acc[qs][8 * slab + e]);
+                    for (int e = 0; e < 8; e++) p[qs][slab][e] = static_cast<bf16_t>(s_acc[qs][8 * slab + e]);
+            }
         };
         softmax(0);
         __builtin_amdgcn_sched_barrier(0);
@@ -341,7 +386,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
 #pragma unroll
                     for (int v = 0; v < 16; v++) start[v] = 0.0f;
                 }
-                s_next[qs] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8*>(&k_frag[s]), *reinterpret_cast<const bf16x8*>(&q_reg[qs][s]), start, 0, 0, 0);
+                s_next[qs] = piece_product(*reinterpret_cast<const Vec16*>(&k_frag[s]), q_reg[qs][s], start);
             }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -349,6 +394,26 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
 
         // ---- O^T += V^T . P^T : two slabs of 16 keys; a lane's eight are keys 4 half .. + 4 and 8 + 4 half .. + 4 of the slab ----
         wait_vmcnt<3 * L::LOADS>();  // the newest three are K(i+2) V(i+1) K(i+3): V(i) has landed
+        if constexpr (FP32) {
+            // 32-bit: O^T += V^T . P^T by products of two keys: register v of the scores holds, in the lanes of half h, key
+            // 8 (v / 4) + 4 h + v % 4 of the tile, so product v takes that key's values (column 32 i2 + lane % 32, read as
+            // stored) against the register itself. Eight values a read, for each 32 columns.
+#pragma unroll
+            for (int i2 = 0; i2 < DT; i2++) {
+                const unsigned address = lds_address(v_tile + (4 * half) * L::ROW_BYTES + (i2 * 32 + lane32) * 4);
+                float values[8];
+                read_eight<L::ROW_BYTES, 0>(address, values);
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+#pragma unroll
+                    for (int qs = 0; qs < QSUB; qs++) acc_o[qs][i2] = __builtin_amdgcn_mfma_f32_32x32x2f32(values[e], s_acc[qs][e], acc_o[qs][i2], 0, 0, 0);
+                read_eight<L::ROW_BYTES, 1>(address, values);
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+#pragma unroll
+                    for (int qs = 0; qs < QSUB; qs++) acc_o[qs][i2] = __builtin_amdgcn_mfma_f32_32x32x2f32(values[e], s_acc[qs][8 + e], acc_o[qs][i2], 0, 0, 0);
+            }
+        } else {
         short4_t v_frag[DT][4];      // per 32 columns: slab 0 low keys, slab 0 high keys, slab 1 low, slab 1 high
         {
             unsigned address[DT];
@@ -371,6 +436,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
 #pragma unroll
                 for (int qs = 0; qs < QSUB; qs++) acc_o[qs][i2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fragment, p[qs][slab], acc_o[qs][i2], 0, 0, 0);
             }
+        }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         issue(i + 2, page_v, true);
@@ -409,78 +475,89 @@ __global__ __launch_bounds__(64 * SPLITS, (HD <= 64 && SPLITS == 4) ? 2 : 1) voi
         float weight[SPLITS], total = 0.0f;
 #pragma unroll
         for (int w = 0; w < SPLITS; w++) {
-            weight[w] = __builtin_amdgcn_exp2f(stats_lds[w][qs * 32 + lane32][0] - best);  // a wave that saw no key: 2^-inf = 0
+            weight[w] = weight_of(stats_lds[w][qs * 32 + lane32][0] - best);  // a wave that saw no key: a weight of 0
             total += weight[w] * stats_lds[w][qs * 32 + lane32][1];
         }
         const float inverse = 1.0f / total;
-        bf16_t* out_row = out + (size_t)(q_first + q_local) * out_stride + head * HD + i2 * 32;
+        T* out_row = out + (size_t)(q_first + q_local) * out_stride + head * HD + i2 * 32;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            bf16x4 o;
+            float o[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 float sum = 0.0f;
 #pragma unroll
                 for (int w = 0; w < SPLITS; w++)
                     sum += weight[w] * reinterpret_cast<const float*>(lds + w * L::WAVE_BYTES)[(share * 16 + 4 * g + e) * WAVE + lane];
-                o[e] = static_cast<bf16_t>(sum * inverse);
+                o[e] = sum * inverse;
             }
-            *reinterpret_cast<bf16x4*>(out_row + 8 * g + 4 * half) = o;
+            if constexpr (FP32) *reinterpret_cast<f32x4*>(out_row + 8 * g + 4 * half) = f32x4{o[0], o[1], o[2], o[3]};
+            else *reinterpret_cast<bf16x4*>(out_row + 8 * g + 4 * half) = bf16x4{static_cast<bf16_t>(o[0]), static_cast<bf16_t>(o[1]), static_cast<bf16_t>(o[2]), static_cast<bf16_t>(o[3])};
         }
     }
 }
 
-// Whether prompt portions with these sizes take this kernel (bfloat16 only; the caller checks the type).
+// Whether prompt portions with these sizes take this kernel.
+template <typename T>
 inline bool takes(int head_size, int page_size, int max_q_len, float scale, int q_stride, int out_stride, const void* q, const void* out) {
-    if (head_size != 32 && head_size != 64 && head_size != 128) return false;
+    const int row_bytes = head_size * (int)sizeof(T);
+    if (row_bytes != 64 && row_bytes != 128 && row_bytes != 256) return false;
+    if (head_size < 32) return false;    // the output's rows are tiles of 32 head dimensions
     if (page_size < KEYS) return false;  // a tile of keys lies in one page (page sizes are powers of two)
     if (max_q_len <= 64) return false;   // shorter portions: the kernel with fewer queries a block
     if (!(scale > 0.0f)) return false;   // the maximum is taken before the scaling
-    // 16-byte loads of q and 8-byte stores of out
-    return q_stride % 8 == 0 && out_stride % 4 == 0 && ((size_t)q) % 16 == 0 && ((size_t)out) % 8 == 0;
+    // 16-byte loads of q and 8- or 16-byte stores of out
+    return (q_stride * sizeof(T)) % 16 == 0 && (out_stride * sizeof(T)) % (4 * sizeof(T)) == 0 && ((size_t)q) % 16 == 0 && ((size_t)out) % (4 * sizeof(T)) == 0;
 }
 
-template <int HD, int QUERIES, int SPLITS>
+template <typename T, int HD, int QUERIES, int SPLITS>
 void launch_queries(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
                     const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int n_heads, int n_kv_heads,
                     int page_shift, int window, float scale, hipStream_t stream) {
-    constexpr int LDS_BYTES = Layout<HD, SPLITS>::LDS_BYTES;
+    constexpr int LDS_BYTES = Layout<T, HD, SPLITS>::LDS_BYTES;
     static bool raised = false;  // per instantiation: the limit on dynamic LDS is a property of the kernel
     if (!raised && LDS_BYTES > 60 * 1024)  // (if this fails the launch below fails too, and the entry point reports that)
-        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<HD, QUERIES, SPLITS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
+        raised = hipFuncSetAttribute((const void*)attention_prefill_stream_kernel<T, HD, QUERIES, SPLITS>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
     // x: (request, head), so that with a multiple of eight heads the blocks of one head share an XCD's L2; y: tiles of queries
     dim3 grid(n_heads * n_requests, ceil_div(max_q_len, QUERIES));
     mllm_count_kernel(MLLM_K_ATTENTION_PREFILL_STREAM);
-    attention_prefill_stream_kernel<HD, QUERIES, SPLITS><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, (bf16_t*)out, out_stride, q_starts, context_lens,
+    attention_prefill_stream_kernel<T, HD, QUERIES, SPLITS><<<grid, 64 * SPLITS, LDS_BYTES, stream>>>(
+        (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_starts, context_lens,
         block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale);
 }
 
-template <int HD>
+template <typename T, int HD>
 void launch(const void* q, int q_stride, const void* k_pages, const void* v_pages, void* out, int out_stride, const int* q_starts,
             const int* context_lens, const int* block_tables, int max_blocks, int n_requests, int max_q_len, int max_len, int n_heads,
             int n_kv_heads, int page_shift, int window, float scale, hipStream_t stream) {
-#define MLLM_STREAM_LAUNCH(QUERIES, SPLITS)                                                                                              \
-    launch_queries<HD, QUERIES, SPLITS>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, \
-                                        n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
-    // blocks of 64 queries where they give every compute unit a block (measured: 2 x 1,024 tokens x 12 heads 15.9 against 17.2 us),
-    // else of 32 (4 x 128 tokens on 896 cached: 9.7 against 13.0 us; 512 on 7,680: 46.7 against 66.0 us)
-    const bool wide = (long)n_heads * n_requests * ceil_div(max_q_len, 64) >= 256;
-    // Eight waves a block where the block of the last queries has sixteen tiles of keys or more to walk (max_len: the longest
-    // sequence after this step, or what bounds it; a window bounds the keys too) AND every block still finds a compute
-    // unit of its own at once (eight waves' tiles leave room for one block a unit): a long context with few queries.
-    // Measured, heads of 64: 512 queries on 7,680 cached keys 38.2 against 46.7 us with four waves; but two prompts of 1,024
-    // tokens (384 blocks: a second round) 19.1 against 15.9 us, one of 4,096 64.8 against 57 us.
-    const int reach = window > 0 ? min(max_len, window + 64) : max_len;
-    const long blocks = (long)n_heads * n_requests * ceil_div(max_q_len, wide ? 64 : 32);
-    bool eight = false;
-    if constexpr (HD <= 64) {  // (eight waves' tiles of a head of 128 do not fit a compute unit's LDS)
-        eight = reach >= 16 * KEYS && blocks <= 256;
-        if (wide && eight) MLLM_STREAM_LAUNCH(64, 8);
-        else if (eight) MLLM_STREAM_LAUNCH(32, 8);
+#define MLLM_STREAM_LAUNCH(QUERIES, SPLITS)                                                                                                 \
+    launch_queries<T, HD, QUERIES, SPLITS>(q, q_stride, k_pages, v_pages, out, out_stride, q_starts, context_lens, block_tables, max_blocks, \
+                                           n_requests, max_q_len, n_heads, n_kv_heads, page_shift, window, scale, stream)
+    if constexpr (sizeof(T) == 4) {
+        // 32-bit: the matrix cores are what a wave waits for (a tile of 32 keys is 96 products of 64 cycles for 32 queries),
+        // so blocks of 32 queries, which the compute units take in turn, the ones with the most keys first
+        // (blocks of 64 queries: 59.2 against 62.1 us for two prompts of 1,024 tokens x 12 heads of 64, 35.0 against 32.2 us for eight of 256)
+        MLLM_STREAM_LAUNCH(32, 4);
+    } else {
+        // blocks of 64 queries where they give every compute unit a block (measured: 2 x 1,024 tokens x 12 heads 15.9 against 17.2 us),
+        // else of 32 (4 x 128 tokens on 896 cached: 9.7 against 13.0 us; 512 on 7,680: 46.7 against 66.0 us)
+        const bool wide = (long)n_heads * n_requests * ceil_div(max_q_len, 64) >= 256;
+        // Eight waves a block where the block of the last queries has sixteen tiles of keys or more to walk (max_len: the longest
+        // sequence after this step, or what bounds it; a window bounds the keys too) AND every block still finds a compute
+        // unit of its own at once (eight waves' tiles leave room for one block a unit): a long context with few queries.
+        // Measured, heads of 64: 512 queries on 7,680 cached keys 38.2 against 46.7 us with four waves; but two prompts of 1,024
+        // tokens (384 blocks: a second round) 19.1 against 15.9 us, one of 4,096 64.8 against 57 us.
+        const int reach = window > 0 ? min(max_len, window + 64) : max_len;
+        const long blocks = (long)n_heads * n_requests * ceil_div(max_q_len, wide ? 64 : 32);
+        bool eight = false;
+        if constexpr (HD * sizeof(T) <= 128) {  // (eight waves' tiles of rows of 256 bytes do not fit a compute unit's LDS)
+            eight = reach >= 16 * KEYS && blocks <= 256;
+            if (wide && eight) MLLM_STREAM_LAUNCH(64, 8);
+            else if (eight) MLLM_STREAM_LAUNCH(32, 8);
+        }
+        if (wide && !eight) MLLM_STREAM_LAUNCH(64, 4);
+        else if (!eight) MLLM_STREAM_LAUNCH(32, 4);
     }
-    if (wide && !eight) MLLM_STREAM_LAUNCH(64, 4);
-    else if (!eight) MLLM_STREAM_LAUNCH(32, 4);
 #undef MLLM_STREAM_LAUNCH
 }
 

@@ -403,7 +403,7 @@ def test_a_step_takes_the_kernels_it_is_meant_to(tmp_path, dtype):
         assert sum(decode_step.values()) == 2 * layers + 3
     else:
         assert prompt_step.get("gemm_tiled") == 4 * layers + 1 and "gemm_stream" not in prompt_step, prompt_step
-        assert prompt_step.get("attention_prefill") == layers, prompt_step
+        assert prompt_step.get("attention_prefill_stream") == layers and "attention_prefill" not in prompt_step, prompt_step
         # the separate kernels: norm, q/k/v with the cache write, attention, output product cut along K, norm taking its
         # partial products, up product, down product cut along K; the final norm takes the last partial products
         assert decode_step == {"embed": 1, "layernorm": 1, "pending_layernorm": 2 * layers, "gemm_skinny": 4 * layers,
