@@ -570,7 +570,7 @@ def main() -> int:
                 "tokens": 8}
 
     record = {
-        "metric": f"decode tokens/s at batch {args.batch}, GPT-2 {args.shape}, {args.prompt_len}-token prompts decoding towards 1024",
+        "metric": f"decode tokens/s at batch {args.batch}, GPT-2 {args.shape}, {args.prompt_len}-token prompts decoding towards {CONTEXT}",
         "value": round(args.batch * args.steps / seconds, 1),
         "unit": "tokens/s",
         "n_gpus": 1,

@@ -339,7 +339,9 @@ class DecodeBatchBuilder:
         self.filled = n
         return self.flat
 
-    def batch(self, device_flat, entries) -> StepBatch:
+    def batch(self, device_flat, entries, reach: int | None = None) -> StepBatch:
+        """``reach``: the longest sequence, after the step, of any batch that will lie in these views (None: the
+        cache's own limit)."""
         views = [device_flat[o : o + n] for o, n in zip(self.offsets, self.lengths)]
         n_groups = len(self.tables)
         groups = [GroupStepData(block_tables=views[8 + 2 * g].reshape(self.capacity, self.table_width), slots=views[9 + 2 * g])
@@ -347,7 +349,7 @@ class DecodeBatchBuilder:
         return StepBatch(
             n_tokens=self.capacity, n_requests=self.capacity, n_logit_rows=self.capacity, max_q_len=1,
             short_requests=self.capacity, short_rows=self.capacity,
-            max_total_len=self.cache.max_length, tokens=views[0], positions=views[1], token_request=views[2],
+            max_total_len=self.cache.max_length if reach is None else reach, tokens=views[0], positions=views[1], token_request=views[2],
             q_starts=views[3], context_lens=views[4], state_slots=views[5], logit_rows=views[6], token_sources=views[7],
             logit_slots=views[5],  # every request has one logit row, in its own place
             groups=groups, request_ids=[e.request_id for e in entries], host={},

@@ -137,13 +137,13 @@ class _DecodeGraph:
     of the same requests, each taking its token from its last-token slot, is replayed without anything being copied to
     the device before it or from the device after it: the tokens arrive in a ring of rows in page-locked host memory."""
 
-    def __init__(self, runner: "ModelRunner", capacity: int, chooses: bool = False):
+    def __init__(self, runner: "ModelRunner", capacity: int, chooses: bool = False, reach: int | None = None):
         import torch
 
         self.runner, self.capacity, self.chooses = runner, capacity, chooses
         self.builder = DecodeBatchBuilder(runner.cache, capacity)
         self.buffer = torch.zeros(len(self.builder.flat), dtype=torch.int32, device=runner.device)
-        self.static_batch = self.builder.batch(self.buffer, [])
+        self.static_batch = self.builder.batch(self.buffer, [], reach)
         self.graph = None
         self.logits = None
         # from so many rows on the requests go through the layers in two groups side by side
@@ -282,6 +282,7 @@ class ModelRunner:
         self.last_batch: StepBatch | None = None
         self.use_graphs = bool(use_graphs and device is not None and cache.max_length is not None and model.all_graph_safe())
         self._graphs: dict = {}
+        self._decode_reaches = [r for r in model.decode_reaches() if cache.max_length is not None and r < cache.max_length]
         self._portion_graphs: OrderedDict = OrderedDict()   # shape of batch -> _PortionGraph, least recently used first
         self._shapes_seen: dict = {}                         # shape of batch -> how often it has come
         self.portion_graph_after = PORTION_GRAPH_AFTER if portion_graph_after is None else int(portion_graph_after)
@@ -373,9 +374,15 @@ class ModelRunner:
         if len(entries) > GRAPH_BUCKETS[-1]:
             return None
         capacity = next(b for b in GRAPH_BUCKETS if b >= len(entries))
-        if (capacity, choose) not in self._graphs:
-            self._graphs[capacity, choose] = _DecodeGraph(self, capacity, chooses=choose)
-        return self._graphs[capacity, choose]
+        # the range of sequence lengths the step falls in, where the model's kernels differ between ranges
+        reach = self.cache.max_length
+        if self._decode_reaches:
+            longest = max(self.cache.length(e.request_id) for e in entries) + 1
+            reach = next((r for r in self._decode_reaches if r >= longest), reach)
+        key = (capacity, choose, reach)
+        if key not in self._graphs:
+            self._graphs[key] = _DecodeGraph(self, capacity, chooses=choose, reach=reach)
+        return self._graphs[key]
 
     def _portion_graph_for(self, entries):
         """The captured step for batches of this shape, once the shape has come often enough."""

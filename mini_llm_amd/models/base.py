@@ -95,6 +95,11 @@ class Model(Part):
         limits = [limit for limit in (block.mixer_part().short_portion for block in self.blocks) if limit is not None]
         return min(limits) if limits else 1
 
+    def decode_reaches(self) -> list[int]:
+        """The sequence lengths at which some mixer decodes through other kernels, ascending: the engine keeps a
+        captured decode step for each range between them."""
+        return sorted({int(reach) for block in self.blocks for reach in block.mixer_part().decode_reaches})
+
     def cache_groups(self) -> list[CacheGroupSpec]:
         groups: dict = {}
         for call in self.schedule:

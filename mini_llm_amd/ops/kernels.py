@@ -589,6 +589,19 @@ MLP_SLICE_UNITS = 64         # hidden units a block of the feed-forward kernel t
 LAYER_KERNEL_MAX_ROWS = 64   # more rows than this go through the separate kernels
 
 
+# The longest sequence that the two layer kernels decode, for up to four rows and for more: a block of the attention half
+# walks all keys of its (row, head) alone, which past some 1,000 keys takes longer than the kernels it saves, the kernel
+# that spreads a row's keys over many blocks among them. Measured in steps of 12 layers at GPT-2 small's sizes, layer
+# kernels against separate kernels: 1 row 383 : 390 us at 500 keys, 459 : 442 at 1,200, 569 : 490 at 2,000; 8 rows
+# 396 : 439, 455 : 487, 571 : 539, and 817 : 665 at 3,800; 16 rows 413 : 468 at 500, 613 : 612 at 2,000. (The feed-forward
+# half changes with the attention half: alone beside the separate attention kernels it is 15 us a step behind them.)
+DECODE_LAYER_REACHES = (1024, 1792)
+
+
+def decode_layer_reach(rows: int) -> int:
+    return DECODE_LAYER_REACHES[0] if rows <= 4 else DECODE_LAYER_REACHES[1]
+
+
 _layer_kernel_rows: dict = {}
 
 

@@ -27,6 +27,7 @@ MAX_HEAD_SIZE = 256
 class CausalSelfAttention(Mixer):
     graph_safe = True
     short_portion = kernels.DECODE_MAX_Q_LEN   # what the split-key kernel takes
+    decode_reaches = kernels.DECODE_LAYER_REACHES
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int | None = None, head_size: int | None = None,
                  window: int | None = None, out_std: float = 0.02, qkv_name: str = "c_attn.", out_name: str = "c_proj."):
@@ -82,8 +83,9 @@ class CausalSelfAttention(Mixer):
         return self.out.forward_pending(mixed, residual)
 
     def forward_normed(self, hidden, norm, compute_dtype, ctx: LayerContext):
-        # rows that are each the newest token of their request: the whole chain in one kernel
-        if (ctx.batch.max_q_len == 1 and hidden.shape[0] <= kernels.layer_kernel_rows(self.width) and isinstance(norm, LayerNorm)
+        # rows that are each the newest token of their request: the whole chain in one kernel, while a block of it can
+        # walk a row's keys alone (past that the kernel that spreads a row's keys over many blocks is worth its company)
+        if (ctx.batch.max_q_len == 1 and ctx.batch.max_total_len <= kernels.decode_layer_reach(hidden.shape[0]) and hidden.shape[0] <= kernels.layer_kernel_rows(self.width) and isinstance(norm, LayerNorm)
                 and isinstance(self.qkv.weight, kernels.PackedMatrix) and isinstance(self.out.weight, kernels.PackedMatrix)
                 and self.qkv.weight.dtype == torch.bfloat16 and ctx.k_pages.dtype == torch.bfloat16
                 and kernels.decode_layer_supported(self.width, self.head_size, ctx.k_pages.shape[2])):

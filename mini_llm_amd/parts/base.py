@@ -116,6 +116,9 @@ class Mixer(Part):
     # Portions up to so many tokens this mixer runs through a kernel of their own, apart from longer
     # ones (None: it makes no difference): the batch lays such portions out first.
     short_portion: int | None = None
+    # Sequence lengths at which this mixer's kernels for decoding change: a captured decode step is made for each range
+    # between them, and learns the range's end as the longest sequence of its batch (StepBatch.max_total_len).
+    decode_reaches: tuple = ()
 
     def kv_need(self) -> KVNeed | None:
         return None

@@ -33,6 +33,7 @@ class DenseMLP(FeedForward):
     def forward_normed(self, hidden, norm, compute_dtype, ctx):
         # few rows: the whole chain in one kernel, cut along the hidden units
         if (hidden.shape[0] <= kernels.layer_kernel_rows(self.width) and ctx.batch.max_q_len == 1 and isinstance(norm, LayerNorm)
+                and ctx.batch.max_total_len <= kernels.decode_layer_reach(hidden.shape[0])   # changes with the attention half
                 and isinstance(self.up.weight, kernels.PackedMatrix) and isinstance(self.down.weight, kernels.PackedMatrix)
                 and self.up.weight.dtype == torch.bfloat16 and kernels.decode_layer_supported(self.width, inner=self.inner)):
             return kernels.decode_mlp_half(hidden, norm.weight, norm.bias, norm.eps, self.up.weight, self.up.bias,

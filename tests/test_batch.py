@@ -90,6 +90,9 @@ def test_hot_shapes_beyond_the_kept_graphs_are_not_captured_at_every_turn():
         def all_graph_safe(self):
             return True
 
+        def decode_reaches(self):
+            return []
+
     groups = [CacheGroupSpec("full", (0,), 2, 16, None)]
     cache = CacheManager(groups, {}, num_pages=8, page_size=16, max_requests=4, max_length=64)
     runner = ModelRunner(NoModel(), cache, None, portion_graph_after=2)

@@ -412,6 +412,58 @@ def test_a_step_takes_the_kernels_it_is_meant_to(tmp_path, dtype):
     engine.close()
 
 
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_decoding_changes_kernels_where_the_sequences_grow_long(model_dirs, monkeypatch, use_graphs):
+    # Past a length that the mixer names, a decode step runs its attention through the separate kernels instead of the
+    # layer kernel (whose block walks all keys of a row alone); a captured step is kept for either range. The length is
+    # brought down to 48 here so that two requests cross it one after the other, and every step is checked against the
+    # plain implementation; the tokens a choosing step leaves are the argmax of those logits.
+    import replay
+    from mini_llm_amd.engine import StepEntry
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.ops import kernels
+    from mini_llm_amd.parts.attention import CausalSelfAttention
+
+    monkeypatch.setattr(kernels, "DECODE_LAYER_REACHES", (48, 48))
+    monkeypatch.setattr(CausalSelfAttention, "decode_reaches", (48,))
+    folder, config, weights = model_dirs["A"]
+    seqs = {"a": random_tokens(7, 70, config["vocab_size"]), "b": random_tokens(8, 62, config["vocab_size"])}
+    ref = replay.plain_logits(config, weights, seqs, bf16=True)
+    tol = replay.tolerance("bfloat16")
+    engine = Engine(folder, EngineOptions(dtype="bfloat16", max_sessions=4, use_graphs=use_graphs))
+    handles = {name: engine.try_take_cache() for name in seqs}
+    engine.runner.step([StepEntry(handles["a"], seqs["a"][:40], []), StepEntry(handles["b"], seqs["b"][:32], [])])
+    fed = {"a": 40, "b": 32}
+    kinds = []
+    for i in range(30):
+        before = kernels.launch_counts()
+        entries = [StepEntry(handles[name], [seqs[name][fed[name]]], [0]) for name in seqs]
+        logits = engine.runner.step(entries).cpu().numpy()
+        kinds.append("decode_attention_half" in kernels.launches_since(before))
+        for row, name in zip(logits, seqs):
+            np.testing.assert_allclose(row, ref[name][fed[name]], err_msg=f"{name} {fed[name]}", **tol)
+            fed[name] += 1
+    if use_graphs:
+        assert sorted(key[2] for key in engine.runner._graphs) == [48, config["n_positions"]]
+    else:  # a's newest token is the 41st..70th: the first eight steps stay within 48
+        assert kinds == [True] * 8 + [False] * 22
+    # the same through steps that choose their tokens: from a's 45th token on, across the change
+    for name in seqs:
+        engine.release_cache(handles[name])
+        handles[name] = engine.try_take_cache()
+    first = engine.runner.step([StepEntry(handles["a"], seqs["a"][:44], [43]), StepEntry(handles["b"], seqs["b"][:36], [35])], choose=True)
+    chosen = [first.tolist()]
+    for _ in range(9):
+        chosen.append(engine.runner.step([StepEntry(handles[name], [0], [0], from_slot=True) for name in seqs], choose=True).tolist())
+    rounded = plain_gpt2.bf16_weights(weights)
+    for j, (name, start) in enumerate((("a", 44), ("b", 36))):
+        tokens = list(seqs[name][:start])
+        for step in chosen:
+            plain_check_greedy(config, rounded, tokens, [step[j]], margin=0.03, stored=plain_gpt2.stored_as_bf16)
+            tokens.append(step[j])
+    engine.close()
+
+
 def test_no_garbage_collection_while_a_step_is_captured():
     # the collector may finalise another engine's captured graphs, and giving memory back inside a capture aborts the
     # process: it is off from the start of a capture to its end, and as it was again afterwards
@@ -526,7 +578,7 @@ def test_queued_decoding_of_many_sequences_side_by_side_without_copies(model_dir
             g.append(t)
     for g, t in zip(got, engine.take()):
         g.append(t)
-    graph = engine.runner._graphs[64, True]
+    graph, = [g for key, g in engine.runner._graphs.items() if key[:2] == (64, True)]
     assert graph.lanes is not None and len(graph.lanes.cuts(64)) == 2
     assert engine.runner.graph_steps == steps and graph.uploads <= 2 + steps // 16, graph.uploads
     rounded = plain_gpt2.bf16_weights(weights) if dtype == "bfloat16" else None
