@@ -183,13 +183,16 @@ constexpr int DECODE_MAX_SPLITS = 16;
 // A block per (token, head); its waves (blockDim.x / 64 of them, a power of two up to 16) split
 // the token's keys evenly among themselves, and their partial results meet in LDS.
 // TOGETHER: how a wave starts (see there); the host chooses.
+// parts (gridDim.z) > 1: few tokens with many keys, where a block per (token, head) would leave most of the chip idle.
+// The token's keys are cut into so many runs, a block each, and a block leaves its unnormalised sums with their maximum
+// and weight in `parts_out` ([token, head, part, HD + 2] floats) for attention_decode_merge_kernel instead of writing `out`.
 template <typename T, int HD, bool TOGETHER>
 __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int page_shift, int window, float scale, int out_packed) {
+    int page_shift, int window, float scale, int out_packed, float* __restrict__ parts_out) {
     constexpr int VEC = KeySweep<T, HD>::VEC, LPR = KeySweep<T, HD>::LPR, RPI = KeySweep<T, HD>::RPI;
     __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
 
@@ -201,19 +204,27 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     auto out_at = [&](int d) -> T* {
         return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
     };
-    if (request < 0) {  // a padding row; the whole block leaves together
-        for (int d = threadIdx.x; d < HD; d += blockDim.x) *out_at(d) = from_float<T>(0.0f);
+    const int n_parts = gridDim.z, part = blockIdx.z;
+    if (request < 0) {  // a padding row; the whole block leaves together (the merge writes its zeros where there are parts)
+        if (n_parts == 1)
+            for (int d = threadIdx.x; d < HD; d += blockDim.x) *out_at(d) = from_float<T>(0.0f);
         return;
     }
     const int position = positions[token];
-    const int first_key = window > 0 ? max(0, position - window + 1) : 0;
-    const int n_keys = position + 1 - first_key;
+    constexpr int KPI = KeySweep<T, HD>::KPI;
+    int first_key = window > 0 ? max(0, position - window + 1) : 0;
+    int last_key = position + 1;  // exclusive
+    if (n_parts > 1) {  // this block's run of the keys, in whole rounds of the sweep
+        const int run = (((last_key - first_key + n_parts - 1) / n_parts + KPI - 1) / KPI) * KPI;
+        first_key = min(first_key + part * run, last_key);
+        last_key = min(last_key, first_key + run);
+    }
+    const int n_keys = last_key - first_key;
     // keys per wave: whole rounds of the sweep (a round asks for KPI keys whether it needs them or
     // not), so that a wave either has a full round to do or none
-    constexpr int KPI = KeySweep<T, HD>::KPI;
     const int chunk = (((n_keys + n_splits - 1) / n_splits + KPI - 1) / KPI) * KPI;
     const int begin = first_key + split * chunk;
-    const int end = min(position + 1, begin + chunk);  // exclusive
+    const int end = min(last_key, begin + chunk);  // exclusive
     const int sub = lane % LPR;
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
@@ -273,7 +284,20 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     float total_max = -INFINITY;
     for (int s = 0; s < n_splits; s++) total_max = fmaxf(total_max, partial[s][HD]);
     float total = 0.0f;
-    for (int s = 0; s < n_splits; s++) total += partial[s][HD + 1] * expf(partial[s][HD] - total_max);
+    for (int s = 0; s < n_splits; s++) total += total_max == -INFINITY ? 0.0f : partial[s][HD + 1] * expf(partial[s][HD] - total_max);
+    if (n_parts > 1) {  // a run without keys (a short sequence in a launch cut for long ones) leaves max -inf and weight 0
+        float* mine = parts_out + (((size_t)token * n_heads + head) * n_parts + part) * (HD + 2);
+        for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+            float value = 0.0f;
+            for (int s = 0; s < n_splits; s++) value += total_max == -INFINITY ? 0.0f : partial[s][d] * expf(partial[s][HD] - total_max);
+            mine[d] = value;
+        }
+        if (threadIdx.x == 0) {
+            mine[HD] = total_max;
+            mine[HD + 1] = total;
+        }
+        return;
+    }
     float inverse = 1.0f / total;
     for (int d = threadIdx.x; d < HD; d += blockDim.x) {
         float value = 0.0f;
@@ -282,12 +306,39 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     }
 }
 
+// The runs of one (token, head) put together: out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M). A wave per (token, head).
+template <typename T, int HD>
+__global__ __launch_bounds__(WAVE) void attention_decode_merge_kernel(
+    const float* __restrict__ parts, int n_parts, T* __restrict__ out, int out_stride,
+    const int* __restrict__ token_request, int n_heads, int out_packed) {
+    const int head = blockIdx.x, token = blockIdx.y, lane = threadIdx.x;
+    auto out_at = [&](int d) -> T* {
+        return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
+    };
+    if (token_request[token] < 0) {
+        for (int d = lane; d < HD; d += WAVE) *out_at(d) = from_float<T>(0.0f);
+        return;
+    }
+    const float* mine = parts + ((size_t)token * n_heads + head) * n_parts * (HD + 2);
+    float total_max = -INFINITY;
+    for (int p = 0; p < n_parts; p++) total_max = fmaxf(total_max, mine[p * (HD + 2) + HD]);
+    float total = 0.0f;
+    for (int p = 0; p < n_parts; p++) total += mine[p * (HD + 2) + HD + 1] * expf(mine[p * (HD + 2) + HD] - total_max);
+    const float inverse = 1.0f / total;
+    for (int d = lane; d < HD; d += WAVE) {
+        float value = 0.0f;
+        for (int p = 0; p < n_parts; p++) value += mine[p * (HD + 2) + d] * expf(mine[p * (HD + 2) + HD] - total_max);
+        *out_at(d) = from_float<T>(value * inverse);
+    }
+}
+
 template <typename T>
 int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                     void* out, int out_stride, const int* token_request, const int* positions,
                     const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
-                    int page_shift, int window, float scale, int n_splits, int out_packed, hipStream_t stream) {
-    dim3 grid(n_heads, n_tokens), block(WAVE * n_splits);
+                    int page_shift, int window, float scale, int n_splits, int out_packed, int n_parts, float* parts,
+                    hipStream_t stream) {
+    dim3 grid(n_heads, n_tokens, n_parts), block(WAVE * n_splits);
     // Measured on MI355X: starting with query and pages together (and, in bfloat16, the pages a
     // round ahead) is 3 to 15 % faster wherever a wave has few rounds, which is where a kernel's
     // start counts; in 32-bit it takes twice the registers, and over the many rounds of long
@@ -295,7 +346,7 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
     // order is 5 % faster.
     const int reach = max_blocks << page_shift;
     const int keys_per_round = (sizeof(T) == 2 ? 4096 : 2048) / head_size;  // KeySweep's KPI
-    const int rounds = ceil_div(ceil_div(window > 0 && window < reach ? window : reach, n_splits), keys_per_round);
+    const int rounds = ceil_div(ceil_div(window > 0 && window < reach ? window : reach, n_splits * n_parts), keys_per_round);
     const bool together = sizeof(T) == 2 || rounds <= 12;
 #define MLLM_DECODE_CASE(HD)                                                                                   \
     case HD:                                                                                                   \
@@ -303,11 +354,16 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
         if (together)                                                                                          \
             attention_decode_kernel<T, HD, true><<<grid, block, 0, stream>>>(                                  \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts);  \
         else                                                                                                   \
             attention_decode_kernel<T, HD, false><<<grid, block, 0, stream>>>(                                 \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed);  \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts);  \
+        if (n_parts > 1) {                                                                                     \
+            mllm_count_kernel(MLLM_K_ATTENTION_DECODE_MERGE);                                                  \
+            attention_decode_merge_kernel<T, HD><<<dim3(n_heads, n_tokens), WAVE, 0, stream>>>(                \
+                parts, n_parts, (T*)out, out_stride, token_request, n_heads, out_packed);                      \
+        }                                                                                                      \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
@@ -333,7 +389,7 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    void* out, int out_stride, const int* token_request, const int* positions,
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
-                                   int n_splits, int dtype, int out_packed, hipStream_t stream) {
+                                   int n_splits, int dtype, int out_packed, int n_parts, float* parts, hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
@@ -343,16 +399,18 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                  "attention_decode: %d splits is not a power of two in 1..%d", n_splits, DECODE_MAX_SPLITS);
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_decode: rows are too short for the heads");
     MLLM_REQUIRE(n_tokens <= 65535, "attention_decode: too many tokens for one launch");
+    // parts: the keys of a token in so many runs, a block each; `parts` then holds n_tokens * n_heads * n_parts * (head_size + 2) floats
+    MLLM_REQUIRE(n_parts >= 1 && n_parts <= 64 && (n_parts == 1 || parts != nullptr), "attention_decode: %d parts (1..64, with memory for them)", n_parts);
     if (n_tokens == 0) return 0;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) page_shift++;
     int refused = 1;
     if (dtype == MLLM_F32)
         refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, stream);
+                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, stream);
     else
         refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, stream);
+                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, stream);
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }

@@ -351,11 +351,28 @@ def linear_qkv_cache(x, weight, bias, k_pages, v_pages, slots, n_heads, n_kv_hea
     return q
 
 
+_units: dict = {}
+
+
+def _compute_units(device) -> int:
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _units:
+        _units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _units[index]
+
+
 DECODE_MAX_Q_LEN = 8        # portions up to this many tokens take the split-key kernel
 DECODE_TARGET_WAVES = 4096  # the most waves a launch should have: 16 to each of 256 compute units are resident at once (measured: a
                             # second round of blocks costs more than longer shares of the keys per wave)
 DECODE_MIN_SPLIT = 64       # keys a wave should at least have
 DECODE_MAX_SPLITS = 16      # waves per block
+DECODE_MAX_PARTS = 64       # runs a token's keys are cut into at most, a block each, where (token, head) pairs are few
+# What such a run should at least hold. Measured on MI355X with heads of 64: up to some 32 pairs (a single token) runs
+# of 512 keys pay (12 pairs, 3,000 keys: 15.3 -> 12.4 us in bfloat16, 23.2 -> 15.1 in 32-bit; 32 pairs with heads of
+# 128, 8,000 keys: 76.8 -> 33.5 us); around 100 pairs only runs of 4 KiB a head dimension do, which is 1,024 keys in
+# 32-bit (3,900 keys: 53.7 -> 42.3 us) and 2,048 in bfloat16 (where two runs of 1,000 cost 2 us more than one of 2,000).
+DECODE_MIN_PART_FEW = 512
+DECODE_MIN_PART_BYTES = 4096
 
 
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
@@ -413,16 +430,27 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         # waves per block as keep the launch within what is resident at once, never more than one
         # per 64 keys of reach
         reach = block_tables.shape[1] * page_size if max_len is None else max(1, min(max_len, block_tables.shape[1] * page_size))
+        if window:
+            reach = min(reach, int(window))
+        # few tokens with many keys: a token's keys in several runs, a block each, so that the blocks are about as many
+        # as the chip has compute units, and a second small kernel that puts the runs together
+        n_parts, units = 1, _compute_units(q.device)
+        min_part = DECODE_MIN_PART_FEW if 8 * n * n_heads <= units else DECODE_MIN_PART_BYTES // q.element_size()
+        while n_parts < DECODE_MAX_PARTS and 2 * n * n_heads * n_parts <= units and 2 * n_parts * min_part <= reach:
+            n_parts *= 2
+        part_reach = -(-reach // n_parts)
         n_splits = 1
-        while n_splits < DECODE_MAX_SPLITS and 2 * n * n_heads * n_splits <= DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < reach:
+        while n_splits < DECODE_MAX_SPLITS and 2 * n * n_heads * n_parts * n_splits <= DECODE_TARGET_WAVES and n_splits * DECODE_MIN_SPLIT < part_reach:
             n_splits *= 2
         result = out
         if packed_out:
             result = empty_packed_rows(n, width, q.dtype, q.device)
             out = result.data
+        parts = torch.empty((n, n_heads, n_parts, head_size + 2), dtype=torch.float32, device=q.device) if n_parts > 1 else None
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
                                         _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
-                                        head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out), _stream()))
+                                        head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out),
+                                        n_parts, _ptr(parts), _stream()))
         return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):

@@ -402,6 +402,56 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize(
+    "n_heads,n_kv_heads,head_size,page_size,window,lengths,min_part",
+    [(12, 12, 64, 64, 0, (1500,), None),                 # one token, 1,500 keys: two runs by the kernel's own rule
+     (4, 2, 32, 16, 0, (700, 3, 260), 64),               # three tokens, one with 3 keys: most of its runs are empty
+     (3, 3, 128, 32, 300, (900, 450), 32),               # a window: the runs cut the window, not the sequence
+     (1, 1, 16, 16, 0, (1100, 1), 16),                   # a head of 16: a round of the sweep is 256 keys
+     (5, 5, 256, 64, 0, (520,), 64)],
+)
+def test_decode_attention_with_the_keys_in_runs(K, monkeypatch, dtype, n_heads, n_kv_heads, head_size, page_size, window, lengths, min_part):
+    # Few tokens with many keys: each token's keys are cut into runs, a block each, and a second kernel puts the runs
+    # together. One far key stands out in each sequence, in a run other than the last where there are several.
+    if min_part is not None:
+        monkeypatch.setattr(K, "DECODE_MIN_PART_FEW", min_part)
+        monkeypatch.setattr(K, "DECODE_MIN_PART_BYTES", min_part * (2 if dtype == torch.bfloat16 else 4))
+    rng = np.random.default_rng(head_size + len(lengths))
+    rnd = lambda *s: bf16_round(rng.standard_normal(s)) if dtype == torch.bfloat16 else rng.standard_normal(s).astype(np.float32).astype(np.float64)
+    n_blocks = [(n + page_size - 1) // page_size for n in lengths]
+    order = rng.permutation(sum(n_blocks) + 3).tolist()
+    kp = torch.full((len(order), n_kv_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
+    vp = torch.full_like(kp, float("nan"))
+    tables = np.zeros((len(lengths) + 1, max(n_blocks)), dtype=np.int32)
+    q_rows, refs = [], []
+    for r, total in enumerate(lengths):
+        k_all, v_all = rnd(total, n_kv_heads * head_size), rnd(total, n_kv_heads * head_size)
+        q = rnd(1, n_heads * head_size)
+        stands_out = min(total - 1, max(0, total - 1 - (window - 5 if window else total - 2)))   # the second key, or one near the window's far edge
+        far = q[0].reshape(n_heads, head_size)[:: n_heads // n_kv_heads].reshape(-1) * 3
+        k_all[stands_out] = bf16_round(far) if dtype == torch.bfloat16 else far
+        pages = [order.pop() for _ in range(n_blocks[r])]
+        tables[r + 1, : len(pages)] = pages     # row 0 of the tables belongs to nobody
+        slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+        K.cache_write(dev(k_all, dtype), dev(v_all, dtype), kp, vp, dev(slots, torch.int32), n_kv_heads, head_size)
+        q_rows.append(q)
+        refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_kv_heads, window or None))
+    # a padding row between the tokens
+    q_rows.insert(1, np.zeros((1, n_heads * head_size)))
+    refs.insert(1, np.zeros((1, n_heads * head_size)))
+    treq = [1, -1] + list(range(2, len(lengths) + 1))
+    tpos = [lengths[0] - 1, 0] + [n - 1 for n in lengths[1:]]
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    for packed_out in (False, True):
+        before = K.launch_counts()
+        out = K.paged_attention(
+            dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+            n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=1, max_len=max(lengths), packed_out=packed_out)
+        assert K.launches_since(before) == {"attention_decode": 1, "attention_decode_merge": 1}
+        np.testing.assert_allclose(unpacked(out) if packed_out else host(out), np.concatenate(refs), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize(
     "n_heads,n_kv_heads,head_size,page_size,window",
     [(3, 3, 32, 16, 0), (2, 2, 64, 64, 0), (4, 2, 64, 16, 150), (2, 1, 128, 8, 0), (2, 2, 128, 256, 0), (3, 3, 32, 32, 70),
      (2, 2, 48, 32, 0), (5, 5, 64, 4, 0)],
