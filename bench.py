@@ -227,7 +227,7 @@ def reps_of_a_step() -> int:
     return 5
 
 
-def measure_kernels(engine, batch: int = 8, context: int = 776):
+def measure_kernels(engine, batch: int = 8, context: int = 776, decode: bool = True):
     """What the kernels that a step's time goes to take inside the step and reach of their own roofline
     (``kernel_times_inside_a_step``): for a 2,048-token prompt step the four products of a layer and the prompt
     attention (flops / time / the matrix cores' peak), for a greedy decode step of ``batch`` sequences at ``context``
@@ -281,6 +281,8 @@ def measure_kernels(engine, batch: int = 8, context: int = 776):
         out["prefill_norms"] = {"us": round(norm_1 + norm_2, 2)}
     else:
         out["prefill_step"]["by_entry_point"] = _by_entry_point(names, each)
+    if not decode:
+        return out
 
     # --- a greedy decode step: ``batch`` sequences that hold ``context`` tokens each (the replays of the whole step move
     # the sequences on by a token each, and must stay on the page the step has reserved)
@@ -555,7 +557,7 @@ def main() -> int:
     engine = make_engine(args.dtype)
     checked = None if args.no_check else check_before_timing(engine, host_weights())
     if args.prefill_only:
-        emit({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}, args.json)
+        emit({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype, "kernels": measure_kernels(engine, decode=False)}, args.json)
         return 0
     seconds, step_bytes = DecodeBench(engine, args.batch, args.prompt_len).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
