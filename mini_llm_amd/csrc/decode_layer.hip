@@ -768,6 +768,25 @@ __device__ __forceinline__ f32x4 pending_piece(const PendingSum& in, int row_ind
     return value;
 }
 
+// The share of group `group` of `n_groups` in those four columns: the partial rows group, group + n_groups, ..., and with
+// group 0 the base row and the bias.
+__device__ __forceinline__ f32x4 pending_piece_share(const PendingSum& in, int row_index, int width, int piece, int group, int n_groups) {
+    f32x4 value = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (group == 0) {
+        value = load4(in.base + (size_t)row_index * width + 4 * piece);
+        if (in.bias) value += load4(in.bias + 4 * piece);
+    }
+    for (int s0 = group; s0 < in.n_partials; s0 += 8 * n_groups) {
+        f32x4 part[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            part[u] = load4(in.partials + ((size_t)min(s0 + u * n_groups, in.n_partials - 1) * in.rows + row_index) * width + 4 * piece);
+#pragma unroll
+        for (int u = 0; u < 8; u++) value += part[u] * (s0 + u * n_groups < in.n_partials ? 1.0f : 0.0f);
+    }
+    return value;
+}
+
 // out = base + bias + the partial rows: the pending stream as plain rows, for whatever does not
 // take it pending. grid (pieces of 256 x 4 columns, rows).
 __global__ __launch_bounds__(256) void pending_sum_kernel(PendingSum in, float* __restrict__ out, int width) {
@@ -776,21 +795,36 @@ __global__ __launch_bounds__(256) void pending_sum_kernel(PendingSum in, float* 
     *reinterpret_cast<f32x4*>(out + (size_t)row_index * width + 4 * piece) = pending_piece(in, row_index, width, piece);
 }
 
-// Row LayerNorm of pending rows (the sums are taken on the way in): a block of four waves a row,
-// the row kept in LDS; row_index, if given, names the pending row of each output row. Centred, in
-// 32-bit, like the norm of plain rows (elementwise.hip).
-template <typename OutT>
-__global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, const int* __restrict__ row_index,
-                                                                const float* __restrict__ gamma, const float* __restrict__ beta,
-                                                                OutT* __restrict__ out, float* __restrict__ summed, int width,
-                                                                float eps, int packed_out) {
-    extern __shared__ f32x4 row_pieces[];  // width / 4
-    __shared__ float red[2][4];
+// Row LayerNorm of pending rows (the sums are taken on the way in): a block a row, the row kept in LDS; row_index, if
+// given, names the pending row of each output row. Centred, in 32-bit, like the norm of plain rows (elementwise.hip).
+// GROUPS > 1 (a row of many partial rows, few of them in a launch: the rows a decode step's last layer leaves for the
+// final norm): the block's threads in so many groups of `group_lanes`, each of which adds up every GROUPS-th partial row,
+// all asked for at once; their shares meet in LDS, in a fixed order.
+template <typename OutT, int GROUPS>
+__global__ __launch_bounds__(GROUPS == 1 ? 256 : 1024) void pending_layernorm_kernel(
+    PendingSum in, const int* __restrict__ row_index, const float* __restrict__ gamma, const float* __restrict__ beta,
+    OutT* __restrict__ out, float* __restrict__ summed, int width, float eps, int packed_out, int group_lanes) {
+    constexpr int THREADS = GROUPS == 1 ? 256 : 1024, WAVES = THREADS / WAVE;
+    extern __shared__ f32x4 row_pieces[];  // width / 4, and behind them GROUPS x width / 4 for the groups' shares
+    __shared__ float red[2][WAVES];
     const int tid = threadIdx.x, n_pieces = width / 4;
     const int source = row_index ? row_index[blockIdx.x] : blockIdx.x;
+    if constexpr (GROUPS > 1) {
+        const int group = tid / group_lanes, piece = tid % group_lanes;
+        if (group < GROUPS && piece < n_pieces)
+            row_pieces[(1 + group) * n_pieces + piece] = pending_piece_share(in, source, width, piece, group, GROUPS);
+        __syncthreads();
+    }
     float sum = 0.0f;
-    for (int piece = tid; piece < n_pieces; piece += 256) {
-        f32x4 value = pending_piece(in, source, width, piece);
+    for (int piece = tid; piece < n_pieces; piece += THREADS) {
+        f32x4 value;
+        if constexpr (GROUPS > 1) {
+            value = row_pieces[n_pieces + piece];
+#pragma unroll
+            for (int g = 1; g < GROUPS; g++) value += row_pieces[(1 + g) * n_pieces + piece];
+        } else {
+            value = pending_piece(in, source, width, piece);
+        }
         row_pieces[piece] = value;
         if (summed) *reinterpret_cast<f32x4*>(summed + (size_t)blockIdx.x * width + 4 * piece) = value;  // the row with its sums taken
         sum += (value[0] + value[1]) + (value[2] + value[3]);
@@ -799,17 +833,23 @@ __global__ __launch_bounds__(256) void pending_layernorm_kernel(PendingSum in, c
     if (tid % WAVE == 0) red[0][tid / WAVE] = sum;
     __syncthreads();
     const float n = (float)width;
-    const float mean = ((red[0][0] + red[0][1]) + (red[0][2] + red[0][3])) / n;
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; w += 4) total += (red[0][w] + red[0][w + 1]) + (red[0][w + 2] + red[0][w + 3]);
+    const float mean = total / n;
     float squares = 0.0f;
-    for (int piece = tid; piece < n_pieces; piece += 256) {
+    for (int piece = tid; piece < n_pieces; piece += THREADS) {
         f32x4 d = row_pieces[piece] - mean;
         squares += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
     }
     squares = wave_total(squares);
     if (tid % WAVE == 0) red[1][tid / WAVE] = squares;
     __syncthreads();
-    const float inverse_stddev = 1.0f / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / n + eps);
-    for (int piece = tid; piece < n_pieces; piece += 256) {
+    total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; w += 4) total += (red[1][w] + red[1][w + 1]) + (red[1][w + 2] + red[1][w + 3]);
+    const float inverse_stddev = 1.0f / sqrtf(total / n + eps);
+    for (int piece = tid; piece < n_pieces; piece += THREADS) {
         f32x4 y = (row_pieces[piece] - mean) * inverse_stddev * load4(gamma + 4 * piece) + load4(beta + 4 * piece);
         // four consecutive columns lie together in the packed layout too (inside one 16-byte piece)
         OutT* at = out + (packed_out ? packed_element<OutT>(blockIdx.x, 4 * piece, width) : (size_t)blockIdx.x * width + 4 * piece);
@@ -969,13 +1009,23 @@ MLLM_API int mllm_pending_layernorm(const float* base, const float* partials, co
     MLLM_REQUIRE(n_rows >= 0 && pending_rows >= 0 && eps > 0.0f, "pending_layernorm: bad sizes");
     if (n_rows == 0) return 0;
     PendingSum in{base, partials, pending_bias, n_partials, pending_rows};
-    const size_t lds = (size_t)width * 4;
     mllm_count_kernel(MLLM_K_PENDING_LAYERNORM);
-    if (out_dtype == MLLM_F32)
-        pending_layernorm_kernel<float><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (float*)out, summed, width, eps, packed_out);
-    else if (out_dtype == MLLM_BF16)
-        pending_layernorm_kernel<bf16_t><<<n_rows, 256, lds, stream>>>(in, row_index, gamma, beta, (bf16_t*)out, summed, width, eps, packed_out);
-    else
+    // Many partial rows to a row and few rows (the final norm of a decode step behind the feed-forward half's 48 slices): four
+    // groups of threads take every fourth partial row each. Where the rows are many the compute units are busy as it is.
+    const int group_lanes = (width / 4 + WAVE - 1) / WAVE * WAVE;
+    const bool grouped = n_partials >= 16 && n_rows <= 64 && 4 * group_lanes <= 1024;
+#define MLLM_PENDING_NORM(OutT)                                                                                              \
+    if (grouped)                                                                                                             \
+        pending_layernorm_kernel<OutT, 4><<<n_rows, 1024, (size_t)width * 4 * 5, stream>>>(in, row_index, gamma, beta, (OutT*)out, summed, width, eps, packed_out, group_lanes); \
+    else                                                                                                                     \
+        pending_layernorm_kernel<OutT, 1><<<n_rows, 256, (size_t)width * 4, stream>>>(in, row_index, gamma, beta, (OutT*)out, summed, width, eps, packed_out, group_lanes);
+    if (out_dtype == MLLM_F32) {
+        MLLM_PENDING_NORM(float)
+    } else if (out_dtype == MLLM_BF16) {
+        MLLM_PENDING_NORM(bf16_t)
+    } else {
         MLLM_REQUIRE(false, "pending_layernorm: unknown output dtype %d", out_dtype);
+    }
+#undef MLLM_PENDING_NORM
     return mllm_check_launch("pending_layernorm");
 }

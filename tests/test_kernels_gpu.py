@@ -939,7 +939,9 @@ def test_layer_kernels_refuse_what_they_do_not_take(K):
 
 
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,width,n_partials,with_bias", [(1, 64, 0, False), (5, 96, 3, True), (9, 768, 48, True), (3, 1032, 17, False), (2, 2500, 9, True)])
+@pytest.mark.parametrize("rows,width,n_partials,with_bias", [(1, 64, 0, False), (5, 96, 3, True), (9, 768, 48, True), (3, 1032, 17, False), (2, 2500, 9, True),
+                                                            # few rows of many partial rows each: groups of threads share a row's sums
+                                                            (4, 1000, 33, True), (7, 64, 16, False), (64, 1024, 21, True), (65, 768, 48, False)])
 def test_layernorm_of_pending_rows(K, out_dtype, rows, width, n_partials, with_bias):
     # the sums are taken on the way into the norm; row_index picks and repeats rows
     rng = np.random.default_rng(rows + width)
