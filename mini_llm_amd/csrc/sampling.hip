@@ -177,8 +177,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 // memory (one store of the whole row by the first lanes: the host reads it after the event that
 // follows the step). With `advance` the row's position and stored length grow by one, its cache row
 // of every group is looked up in the block table for the new position (-1 where the table has no page
-// there yet: the host brings the table before that step runs), and its token source becomes its own
-// slot. A block takes 16 rows, a wave a row.
+// there yet: the host brings the table before that step runs), its token source becomes its own
+// slot, and its entry of draw_counts (if given: how many tokens the row's request has drawn, which the
+// sampler's random numbers are a function of) grows by one. A block takes 16 rows, a wave a row.
 struct StepGroups {
     const int* tables[4];
     int* slots[4];
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
     const int* __restrict__ state_slots, int* __restrict__ token_slots,
     int* __restrict__ out_tokens, int* __restrict__ host_ring, int ring_rows, int ring_stride, int* __restrict__ cursor,
     int advance, int* __restrict__ positions, int* __restrict__ context_lens, int* __restrict__ token_sources,
-    StepGroups groups) {
+    int* __restrict__ draw_counts, StepGroups groups) {
     __shared__ int chosen[CHOOSE_ROWS];
     const int tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
     const int ring_row = cursor ? cursor[0] : 0;
@@ -251,6 +252,7 @@ __global__ __launch_bounds__(CHOOSE_THREADS) void choose_kernel(
                 positions[row] = position;
                 context_lens[row] = position;
                 token_sources[row] = slot;
+                if (draw_counts) draw_counts[row] += 1;   // a sampled row's next draw is its request's next one
                 const int block = position >> groups.page_shift, offset = position & ((1 << groups.page_shift) - 1);
                 for (int g = 0; g < groups.count; g++) {
                     int page = block < groups.table_width ? groups.tables[g][(size_t)row * groups.table_width + block] : -1;
@@ -295,7 +297,7 @@ MLLM_API int mllm_sample(const float* logits, int n_rows, int vocab, const float
 MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, int n_rows,
                          const int* state_slots, int* token_slots, int* out_tokens, int* host_ring, int ring_rows,
                          int ring_stride, int* cursor, int advance, int* positions, int* context_lens, int* token_sources,
-                         const int* const* group_tables, int* const* group_slots, int n_groups, int table_width,
+                         int* draw_counts, const int* const* group_tables, int* const* group_slots, int n_groups, int table_width,
                          int page_size, hipStream_t stream) {
     MLLM_REQUIRE(n_rows >= 0 && n_rows <= 8192 && per_row >= 1, "choose: bad sizes rows=%d candidates=%d", n_rows, per_row);
     MLLM_REQUIRE(indices && state_slots && token_slots && out_tokens, "choose: an operand is missing");
@@ -320,6 +322,6 @@ MLLM_API int mllm_choose(const float* values, const int* indices, int per_row, i
     mllm_count_kernel(MLLM_K_CHOOSE);
     choose_kernel<<<n_blocks, CHOOSE_THREADS, 0, stream>>>(
         values, indices, per_row, n_rows, state_slots, token_slots, out_tokens, host_ring, ring_rows, ring_stride,
-        cursor, advance, positions, context_lens, token_sources, groups);
+        cursor, advance, positions, context_lens, token_sources, advance ? draw_counts : nullptr, groups);
     return mllm_check_launch("choose");
 }

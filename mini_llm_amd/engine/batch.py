@@ -285,7 +285,9 @@ class DecodeBatchBuilder:
     arrays are kept and only the rows of the live requests are rewritten, so a step costs a short
     loop instead of a dozen array constructions."""
 
-    def __init__(self, cache, capacity: int):
+    def __init__(self, cache, capacity: int, draws: bool = False):
+        """``draws``: the step also draws its tokens on the device (temperature, top-p): room for each row's seed,
+        temperature, nucleus mass and count of tokens drawn so far."""
         self.cache, self.capacity = cache, capacity
         self.table_width = cache.max_blocks()
         n_groups = len(cache.groups)
@@ -293,6 +295,8 @@ class DecodeBatchBuilder:
         for _ in range(n_groups):
             lengths += [capacity * self.table_width, capacity]
         lengths.append(3)   # for a step that chooses its tokens on the device: the row of the token ring it writes next, its number, and a count that is zero between steps
+        if draws:
+            lengths += [2 * capacity, capacity, capacity, capacity]   # seeds (64-bit), temperatures, nucleus masses (32-bit floats), counts
         self.offsets, total = [], 0
         for n in lengths:
             self.offsets.append(total)
@@ -305,7 +309,30 @@ class DecodeBatchBuilder:
         self.tables = [view(8 + 2 * g).reshape(capacity, self.table_width) for g in range(n_groups)]
         self.slots = [view(9 + 2 * g) for g in range(n_groups)]
         self.cursor = view(8 + 2 * n_groups)
+        self.draws = draws
+        if draws:
+            at = 9 + 2 * n_groups
+            self.seeds, self.temperatures, self.top_ps = view(at).view(np.int64), view(at + 1).view(np.float32), view(at + 2).view(np.float32)
+            self.draw_counts = view(at + 3)
         self.filled = capacity  # rows that held a request in the previous step (all, so the first fill pads all)
+
+    def fill_draws(self, sampling, counts) -> None:
+        """How each row draws its token (objects with temperature, top_p and seed; a temperature of 0 or less: greedily)
+        and how many tokens its request has drawn so far. Padding rows draw greedily."""
+        n = len(sampling)
+        self.seeds[:n] = [p.seed & 0x7FFFFFFFFFFFFFFF for p in sampling]
+        self.temperatures[:n] = [max(p.temperature, 0.0) for p in sampling]
+        self.top_ps[:n] = [p.top_p for p in sampling]
+        self.draw_counts[:n] = counts
+        self.seeds[n:], self.temperatures[n:], self.top_ps[n:], self.draw_counts[n:] = 0, 0.0, 1.0, 0
+
+    def draw_views(self, device_flat):
+        """(seeds int64, temperatures, top_ps float32, counts int32) as views of the buffer on the device."""
+        import torch
+
+        at = 9 + 2 * len(self.tables)
+        section = lambda i: device_flat[self.offsets[at + i] : self.offsets[at + i] + self.lengths[at + i]]
+        return section(0).view(torch.int64), section(1).view(torch.float32), section(2).view(torch.float32), section(3)
 
     def fill(self, entries) -> np.ndarray:
         n, cache, page = len(entries), self.cache, self.cache.page_size

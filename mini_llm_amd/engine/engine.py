@@ -91,17 +91,8 @@ class _Executor:
     def launch(self, entries, sampling, steps):
         engine = self._engine
         entries = [StepEntry(("scheduled", e.request_id), e.tokens, e.want, e.from_slot) for e in entries]
-        if all(p.greedy for p in sampling):
-            return engine.runner.step(entries, choose=True)     # greedy: chosen inside the step
-        logits = engine.runner.step(entries)
-        if logits is None:
-            return None
-        tokens = engine.sampler.sample(logits, sampling, steps, token_slots=engine.cache.last_token,
-                                       slot_of_row=engine.runner.last_batch.logit_slots)
-        for entry in entries:
-            if entry.want:
-                engine.cache.note_sampled(entry.request_id)
-        return engine.runner.tokens_to_host(tokens, logits.shape[0])
+        # the tokens are chosen inside the step, greedily or as each row's parameters say
+        return engine.runner.step(entries, choose=True, sampling=(sampling, steps))
 
     def collect(self, handle):
         return [] if handle is None else handle.tolist()

@@ -135,13 +135,15 @@ class _DecodeGraph:
     """One captured decode step for up to ``capacity`` requests. ``chooses``: the captured step ends with the greedy
     choice of its tokens (models.TokenChoice) and moves its batch on by one token on the device, so that the next step
     of the same requests, each taking its token from its last-token slot, is replayed without anything being copied to
-    the device before it or from the device after it: the tokens arrive in a ring of rows in page-locked host memory."""
+    the device before it or from the device after it: the tokens arrive in a ring of rows in page-locked host memory.
+    ``draws``: such a step draws its tokens as each row's sampling parameters say (temperature, top-p; they and the count
+    of tokens a request has drawn lie in the same device buffer, and the count moves on with the batch)."""
 
-    def __init__(self, runner: "ModelRunner", capacity: int, chooses: bool = False, reach: int | None = None):
+    def __init__(self, runner: "ModelRunner", capacity: int, chooses: bool = False, reach: int | None = None, draws: bool = False):
         import torch
 
-        self.runner, self.capacity, self.chooses = runner, capacity, chooses
-        self.builder = DecodeBatchBuilder(runner.cache, capacity)
+        self.runner, self.capacity, self.chooses, self.draws = runner, capacity, chooses, draws and chooses
+        self.builder = DecodeBatchBuilder(runner.cache, capacity, draws=self.draws)
         self.buffer = torch.zeros(len(self.builder.flat), dtype=torch.int32, device=runner.device)
         self.static_batch = self.builder.batch(self.buffer, [], reach)
         self.graph = None
@@ -159,10 +161,10 @@ class _DecodeGraph:
             self.on_device = None   # per row (request's cache entry, its table_changes, its length) that the device's batch stands at
             self.uploads = 0
 
-    def run(self, entries):
+    def run(self, entries, sampling=None):
         runner = self.runner
         if self.chooses:
-            return self._run_choosing(entries)
+            return self._run_choosing(entries, sampling)
         runner.staging.upload(self.builder.fill(entries), into=self.buffer)
         batch = self.static_batch
         batch.request_ids = [e.request_id for e in entries]
@@ -171,34 +173,44 @@ class _DecodeGraph:
         self.graph.replay()
         return batch, self.logits[: len(entries)]
 
-    def _run_choosing(self, entries):
+    def _run_choosing(self, entries, sampling=None):
         import torch
 
-        from ..models.base import TokenChoice
+        from ..models.base import DrawParameters, TokenChoice
 
         runner, cache = self.runner, self.runner.cache
         records = [cache.requests[e.request_id] for e in entries]
         stands = self.on_device
+        if self.draws:
+            if sampling is None or len(sampling[0]) != len(entries) or len(sampling[1]) != len(entries):
+                raise ValueError("a step that draws its tokens needs each row's sampling parameters and count of tokens drawn")
+            hows, counts = sampling
+        else:
+            hows = counts = [None] * len(entries)
         # The device has moved the last step's batch on by itself. It is this step's batch if the same requests come
         # again in the same rows, each with the token in its slot, and no block table has changed since (a request that
         # reaches a new page, or gives one back, has: then everything is brought from the host as ever).
         carried_on = (stands is not None and len(stands) == len(records) and all(e.from_slot for e in entries)
-                      and all(r is at[0] and r.table_changes == at[1] and r.length == at[2] for r, at in zip(records, stands)))
+                      and all(r is at[0] and r.table_changes == at[1] and r.length == at[2] and (how is at[3] or how == at[3]) and count == at[4]
+                              for r, at, how, count in zip(records, stands, hows, counts)))
         if not carried_on:
             flat = self.builder.fill(entries)
+            if self.draws:
+                self.builder.fill_draws(hows, counts)
             self.builder.cursor[:] = (self.ring_at, self.number, 0)
             runner.staging.upload(flat, into=self.buffer)
             self.uploads += 1
         batch = self.static_batch
         batch.request_ids = [e.request_id for e in entries]
         if self.graph is None:
-            choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True)
+            draws = DrawParameters(*self.builder.draw_views(self.buffer)) if self.draws else None
+            choice = TokenChoice(cache.last_token, host_ring=self.ring, cursor=self.builder.cursor_view(self.buffer), advance=True, draws=draws)
             self.graph, self.logits = _capture(runner, batch, choice, self.lanes)
         self.graph.replay()
         chosen = ChosenTokens(self.logits[: len(entries)], self.ring_rows[self.ring_at], len(entries), number=self.number, flags=self.flags)
         self.ring_at = (self.ring_at + 1) % TOKEN_RING_ROWS
         self.number = (self.number + 1) & 0x3FFFFFFF
-        self.on_device = [(r, r.table_changes, r.length + 1) for r in records]
+        self.on_device = [(r, r.table_changes, r.length + 1, how, None if count is None else count + 1) for r, how, count in zip(records, hows, counts)]
         return batch, chosen
 
 
@@ -288,6 +300,7 @@ class ModelRunner:
         self.portion_graph_after = PORTION_GRAPH_AFTER if portion_graph_after is None else int(portion_graph_after)
         self.portion_graph_steps = 0
         self._token_rows, self._token_turn = [], 0
+        self._sampler = None
         self.portion_graphs_made = 0      # captures of steps with prompt portions, and those given up for a newer shape
         self.portion_graphs_dropped = 0
 
@@ -366,7 +379,7 @@ class ModelRunner:
             extra["lanes"] = lanes
         return self.model.forward(batch, self.cache, resolve_tokens=resolve, **extra)
 
-    def _graph_for(self, entries, choose: bool = False):
+    def _graph_for(self, entries, choose: bool = False, draws: bool = False):
         if not self.use_graphs:
             return None
         if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
@@ -379,9 +392,9 @@ class ModelRunner:
         if self._decode_reaches:
             longest = max(self.cache.length(e.request_id) for e in entries) + 1
             reach = next((r for r in self._decode_reaches if r >= longest), reach)
-        key = (capacity, choose, reach)
+        key = (capacity, choose, reach) + ((True,) if choose and draws else ())
         if key not in self._graphs:
-            self._graphs[key] = _DecodeGraph(self, capacity, chooses=choose, reach=reach)
+            self._graphs[key] = _DecodeGraph(self, capacity, chooses=choose, reach=reach, draws=draws)
         return self._graphs[key]
 
     def _portion_graph_for(self, entries):
@@ -414,7 +427,7 @@ class ModelRunner:
         self.portion_graphs_made += 1
         return graph
 
-    def step(self, entries: list[StepEntry], observer=None, choose: bool = False):
+    def step(self, entries: list[StepEntry], observer=None, choose: bool = False, sampling=None):
         """Runs the entries as one batch. Returns float32 logits [wanted places, vocab] on the
         device (None if nothing is wanted), in the order of the entries and of each ``want``;
         they are valid until the next step. Raises StepError / OutOfPages before anything has
@@ -424,8 +437,16 @@ class ModelRunner:
 
         ``choose``: the step also chooses the greedy token at every wanted place, on the device, leaves it in the
         request's last-token slot and returns ``ChosenTokens`` instead of logits (a decode step does all of it inside
-        its captured graph, and is replayed without a copy to or from the device while the same requests go on)."""
+        its captured graph, and is replayed without a copy to or from the device while the same requests go on).
+        ``sampling`` (with ``choose``): (one SamplingParams per wanted place, the number of tokens its request has drawn
+        before this one), in the order of the logits: the tokens are drawn as those say instead of greedily."""
         self.validate(entries)
+        if sampling is not None:
+            wanted = sum(len(e.want) for e in entries)
+            if not choose or len(sampling[0]) != wanted or len(sampling[1]) != wanted:
+                raise StepError("sampling goes with choose=True, one parameter set and one count per wanted place")
+            if all(how.greedy for how in sampling[0]):
+                sampling = None
         reserved = []
         try:
             for entry in entries:
@@ -436,9 +457,9 @@ class ModelRunner:
                 self.cache.rollback(request_id)
             raise
         try:
-            graph = self._graph_for(entries, choose) if observer is None else None
+            graph = self._graph_for(entries, choose, sampling is not None) if observer is None else None
             if graph is not None:
-                batch, logits = graph.run(entries)
+                batch, logits = graph.run(entries, sampling) if isinstance(graph, _DecodeGraph) else graph.run(entries)
                 if isinstance(graph, _PortionGraph):
                     self.portion_graph_steps += 1
                 else:
@@ -451,7 +472,7 @@ class ModelRunner:
                     in_given_order = lambda name, hidden: observer(name, hidden[rows])
                 logits = self.forward(batch, resolve=any(e.from_slot for e in entries), observer=in_given_order)
             if choose and not isinstance(logits, ChosenTokens):
-                logits = self._choose_from_logits(logits, batch)
+                logits = self._choose_from_logits(logits, batch, sampling)
         except Exception:
             for request_id in reserved:
                 self.cache.rollback(request_id)
@@ -464,14 +485,21 @@ class ModelRunner:
         self.last_batch = batch
         return logits
 
-    def _choose_from_logits(self, logits, batch):
-        """The greedy tokens of a step that was not captured with its choice: the sampler's argmax over the logits, each
-        token left in its request's last-token slot."""
+    def _choose_from_logits(self, logits, batch, sampling=None):
+        """The tokens of a step that was not captured with its choice: the sampler over the logits (its argmax, or a draw
+        as ``sampling`` says), each token left in its request's last-token slot."""
         if logits is None:
             return None
-        from ..ops import kernels
+        if sampling is None:
+            from ..ops import kernels
 
-        tokens = kernels.sample(logits, token_slots=self.cache.last_token, slot_of_row=batch.logit_slots)
+            tokens = kernels.sample(logits, token_slots=self.cache.last_token, slot_of_row=batch.logit_slots)
+        else:
+            if self._sampler is None:
+                from ..sampling import Sampler
+
+                self._sampler = Sampler(self.staging)
+            tokens = self._sampler.sample(logits, list(sampling[0]), list(sampling[1]), token_slots=self.cache.last_token, slot_of_row=batch.logit_slots)
         return self.tokens_to_host(tokens, logits.shape[0])
 
     def tokens_to_host(self, tokens, n: int) -> ChosenTokens:

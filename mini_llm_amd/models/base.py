@@ -33,16 +33,30 @@ class CacheGroupSpec:
 
 
 @dataclass
+class DrawParameters:
+    """How the rows of a step draw their tokens, one entry a wanted row, on the device: ``seeds`` (int64),
+    ``temperatures`` (float32; 0: the argmax), ``top_ps`` (float32) and ``counts`` (int32: the tokens the row's request
+    has drawn so far; the random numbers are a function of seed and count, kernels.sample)."""
+
+    seeds: object
+    temperatures: object
+    top_ps: object
+    counts: object
+
+
+@dataclass
 class TokenChoice:
-    """Asks a step to choose its tokens on the device, greedily, as its last kernel: one token per wanted row, left in
-    the request's last-token slot (``token_slots``: the cache's), and, with ``host_ring`` / ``cursor``, in a ring of
-    rows in page-locked host memory (kernels.choose). ``advance``: a step of single tokens also moves its batch on by
-    one token on the device, so that the same requests' next step needs nothing from the host."""
+    """Asks a step to choose its tokens on the device as its last kernel: one token per wanted row, the greedy one
+    or, with ``draws``, one drawn as those say; left in the request's last-token slot (``token_slots``: the cache's), and,
+    with ``host_ring`` / ``cursor``, in a ring of rows in page-locked host memory (kernels.choose). ``advance``: a step of
+    single tokens also moves its batch on by one token on the device (and the counts of ``draws``), so that the same
+    requests' next step needs nothing from the host."""
 
     token_slots: object
     host_ring: object = None
     cursor: object = None
     advance: bool = False
+    draws: DrawParameters | None = None
 
 
 class Model(Part):
@@ -192,8 +206,11 @@ class Model(Part):
             return self.head.forward(normed)
         # Greedy tokens on the device. A head that can leave the best of its columns instead of all of them does (the
         # logits of a greedy step are read by nobody); any other head's logits go through the sampler's argmax.
-        best = self.head.forward_best(normed) if hasattr(self.head, "forward_best") else None
-        if best is None:
+        draws = choice.draws
+        best = self.head.forward_best(normed) if draws is None and hasattr(self.head, "forward_best") else None
+        if draws is not None:    # drawn from the logits; what is left to choose from is the one token a row
+            values, indices = None, kernels.sample(self.head.forward(normed), draws.temperatures, draws.top_ps, draws.seeds, draws.counts).view(-1, 1)
+        elif best is None:
             values, indices = None, kernels.sample(self.head.forward(normed)).view(-1, 1)
         else:
             values, indices = best
@@ -202,6 +219,7 @@ class Model(Part):
             if batch.max_q_len != 1 or batch.n_logit_rows != batch.n_tokens:
                 raise ValueError("only a step of single tokens that all want their logits can be moved on by one on the device")
             advance = kernels.StepAdvance(batch.positions, batch.context_lens, batch.token_sources, [g.block_tables for g in batch.groups],
-                                          [g.slots for g in batch.groups], cache.page_size)
+                                          [g.slots for g in batch.groups], cache.page_size,
+                                          draw_counts=None if draws is None else draws.counts)
         return kernels.choose(values, indices, batch.logit_slots, choice.token_slots, host_ring=choice.host_ring, cursor=choice.cursor,
                               advance=advance)

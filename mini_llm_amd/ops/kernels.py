@@ -522,7 +522,8 @@ class StepAdvance:
     """What ``choose`` moves on by one token for every live row, so that the same requests' next step finds its batch on
     the device: positions and stored lengths, the source of each row's token (its own last-token slot from then on), and
     per cache group the row a token's key and value go to, looked up in the group's block table ([rows, table_width],
-    int32; pages of ``page_size`` tokens)."""
+    int32; pages of ``page_size`` tokens). ``draw_counts`` (optional, int32 [rows]): how many tokens each row's request has
+    drawn so far, which a sampler's random numbers are a function of; grows by one too."""
 
     positions: torch.Tensor
     context_lens: torch.Tensor
@@ -530,6 +531,7 @@ class StepAdvance:
     block_tables: list
     slots: list
     page_size: int
+    draw_counts: torch.Tensor | None = None
 
 
 def choose_flags(rows: int) -> int:
@@ -573,10 +575,10 @@ def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, 
         _require(cursor is None, "a cursor without a ring")
     tables = slots = None
     n_groups = table_width = page_size = 0
-    positions = context_lens = sources = None
+    positions = context_lens = sources = draws = None
     if advance is not None:
-        positions, context_lens, sources = advance.positions, advance.context_lens, advance.token_sources
-        for t, name in ((positions, "positions"), (context_lens, "context_lens"), (sources, "token_sources")):
+        positions, context_lens, sources, draws = advance.positions, advance.context_lens, advance.token_sources, advance.draw_counts
+        for t, name in ((positions, "positions"), (context_lens, "context_lens"), (sources, "token_sources")) + (((draws, "draw_counts"),) if draws is not None else ()):
             _device_tensor(t, name, torch.int32, 1)
             _require(t.shape[0] >= rows, f"{name} has fewer entries than rows")
         n_groups, page_size = len(advance.block_tables), int(advance.page_size)
@@ -593,7 +595,7 @@ def choose(values, indices, state_slots, token_slots, out=None, host_ring=None, 
         slots = (ctypes.c_void_p * max(n_groups, 1))(*[t.data_ptr() for t in advance.slots])
     check(library().mllm_choose(_ptr(values), _ptr(indices), per_row, rows, _ptr(state_slots), _ptr(token_slots), _ptr(out),
                                 _ptr(host_ring), ring_rows, ring_stride, _ptr(cursor), int(advance is not None), _ptr(positions), _ptr(context_lens),
-                                _ptr(sources), tables, slots, n_groups, table_width, page_size, _stream()))
+                                _ptr(sources), _ptr(draws), tables, slots, n_groups, table_width, page_size, _stream()))
     return out
 
 

@@ -37,7 +37,7 @@ _SIGNATURES = {
     "mllm_sample": [P, c_int, c_int, P, P, P, P, P, P, P, P],
     "mllm_gemm_best_per_row": [c_int, c_int, c_int, c_int],
     "mllm_gemm_best": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
-    "mllm_choose": [P, P, c_int, c_int, P, P, P, P, c_int, c_int, P, c_int, P, P, P, P, P, c_int, c_int, c_int, P],
+    "mllm_choose": [P, P, c_int, c_int, P, P, P, P, c_int, c_int, P, c_int, P, P, P, P, P, P, c_int, c_int, c_int, P],
     "mllm_decode_layer_supported": [c_int, c_int, c_int, c_int],
     "mllm_decode_layer_rows": [c_int],
     "mllm_decode_attention_half": [P, P, P, c_int, P, P, P, c_float, P, P, P, P, P, P, P, P, P, c_int, P,

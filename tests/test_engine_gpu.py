@@ -91,6 +91,52 @@ def test_temperature_sampling_in_chunks_beside_decodes(model_dirs, engines):
     assert alone[0] == out[2]
 
 
+def test_sampled_rows_are_drawn_inside_the_captured_decode_step(model_dirs):
+    # Three requests decode side by side through the scheduler, one greedily, one at temperature 0.7, one at 1.3 with a
+    # nucleus: the captured step draws the tokens itself (the rows' parameters and counts of tokens drawn lie in its
+    # device buffer, and the counts move on with the batch), so that between two steps of the same requests nothing is
+    # copied. Every token is checked against the plain implementation and the generator on the host.
+    from mini_llm_amd.engine.engine import Engine, EngineOptions
+    from mini_llm_amd.engine.scheduler import Request
+    from mini_llm_amd.sampling import SamplingParams
+
+    folder, config, weights = model_dirs["A"]
+    vocab = config["vocab_size"]
+    engine = Engine(folder, EngineOptions(dtype="float32", max_sessions=4))
+    prompts = [random_tokens(20 + i, n, vocab) for i, n in enumerate((6, 11, 3))]
+    hows = [SamplingParams(), SamplingParams(temperature=0.7, seed=5), SamplingParams(temperature=1.3, top_p=0.6, seed=9)]
+    new_tokens = 40
+    out = [[] for _ in prompts]
+    for i, (prompt, how) in enumerate(zip(prompts, hows)):
+        engine.submit(Request(prompt, on_token=lambda token, finish, i=i: out[i].append(token), on_error=lambda message: pytest.fail(message),
+                              max_new_tokens=new_tokens, sampling=how))
+    engine.scheduler.run_until_idle()
+    drawn = [g for key, g in engine.runner._graphs.items() if len(key) == 4]
+    assert len(drawn) == 1 and drawn[0].draws
+    # three requests of 9 to 51 tokens cross a page edge (64 tokens a page) never, and finish together: the batch is
+    # brought from the host once, and once more at most for what the scheduler's first decode step finds
+    assert drawn[0].uploads <= 2, drawn[0].uploads
+    assert engine.runner.graph_steps >= new_tokens - 2
+    for i, (prompt, how, generated) in enumerate(zip(prompts, hows, out)):
+        assert len(generated) == new_tokens
+        tokens = list(prompt)
+        for step, token in enumerate(generated):
+            logits = plain_gpt2.forward(config, weights, tokens)[-1]
+            if how.greedy:
+                assert token == int(np.argmax(logits)), (i, step)
+            else:
+                noise = np.array([-math.log(-math.log(host_uniform(how.seed, step, v))) for v in range(vocab)])
+                score = (logits - logits.max()) / how.temperature + noise
+                if how.top_p < 1.0:   # outside the nucleus nothing is drawn (a little slack for rounding at its edge)
+                    p = plain_gpt2.softmax(logits / how.temperature)
+                    assert p[p > p[token] * (1 + 1e-4)].sum() < how.top_p + 1e-4, (i, step)
+                    surely_inside = np.array([p[p > p[v] * (1 - 1e-4)].sum() - p[v] < how.top_p - 1e-3 for v in range(vocab)])
+                    score = np.where(surely_inside | (np.arange(vocab) == token), score, -np.inf)   # it beats all that are surely inside
+                assert score[token] >= score.max() - 1e-3, f"request {i} step {step}: token {token} is not the draw"
+            tokens.append(token)
+    engine.close()
+
+
 def test_top_p_generation_stays_in_the_nucleus(model_dirs, engines):
     _, config, weights = model_dirs["A"]
     prompt = random_tokens(9, 12, config["vocab_size"])

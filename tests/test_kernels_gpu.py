@@ -1081,7 +1081,8 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
     last = torch.full((9,), -1, dtype=torch.int32, device=DEV)
     ring = torch.full((3, 8), -9, dtype=torch.int32).pin_memory()
     cursor = d([2, 41, 0])
-    advance = K.StepAdvance(pos_d, ctx_d, src_d, tab_d, slot_d, page)
+    draws = d(np.arange(rows) * 10)   # how many tokens each row's request has drawn: one more with every step, for live rows
+    advance = K.StepAdvance(pos_d, ctx_d, src_d, tab_d, slot_d, page, draw_counts=draws)
     for turn in range(2):
         tokens = K.choose(None, d(indices), d(live), last, host_ring=ring, cursor=cursor, advance=advance)
         torch.cuda.synchronize()
@@ -1093,6 +1094,7 @@ def test_choose_moves_a_decode_batch_on_by_one_token(K):
         now = positions + (turn + 1) * (live >= 0)
         assert pos_d.cpu().numpy().tolist() == now.tolist() and ctx_d.cpu().numpy().tolist() == now.tolist()
         assert src_d.cpu().numpy().tolist() == np.where(live >= 0, live, -1).tolist()
+        assert draws.cpu().numpy().tolist() == (np.arange(rows) * 10 + (turn + 1) * (live >= 0)).tolist()
         for table, slots in zip(tables, slot_d):
             expect = []
             for r in range(rows):
