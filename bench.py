@@ -601,7 +601,7 @@ def main() -> int:
             s, _ = DecodeBench(engine, batch, args.prompt_len).run(steps, 8)
             points[f"decode_b{batch}"] = round(batch * steps / s, 1)
         record["points"] = points
-        record["kernels"] = measure_kernels(engine, context=(3 * CONTEXT // 4) // 64 * 64 + 8)
+        record["kernels"] = measure_kernels(engine, batch=args.batch, context=(3 * CONTEXT // 4) // 64 * 64 + 8)
         if not args.one_dtype:
             # the same figures in the other precision (the headline names both): one record for the two
             other = "float32" if args.dtype == "bfloat16" else "bfloat16"

@@ -184,17 +184,20 @@ constexpr int DECODE_MAX_SPLITS = 16;
 // the token's keys evenly among themselves, and their partial results meet in LDS.
 // TOGETHER: how a wave starts (see there); the host chooses.
 // parts (gridDim.z) > 1: few tokens with many keys, where a block per (token, head) would leave most of the chip idle.
-// The token's keys are cut into so many runs, a block each, and a block leaves its unnormalised sums with their maximum
-// and weight in `parts_out` ([token, head, part, HD + 2] floats) for attention_decode_merge_kernel instead of writing `out`.
+// The token's keys are cut into so many runs, a block each. A block leaves its unnormalised sums with their maximum and
+// weight in `parts_out` ([token, head, part, HD + 2] floats) and counts itself in arrivals[token, head] (zero before the
+// launch); the block that is through last puts the runs together, out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M),
+// and the count is zero again behind it (it wraps), so the same counters serve the next launch.
 template <typename T, int HD, bool TOGETHER>
 __global__ __launch_bounds__(1024) void attention_decode_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, T* __restrict__ out, int out_stride,
     const int* __restrict__ token_request, const int* __restrict__ positions,
     const int* __restrict__ block_tables, int max_blocks, int n_heads, int n_kv_heads,
-    int page_shift, int window, float scale, int out_packed, float* __restrict__ parts_out) {
+    int page_shift, int window, float scale, int out_packed, float* parts_out, int* __restrict__ arrivals) {
     constexpr int VEC = KeySweep<T, HD>::VEC, LPR = KeySweep<T, HD>::LPR, RPI = KeySweep<T, HD>::RPI;
     __shared__ float partial[DECODE_MAX_SPLITS][HD + 2];
+    __shared__ int through_last;
 
     const int lane = threadIdx.x % WAVE, split = threadIdx.x / WAVE, n_splits = blockDim.x / WAVE;
     const int head = blockIdx.x, token = blockIdx.y;
@@ -205,8 +208,8 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
         return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
     };
     const int n_parts = gridDim.z, part = blockIdx.z;
-    if (request < 0) {  // a padding row; the whole block leaves together (the merge writes its zeros where there are parts)
-        if (n_parts == 1)
+    if (request < 0) {  // a padding row; the whole block leaves together (its zeros come from the block of the first run)
+        if (part == 0)
             for (int d = threadIdx.x; d < HD; d += blockDim.x) *out_at(d) = from_float<T>(0.0f);
         return;
     }
@@ -286,15 +289,46 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     float total = 0.0f;
     for (int s = 0; s < n_splits; s++) total += total_max == -INFINITY ? 0.0f : partial[s][HD + 1] * expf(partial[s][HD] - total_max);
     if (n_parts > 1) {  // a run without keys (a short sequence in a launch cut for long ones) leaves max -inf and weight 0
-        float* mine = parts_out + (((size_t)token * n_heads + head) * n_parts + part) * (HD + 2);
+        float* runs = parts_out + ((size_t)token * n_heads + head) * n_parts * (HD + 2);
+        float* mine = runs + part * (HD + 2);
+        // Stored through to where every compute unit sees it; one thread then counts the block in with release and
+        // acquire (a fence in every wave writes the whole L2 back sixteen times a block: 16 -> 60 us at 96 pairs).
+        auto put = [&](float* at, float value) { __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
         for (int d = threadIdx.x; d < HD; d += blockDim.x) {
             float value = 0.0f;
             for (int s = 0; s < n_splits; s++) value += total_max == -INFINITY ? 0.0f : partial[s][d] * expf(partial[s][HD] - total_max);
-            mine[d] = value;
+            put(mine + d, value);
         }
         if (threadIdx.x == 0) {
-            mine[HD] = total_max;
-            mine[HD + 1] = total;
+            put(mine + HD, total_max);
+            put(mine + HD + 1, total);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0)
+            through_last = __builtin_amdgcn_atomic_inc32(reinterpret_cast<unsigned*>(arrivals + token * n_heads + head), (unsigned)(n_parts - 1),
+                                                          __ATOMIC_ACQ_REL, "agent") == (unsigned)(n_parts - 1);
+        __syncthreads();
+        if (!through_last || split != 0) return;
+        // The last block's first wave: lane p takes run p's maximum and weight (up to 64 runs), the wave settles M and
+        // the sum with shuffles, and each lane adds up its head dimensions over the runs, four runs' loads under way at
+        // a time. The other blocks' stores are read past this compute unit's caches.
+        auto far = [&](int index) { return __hip_atomic_load(runs + index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        const float run_max = lane < n_parts ? far(lane * (HD + 2) + HD) : -INFINITY;
+        const float run_sum = lane < n_parts ? far(lane * (HD + 2) + HD + 1) : 0.0f;
+        const float all_max = wave_max_total(run_max);               // finite: the first run always has a key
+        const float factor = run_max == -INFINITY ? 0.0f : expf(run_max - all_max);
+        const float one_over = 1.0f / wave_total(run_sum * factor);
+        for (int d0 = 0; d0 < HD; d0 += WAVE) {
+            const int d = min(d0 + lane, HD - 1);
+            float value = 0.0f;
+            for (int p0 = 0; p0 < n_parts; p0 += 4) {
+                float o[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) o[u] = far(min(p0 + u, n_parts - 1) * (HD + 2) + d);
+#pragma unroll
+                for (int u = 0; u < 4; u++) value += p0 + u < n_parts ? o[u] * __shfl(factor, p0 + u, WAVE) : 0.0f;
+            }
+            if (d0 + lane < HD) *out_at(d) = from_float<T>(value * one_over);
         }
         return;
     }
@@ -306,38 +340,12 @@ __global__ __launch_bounds__(1024) void attention_decode_kernel(
     }
 }
 
-// The runs of one (token, head) put together: out = sum_p o_p e^(m_p - M) / sum_p l_p e^(m_p - M). A wave per (token, head).
-template <typename T, int HD>
-__global__ __launch_bounds__(WAVE) void attention_decode_merge_kernel(
-    const float* __restrict__ parts, int n_parts, T* __restrict__ out, int out_stride,
-    const int* __restrict__ token_request, int n_heads, int out_packed) {
-    const int head = blockIdx.x, token = blockIdx.y, lane = threadIdx.x;
-    auto out_at = [&](int d) -> T* {
-        return out + (out_packed ? packed_element<T>(token, head * HD + d, n_heads * HD) : (size_t)token * out_stride + head * HD + d);
-    };
-    if (token_request[token] < 0) {
-        for (int d = lane; d < HD; d += WAVE) *out_at(d) = from_float<T>(0.0f);
-        return;
-    }
-    const float* mine = parts + ((size_t)token * n_heads + head) * n_parts * (HD + 2);
-    float total_max = -INFINITY;
-    for (int p = 0; p < n_parts; p++) total_max = fmaxf(total_max, mine[p * (HD + 2) + HD]);
-    float total = 0.0f;
-    for (int p = 0; p < n_parts; p++) total += mine[p * (HD + 2) + HD + 1] * expf(mine[p * (HD + 2) + HD] - total_max);
-    const float inverse = 1.0f / total;
-    for (int d = lane; d < HD; d += WAVE) {
-        float value = 0.0f;
-        for (int p = 0; p < n_parts; p++) value += mine[p * (HD + 2) + d] * expf(mine[p * (HD + 2) + HD] - total_max);
-        *out_at(d) = from_float<T>(value * inverse);
-    }
-}
-
 template <typename T>
 int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pages, const void* v_pages,
                     void* out, int out_stride, const int* token_request, const int* positions,
                     const int* block_tables, int max_blocks, int n_tokens, int n_heads, int n_kv_heads,
                     int page_shift, int window, float scale, int n_splits, int out_packed, int n_parts, float* parts,
-                    hipStream_t stream) {
+                    int* arrivals, hipStream_t stream) {
     dim3 grid(n_heads, n_tokens, n_parts), block(WAVE * n_splits);
     // Measured on MI355X: starting with query and pages together (and, in bfloat16, the pages a
     // round ahead) is 3 to 15 % faster wherever a wave has few rounds, which is where a kernel's
@@ -354,16 +362,11 @@ int dispatch_decode(int head_size, const void* q, int q_stride, const void* k_pa
         if (together)                                                                                          \
             attention_decode_kernel<T, HD, true><<<grid, block, 0, stream>>>(                                  \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts);  \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals);  \
         else                                                                                                   \
             attention_decode_kernel<T, HD, false><<<grid, block, 0, stream>>>(                                 \
                 (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, token_request,   \
-                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts);  \
-        if (n_parts > 1) {                                                                                     \
-            mllm_count_kernel(MLLM_K_ATTENTION_DECODE_MERGE);                                                  \
-            attention_decode_merge_kernel<T, HD><<<dim3(n_heads, n_tokens), WAVE, 0, stream>>>(                \
-                parts, n_parts, (T*)out, out_stride, token_request, n_heads, out_packed);                      \
-        }                                                                                                      \
+                positions, block_tables, max_blocks, n_heads, n_kv_heads, page_shift, window, scale, out_packed, parts, arrivals);  \
         return 0;
     switch (head_size) {
         MLLM_DECODE_CASE(16)
@@ -389,7 +392,8 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                                    void* out, int out_stride, const int* token_request, const int* positions,
                                    const int* block_tables, int max_blocks, int n_tokens, int n_heads,
                                    int n_kv_heads, int head_size, int page_size, int window, float scale,
-                                   int n_splits, int dtype, int out_packed, int n_parts, float* parts, hipStream_t stream) {
+                                   int n_splits, int dtype, int out_packed, int n_parts, float* parts, int* arrivals,
+                                   hipStream_t stream) {
     MLLM_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && max_blocks > 0, "attention_decode: bad sizes");
     MLLM_REQUIRE(n_heads % n_kv_heads == 0, "attention_decode: %d heads do not divide into %d key/value heads", n_heads, n_kv_heads);
     MLLM_REQUIRE(mllm_attention_decode_supported(head_size, page_size, dtype),
@@ -399,18 +403,19 @@ MLLM_API int mllm_attention_decode(const void* q, int q_stride, const void* k_pa
                  "attention_decode: %d splits is not a power of two in 1..%d", n_splits, DECODE_MAX_SPLITS);
     MLLM_REQUIRE(q_stride >= n_heads * head_size && out_stride >= n_heads * head_size, "attention_decode: rows are too short for the heads");
     MLLM_REQUIRE(n_tokens <= 65535, "attention_decode: too many tokens for one launch");
-    // parts: the keys of a token in so many runs, a block each; `parts` then holds n_tokens * n_heads * n_parts * (head_size + 2) floats
-    MLLM_REQUIRE(n_parts >= 1 && n_parts <= 64 && (n_parts == 1 || parts != nullptr), "attention_decode: %d parts (1..64, with memory for them)", n_parts);
+    // parts: the keys of a token in so many runs, a block each; `parts` then holds n_tokens * n_heads * n_parts * (head_size + 2)
+    // floats and `arrivals` n_tokens * n_heads counters that are zero (and are zero again when the kernel is through)
+    MLLM_REQUIRE(n_parts >= 1 && n_parts <= 64 && (n_parts == 1 || (parts != nullptr && arrivals != nullptr)), "attention_decode: %d parts (1..64, with memory and counters for them)", n_parts);
     if (n_tokens == 0) return 0;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) page_shift++;
     int refused = 1;
     if (dtype == MLLM_F32)
         refused = dispatch_decode<float>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, stream);
+                                         block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, stream);
     else
         refused = dispatch_decode<bf16_t>(head_size, q, q_stride, k_pages, v_pages, out, out_stride, token_request, positions,
-                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, stream);
+                                          block_tables, max_blocks, n_tokens, n_heads, n_kv_heads, page_shift, window, scale, n_splits, out_packed, n_parts, parts, arrivals, stream);
     MLLM_REQUIRE(!refused, "attention_decode: no kernel for dtype %d and head size %d", dtype, head_size);
     return mllm_check_launch("attention_decode");
 }

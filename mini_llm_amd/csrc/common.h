@@ -66,7 +66,7 @@ enum MllmKernel : int {
     MLLM_K_EMBED = 0, MLLM_K_LAYERNORM, MLLM_K_ADD, MLLM_K_CACHE_WRITE, MLLM_K_ATTENTION_GENERAL, MLLM_K_ATTENTION_DECODE,
     MLLM_K_ATTENTION_PREFILL, MLLM_K_ATTENTION_PREFILL_STREAM, MLLM_K_PACK, MLLM_K_CONVERT, MLLM_K_DECODE_ATTENTION_HALF,
     MLLM_K_DECODE_MLP_HALF, MLLM_K_PENDING_SUM, MLLM_K_PENDING_LAYERNORM, MLLM_K_GEMM_SKINNY, MLLM_K_GEMM_TILED, MLLM_K_GEMM_STREAM,
-    MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_GEMM_BEST, MLLM_K_CHOOSE, MLLM_K_ATTENTION_DECODE_MERGE, MLLM_K_KINDS
+    MLLM_K_STATIC_SUM, MLLM_K_PROBE, MLLM_K_SAMPLE, MLLM_K_GEMM_BEST, MLLM_K_CHOOSE, MLLM_K_KINDS
 };
 void mllm_count_kernel(MllmKernel kind);
 

@@ -30,7 +30,7 @@ static std::atomic<unsigned long long> g_launches[MLLM_K_KINDS];
 static const char* const g_kernel_names[MLLM_K_KINDS] = {
     "embed", "layernorm", "add", "cache_write", "attention_general", "attention_decode", "attention_prefill",
     "attention_prefill_stream", "pack", "convert", "decode_attention_half", "decode_mlp_half", "pending_sum",
-    "pending_layernorm", "gemm_skinny", "gemm_tiled", "gemm_stream", "static_sum", "probe", "sample", "gemm_best", "choose", "attention_decode_merge",
+    "pending_layernorm", "gemm_skinny", "gemm_tiled", "gemm_stream", "static_sum", "probe", "sample", "gemm_best", "choose",
 };
 
 void mllm_count_kernel(MllmKernel kind) { g_launches[kind].fetch_add(1, std::memory_order_relaxed); }

@@ -57,6 +57,7 @@ class StepBatch:
     short_requests: int     # the first so many requests bring portions of at most SHORT_PORTION tokens,
     short_rows: int         # which are the first so many rows; the requests after them bring longer ones
     short_portion: int = field(default=SHORT_PORTION, kw_only=True)   # the length that cut was made at
+    first_row: int = field(default=0, kw_only=True)   # a part of a step's batch (rows_of_requests): its first row's place in the whole
     max_total_len: int      # the longest sequence after this step
     tokens: object          # int32 [n_tokens]
     positions: object       # int32 [n_tokens]
@@ -85,7 +86,7 @@ class StepBatch:
             q_starts=self.q_starts[lo : hi + 1], context_lens=cut(self.context_lens), state_slots=cut(self.state_slots),
             logit_rows=cut(self.logit_rows), token_sources=cut(self.token_sources), logit_slots=cut(self.logit_slots),
             groups=[GroupStepData(block_tables=g.block_tables, slots=cut(g.slots)) for g in self.groups],
-            request_ids=self.request_ids[lo:hi], host={},
+            request_ids=self.request_ids[lo:hi], host={}, first_row=self.first_row + lo,
         )
 
     def rows_in_order_of(self, request_ids) -> list:

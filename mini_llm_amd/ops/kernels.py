@@ -375,8 +375,29 @@ DECODE_MIN_PART_FEW = 512
 DECODE_MIN_PART_BYTES = 4096
 
 
+_arrival_counters: dict = {}
+_outgrown_counters: list = []
+
+
+def _arrivals(k_pages, rows: int, n_heads: int):
+    """Counters, zero between launches, for the decode attention's blocks that share a (row, head): one set for each
+    cache tensor (a layer of an engine), which serves one step at a time; the parts of a step that run side by side take
+    different rows of it. Never given back: a captured step keeps launching with the address it was captured with."""
+    key = (k_pages.device.index, k_pages.data_ptr())
+    counters = _arrival_counters.get(key)
+    if counters is None or counters.shape[0] < rows * n_heads:
+        if torch.cuda.is_current_stream_capturing():
+            # memory taken inside a capture belongs to the captured graph: this launch alone gets it (and the fill
+            # that zeroes it is replayed with the launch)
+            return torch.zeros(rows * n_heads, dtype=torch.int32, device=k_pages.device)
+        if counters is not None:
+            _outgrown_counters.append(counters)
+        counters = _arrival_counters[key] = torch.zeros(max(rows * n_heads, 1024), dtype=torch.int32, device=k_pages.device)
+    return counters
+
+
 def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables, n_heads, n_kv_heads, head_size, scale, window=0, max_q_len=None, max_len=None, q_starts=None, context_lens=None, out=None,
-                    short_rows=None, short_requests=None, packed_out=False):
+                    short_rows=None, short_requests=None, packed_out=False, first_row=0):
     """Causal attention of each row of q over its request's cached keys (max(0, p-window+1)..p).
 
     q is a 2-D view [rows, n_heads*head_size] (rows may be strided); token_request[row] is the
@@ -391,7 +412,9 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
     both kinds then runs as two launches, each kind in its own kernel (a single decoded token with
     a long context would otherwise walk all its keys in one wave of the kernel for portions).
     ``packed_out``: where the kernel for decoding and short portions runs, the rows come as
-    PackedRows (for the output product of few rows that reads them next); elsewhere as ever."""
+    PackedRows (for the output product of few rows that reads them next); elsewhere as ever.
+    ``first_row``: where the rows are a part of a step's batch whose other parts may run at the same time on other
+    streams, the place of the first of them in the whole batch (kernels that keep counters per row keep them apart by it)."""
     _check_pages(k_pages, v_pages, n_kv_heads, head_size)
     page_size = k_pages.shape[2]
     width = n_heads * head_size
@@ -416,7 +439,7 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
             and lib.mllm_attention_decode_supported(head_size, page_size, _code(q.dtype))
             and lib.mllm_attention_prefill_supported(head_size, page_size)):
         _require(0 < short_requests < context_lens.shape[0], "short_requests does not cut the batch in two")
-        common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len)
+        common = dict(n_heads=n_heads, n_kv_heads=n_kv_heads, head_size=head_size, scale=scale, window=window, max_len=max_len, first_row=first_row)
         paged_attention(q[:short_rows], k_pages, v_pages, token_request, positions, block_tables, max_q_len=DECODE_MAX_Q_LEN,
                         q_starts=q_starts[: short_requests + 1], context_lens=context_lens[:short_requests],
                         out=out[:short_rows], **common)
@@ -446,11 +469,14 @@ def paged_attention(q, k_pages, v_pages, token_request, positions, block_tables,
         if packed_out:
             result = empty_packed_rows(n, width, q.dtype, q.device)
             out = result.data
-        parts = torch.empty((n, n_heads, n_parts, head_size + 2), dtype=torch.float32, device=q.device) if n_parts > 1 else None
+        parts = arrivals = None
+        if n_parts > 1:
+            parts = torch.empty((n, n_heads, n_parts, head_size + 2), dtype=torch.float32, device=q.device)
+            arrivals = _arrivals(k_pages, int(first_row) + n, n_heads)[int(first_row) * n_heads :]
         check(lib.mllm_attention_decode(_ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), width if packed_out else out.stride(0),
                                         _ptr(token_request), _ptr(positions), _ptr(block_tables), block_tables.shape[1], n, n_heads, n_kv_heads,
                                         head_size, page_size, int(window), float(scale), n_splits, _code(q.dtype), int(packed_out),
-                                        n_parts, _ptr(parts), _stream()))
+                                        n_parts, _ptr(parts), _ptr(arrivals), _stream()))
         return result
     if (max_q_len is not None and max_q_len > DECODE_MAX_Q_LEN and q_starts is not None and context_lens is not None
             and rows_aligned and lib.mllm_attention_prefill_supported(head_size, page_size)):

@@ -30,7 +30,7 @@ _SIGNATURES = {
     "mllm_probe_mfma": [P, c_int, c_int, c_int, P],
     "mllm_cache_write": [P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P],
     "mllm_attention": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
-    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P],
+    "mllm_attention_decode": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, P, P, P],
     "mllm_attention_decode_supported": [c_int, c_int, c_int],
     "mllm_attention_prefill": [P, c_int, P, P, P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, P],
     "mllm_attention_prefill_supported": [c_int, c_int],

@@ -74,7 +74,7 @@ class CausalSelfAttention(Mixer):
             q, ctx.k_pages, ctx.v_pages, ctx.batch.token_request, ctx.batch.positions, ctx.group.block_tables,
             self.n_heads, self.n_kv_heads, self.head_size, self.scale, window=self.window or 0,
             max_q_len=ctx.batch.max_q_len, max_len=ctx.batch.max_total_len,
-            q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens,
+            q_starts=ctx.batch.q_starts, context_lens=ctx.batch.context_lens, first_row=getattr(ctx.batch, "first_row", 0),
             # few rows: the output product reads them faster in the packed layout
             packed_out=kernels.PACKED_ROWS_FROM <= rows <= 64 and self.out.accepts_packed_rows(rows, q.dtype, pending=True),
             **({"short_rows": ctx.batch.short_rows, "short_requests": ctx.batch.short_requests}

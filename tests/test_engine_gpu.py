@@ -471,6 +471,9 @@ def test_decoding_changes_kernels_where_the_sequences_grow_long(model_dirs, monk
     from mini_llm_amd.parts.attention import CausalSelfAttention
 
     monkeypatch.setattr(kernels, "DECODE_LAYER_REACHES", (48, 48))
+    # and the separate attention kernel cuts each row's keys into runs of 16, a block each, as it does for thousands of
+    # keys: the counters the blocks go by serve launch after launch, replayed from a graph or not
+    monkeypatch.setattr(kernels, "DECODE_MIN_PART_FEW", 16)
     monkeypatch.setattr(CausalSelfAttention, "decode_reaches", (48,))
     folder, config, weights = model_dirs["A"]
     seqs = {"a": random_tokens(7, 70, config["vocab_size"]), "b": random_tokens(8, 62, config["vocab_size"])}
@@ -489,6 +492,7 @@ def test_decoding_changes_kernels_where_the_sequences_grow_long(model_dirs, monk
         for row, name in zip(logits, seqs):
             np.testing.assert_allclose(row, ref[name][fed[name]], err_msg=f"{name} {fed[name]}", **tol)
             fed[name] += 1
+    assert kernels._arrival_counters and all((counters == 0).all() for counters in kernels._arrival_counters.values())
     if use_graphs:
         assert sorted(key[2] for key in engine.runner._graphs) == [48, config["n_positions"]]
     else:  # a's newest token is the 41st..70th: the first eight steps stay within 48

@@ -410,8 +410,9 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
      (5, 5, 256, 64, 0, (520,), 64)],
 )
 def test_decode_attention_with_the_keys_in_runs(K, monkeypatch, dtype, n_heads, n_kv_heads, head_size, page_size, window, lengths, min_part):
-    # Few tokens with many keys: each token's keys are cut into runs, a block each, and a second kernel puts the runs
-    # together. One far key stands out in each sequence, in a run other than the last where there are several.
+    # Few tokens with many keys: each token's keys are cut into runs, a block each, and the block of a (token, head) that
+    # is through last puts the runs together (twice over: the counters it goes by must be zero again behind a launch).
+    # One far key stands out in each sequence, in a run other than the last where there are several.
     if min_part is not None:
         monkeypatch.setattr(K, "DECODE_MIN_PART_FEW", min_part)
         monkeypatch.setattr(K, "DECODE_MIN_PART_BYTES", min_part * (2 if dtype == torch.bfloat16 else 4))
@@ -446,8 +447,10 @@ def test_decode_attention_with_the_keys_in_runs(K, monkeypatch, dtype, n_heads, 
         out = K.paged_attention(
             dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
             n_heads, n_kv_heads, head_size, 1.0 / math.sqrt(head_size), window=window, max_q_len=1, max_len=max(lengths), packed_out=packed_out)
-        assert K.launches_since(before) == {"attention_decode": 1, "attention_decode_merge": 1}
+        assert K.launches_since(before) == {"attention_decode": 1}
         np.testing.assert_allclose(unpacked(out) if packed_out else host(out), np.concatenate(refs), rtol=tol, atol=tol)
+    assert (kp.device.index, kp.data_ptr()) in K._arrival_counters   # runs there were
+    assert all((counters == 0).all() for counters in K._arrival_counters.values())
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
