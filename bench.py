@@ -505,6 +505,7 @@ def main() -> int:
     parser.add_argument("--no-check", action="store_true", help="skip the comparison of decoding with a whole-prompt step before timing")
     parser.add_argument("--no-points", action="store_true", help="skip the batch 1 / batch 64 points, the prefill, the kernels and the other precision")
     parser.add_argument("--one-dtype", action="store_true", help="skip the figures in the other precision")
+    parser.add_argument("--no-kernels", action="store_true", help="with --prefill-only: without the times of the step's kernels (for profiling: those take thousands of launches of their own)")
     parser.add_argument("--prefill-only", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its record")
     parser.add_argument("--serving", action="store_true", help="continuous batching of 64 requests on the GPT-2 medium shape through the scheduler")
     parser.add_argument("--temperature", type=float, default=0.0, help="sampling temperature of --serving (0: greedy)")
@@ -557,7 +558,10 @@ def main() -> int:
     engine = make_engine(args.dtype)
     checked = None if args.no_check else check_before_timing(engine, host_weights())
     if args.prefill_only:
-        emit({"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype, "kernels": measure_kernels(engine, decode=False)}, args.json)
+        record = {"prefill": measure_prefill(engine, runs=max(args.steps, 1)), "dtype": args.dtype}
+        if not args.no_kernels:
+            record["kernels"] = measure_kernels(engine, decode=False)
+        emit(record, args.json)
         return 0
     seconds, step_bytes = DecodeBench(engine, args.batch, args.prompt_len).run(args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3

@@ -561,6 +561,21 @@ template <typename T>
 int tiled_k_blocks(int M, int N, int K) {
     int tiles = ceil_div(M, 128) * ceil_div(N, 64);
     int k_blocks = 1;
+    if (sizeof(T) == 4 && tiles > 128) {
+        // In 32-bit the matrix cores set the pace, and a block has two waves on each of them: what counts is that every
+        // compute unit gets the same number of blocks. 192 tiles (2,048 x 768) whole keep 192 units busy for a block's
+        // time; cut in four along K they are 768 blocks, three to a unit, each a quarter as long: 128.7 -> 98.2 us at
+        // K = 3,072, 35.8 -> 32.0 at K = 768; 400 tiles (2,048 x 1,600 x 6,400) in three 441 -> 379 us. The cost of a cut:
+        // rounds of 256 blocks over the cuts, and 3 % for each further partial product that is written and read.
+        int best = 1;
+        float best_cost = 0.0f;
+        for (int cuts = 1; cuts <= 8; cuts++) {
+            if (cuts > 1 && K < 6 * Tile<T>::BK * cuts) break;   // three turns of the loop at least
+            const float cost = (float)ceil_div(tiles * cuts, 256) / cuts * (1.0f + 0.03f * (cuts - 1));
+            if (cuts == 1 || cost < best_cost) best = cuts, best_cost = cost;
+        }
+        return best;
+    }
     if (tiles > 128) return 1;
     const int least_tiles = M <= 256 ? 4 : 8;
     while (k_blocks < 8 && tiles * k_blocks * 2 <= 384 && K >= least_tiles * Tile<T>::BK * k_blocks * 2) k_blocks *= 2;
