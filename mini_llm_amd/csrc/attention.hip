@@ -490,6 +490,7 @@ __global__ __launch_bounds__(64 * QG * KS) void attention_prefill_kernel(
     const int tile_q0 = (gridDim.x - 1 - blockIdx.x) * (32 * QG);  // long tiles first
     if (tile_q0 >= q_len) return;
     const int context = context_lens[request];
+    if (context < 0) return;  // a padding request of a padded batch: its rows (if it has any) are nobody's, and it has no pages
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
     const int page_mask = (1 << page_shift) - 1;

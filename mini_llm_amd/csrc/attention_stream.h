@@ -185,6 +185,7 @@ __global__ __launch_bounds__(64 * SPLITS, (HD * sizeof(T) <= 128 && SPLITS == 4)
     const int tile_q0 = (gridDim.y - 1 - blockIdx.y) * QUERIES;  // the blocks with the most keys start first
     if (tile_q0 >= q_len) return;
     const int context = context_lens[request];
+    if (context < 0) return;  // a padding request of a padded batch: its rows (if it has any) are nobody's, and it has no pages
     const int kv_head = head / (n_heads / n_kv_heads);
     const int* table = block_tables + (size_t)request * max_blocks;
     const int page_mask = (1 << page_shift) - 1;

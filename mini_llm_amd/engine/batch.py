@@ -164,7 +164,7 @@ def _aligned(n: int) -> int:
 
 
 def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size: int, capacity: int | None = None,
-                     device_buffer=None, short_portion: int = SHORT_PORTION, fixed_reach: bool = False) -> StepBatch:
+                     device_buffer=None, short_portion: int = SHORT_PORTION, fixed_reach: bool = False, pad=None) -> StepBatch:
     """Lays out the batch on the host and uploads it in one copy. The entries have been checked
     and their pages reserved. With ``staging`` None the arrays stay numpy (host-only tests).
 
@@ -174,6 +174,14 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     ``FixedBuffer`` is made to the batch's length at its first use. ``fixed_reach`` names the longest
     sequence the cache can hold as the longest of this batch, as a padded batch does, so that nothing
     a kernel launch is sized by depends on how far the requests have come.
+
+    ``pad`` = (short rows, long rows, long requests) lays a batch of portions out in a padded shape, so that batches
+    of many shapes share one layout (and one captured graph): the short portions' rows padded to so many rows (and as
+    many requests), behind them the long portions' rows and requests padded likewise, and as many logit rows as there
+    are short rows and long requests. Padding rows belong to no request (token -1, request -1, slot -1); padding
+    requests have a stored length of -1 and no pages, and no rows among the long ones (among the short ones the last of
+    them spans the padding rows, none of which names it: a kernel that goes request by request passes a request with
+    a negative length by); padding logit rows name row 0 and no slot.
 
     The requests are laid out short portions first (up to ``short_portion`` tokens); the logit rows
     keep the order of the entries as given."""
@@ -194,10 +202,23 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     table_width = cache.max_blocks() or max(1, -(-max_total // page_size))
     cap_tokens = n_tokens if capacity is None else capacity
     cap_requests = n_requests if capacity is None else capacity
-    if n_tokens > cap_tokens or n_requests > cap_requests:
-        raise ValueError("the batch exceeds the capacity it is laid out for")
     n_logit_rows = sum(len(e.want) for e in entries)
     logit_length = n_logit_rows if capacity is None else max(n_logit_rows, cap_tokens)
+    request_at = list(range(n_requests))       # where each request of the layout lies among the (padded) requests
+    first_long_row = short_rows                # and where the long portions' rows begin
+    if pad is not None:
+        if capacity is not None:
+            raise ValueError("a batch is padded to a capacity or to a shape of portions, not both")
+        pad_short_rows, pad_long_rows, pad_long_requests = (int(n) for n in pad)
+        if (short_rows > pad_short_rows or n_tokens - short_rows > pad_long_rows or n_requests - short_requests > pad_long_requests
+                or n_logit_rows > pad_short_rows + pad_long_requests or (pad_short_rows > short_rows and pad_short_rows <= short_requests)):
+            raise ValueError("the batch exceeds the shape it is laid out for")
+        cap_tokens, cap_requests = pad_short_rows + pad_long_rows, pad_short_rows + pad_long_requests
+        logit_length = pad_short_rows + pad_long_requests
+        request_at = [i if i < short_requests else pad_short_rows + (i - short_requests) for i in range(n_requests)]
+        first_long_row = pad_short_rows
+    if n_tokens > cap_tokens or n_requests > cap_requests:
+        raise ValueError("the batch exceeds the capacity it is laid out for")
 
     # One flat array, its sections starting on 16-byte boundaries, filled in place (no section is built apart and copied):
     # tokens, positions, token_request, q_starts, context_lens, state_slots, logit_rows, token_sources,
@@ -214,22 +235,33 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
     sections = [flat[o : o + n] for o, n in zip(offsets, lengths)]
     tokens, positions, token_request, q_starts, context_lens, state_slots, logit_rows, token_sources = sections[:8]
 
-    starts = [0]
-    for q in q_lens:
-        starts.append(starts[-1] + q)
-    tokens[n_tokens:] = -1
-    token_request[n_tokens:] = -1
+    starts, ends, at_row = [], [], 0
+    for i, q in enumerate(q_lens):
+        if i == short_requests:
+            at_row = first_long_row
+        starts.append(at_row)
+        at_row += q
+        ends.append(at_row)
+    tokens[:] = -1
+    token_request[:] = -1
     token_sources[:] = -1
-    q_starts[: n_requests + 1] = starts
-    q_starts[n_requests + 1 :] = n_tokens
-    context_lens[:n_requests] = contexts
-    state_slots[:n_requests] = [r.state_slot for r in records]
-    state_slots[n_requests:] = -1    # padding: no request, no slot
+    # a request's rows are q_starts[r] .. q_starts[r + 1]: a padding request begins where the request before it ends
+    q_starts[:] = n_tokens if pad is None else (ends[-1] if n_requests > short_requests else first_long_row)
+    if pad is not None:
+        q_starts[short_requests : pad[0]] = short_rows
+        context_lens[:] = -1   # a padding request: kernels that go request by request pass it by
+    for i in range(n_requests):
+        q_starts[request_at[i]] = starts[i]
+        context_lens[request_at[i]] = contexts[i]
+    if pad is None:
+        q_starts[n_requests] = n_tokens
+    state_slots[:] = -1    # padding: no request, no slot
     for i, e in enumerate(entries):
-        lo, hi = starts[i], starts[i + 1]
+        lo, hi = starts[i], ends[i]
         tokens[lo:hi] = e.token_array()
         positions[lo:hi] = np.arange(contexts[i], contexts[i] + q_lens[i], dtype=np.int32)
-        token_request[lo:hi] = i
+        token_request[lo:hi] = request_at[i]
+        state_slots[request_at[i]] = records[i].state_slot
         if e.from_slot:
             token_sources[lo] = records[i].state_slot
     tables, slots = [], []
@@ -237,11 +269,11 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         table = sections[8 + 2 * gi].reshape(cap_requests, table_width)
         slot = sections[9 + 2 * gi]
         table[:] = -1
-        slot[n_tokens:] = -1
+        slot[:] = -1
         for i, e in enumerate(entries):
-            lo, hi = starts[i], starts[i + 1]
+            lo, hi = starts[i], ends[i]
             pages = np.asarray(cache.block_table(e.request_id, gi), dtype=np.int32)
-            table[i, : len(pages)] = pages
+            table[request_at[i], : len(pages)] = pages
             pos = positions[lo:hi]
             slot[lo:hi] = pages[pos // page_size] * page_size + pos % page_size
         tables.append(table)
@@ -270,10 +302,14 @@ def build_step_batch(entries, cache, staging: BatchStaging | None, *, vocab_size
         GroupStepData(block_tables=views[8 + 2 * gi].reshape(cap_requests, table_width), slots=views[9 + 2 * gi])
         for gi in range(n_groups)
     ]
+    longest = max(q_lens)
+    if pad is not None:   # what a launch is sized by depends on the shape alone
+        short_requests = short_rows = pad[0]
+        longest = pad[1] if pad[1] > 0 else short_portion
     return StepBatch(
-        n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=logit_length, max_q_len=max(q_lens),
+        n_tokens=cap_tokens, n_requests=cap_requests, n_logit_rows=logit_length, max_q_len=longest,
         short_requests=short_requests, short_rows=short_rows,
-        max_total_len=max_total if capacity is None and not fixed_reach else (cache.max_length or table_width * page_size),
+        max_total_len=max_total if capacity is None and pad is None and not fixed_reach else (cache.max_length or table_width * page_size),
         tokens=views[0], positions=views[1], token_request=views[2], q_starts=views[3], context_lens=views[4],
         state_slots=views[5], logit_rows=views[6], token_sources=views[7], logit_slots=views[-1], groups=groups,
         request_ids=[e.request_id for e in entries], host=host, short_portion=short_portion,

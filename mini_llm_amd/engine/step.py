@@ -28,16 +28,19 @@ from .batch import BatchStaging, DecodeBatchBuilder, FixedBuffer, StepBatch, Ste
 
 GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 # Steps with portions of prompts: a step of a few thousand tokens of a small model is over on the GPU before the host has
-# launched its kernels one by one, so a shape of batch that keeps coming is captured too. A capture costs about 45 ms
-# (measured; most of it making the graph ready to launch) and a replay saves some tenths of a millisecond, so a shape has to
-# come PORTION_GRAPH_AFTER times before it is captured: the shapes of a serving run with a mixed load change from step to
-# step and would each be captured for nothing (measured with a capture at the second time: 7.5k generated tokens a second
-# against 28.6k without). Larger steps are bound by the GPU and would only hold their activations' memory; so many shapes
-# are kept, the least recently used one going first.
-PORTION_GRAPH_AFTER = 32
+# launched its kernels one by one (a mixed step of 512 tokens through the 24 layers of the medium shape: 3.1 ms of
+# launching for 1.1 ms of work), so a shape of batch that keeps coming is captured too. The shapes of a serving run with a
+# mixed load change from step to step (captured as they are, each at its second coming, they were captured for nothing:
+# 7.5k generated tokens a second against 28.6k without), so a batch is laid out in a padded shape (build_step_batch's
+# ``pad``): the short portions' rows in steps of 16, the long portions' rows in steps of 64 and their requests in powers
+# of two. A serving run then sees a dozen shapes, not hundreds. A capture costs about 45 ms (most of it making the graph
+# ready to launch), so a shape is captured at its PORTION_GRAPH_AFTER-th coming. Larger steps are bound by the GPU and would
+# only hold their activations' memory; so many shapes are kept, the least recently used one going first.
+PORTION_GRAPH_AFTER = 3
 PORTION_GRAPH_MAX_TOKENS = 8192
-PORTION_GRAPHS_KEPT = 8
+PORTION_GRAPHS_KEPT = 16
 PORTION_SHAPES_COUNTED = 4096
+PORTION_SHORT_ROWS, PORTION_LONG_ROWS = 16, 64   # the rows of short and of long portions are padded to multiples of these
 
 
 class StepError(ValueError):
@@ -251,12 +254,12 @@ def _capture(runner, batch, choice=None, lanes=None):
 
 
 class _PortionGraph:
-    """One captured step for batches of one shape: so many tokens, requests and wanted places, the same longest portion and
-    the same cut between short and long portions. Everything else about a batch (tokens, positions, pages, which rows are
-    wanted) lies in the device buffer that the kernels read, and is overwritten before each replay."""
+    """One captured step for batches of one padded shape (so many rows of short portions, rows of long portions and long
+    requests: build_step_batch's ``pad``). Everything else about a batch (tokens, positions, pages, which rows are real
+    and which are wanted) lies in the device buffer that the kernels read, and is overwritten before each replay."""
 
-    def __init__(self, runner: "ModelRunner"):
-        self.runner = runner
+    def __init__(self, runner: "ModelRunner", pad):
+        self.runner, self.pad = runner, pad
         self.buffer = FixedBuffer(runner.device)
         self.graph = None
         self.logits = None
@@ -265,7 +268,7 @@ class _PortionGraph:
     def run(self, entries):
         runner = self.runner
         batch = build_step_batch(entries, runner.cache, runner.staging, vocab_size=runner.model.vocab_size, device_buffer=self.buffer,
-                                 short_portion=runner.model.short_portion(), fixed_reach=True)
+                                 short_portion=runner.model.short_portion(), fixed_reach=True, pad=self.pad)
         if self.graph is None:
             self.graph, self.logits = _capture(runner, batch)
             self.batch = batch
@@ -277,7 +280,8 @@ class _PortionGraph:
             if not same:
                 raise RuntimeError("a captured step was asked to run a batch of another shape")
         self.graph.replay()
-        return batch, self.logits
+        wanted = sum(len(e.want) for e in entries)
+        return batch, self.logits[:wanted] if wanted else None   # (the shape's further logit rows are padding)
 
 
 class ModelRunner:
@@ -406,8 +410,14 @@ class ModelRunner:
         n_tokens = sum(lengths)
         if n_tokens > PORTION_GRAPH_MAX_TOKENS:
             return None
-        shape = (n_tokens, len(entries), sum(len(e.want) for e in entries), max(lengths),
-                 sum(1 for n in lengths if n <= short), sum(n for n in lengths if n <= short))
+        # the padded shape the batch falls in: rows of short portions, rows of long portions, long requests
+        short_rows, long_rows = sum(n for n in lengths if n <= short), sum(n for n in lengths if n > short)
+        long_requests = sum(1 for n in lengths if n > short)
+        round_up = lambda n, step: -(-n // step) * step
+        shape = (round_up(short_rows, PORTION_SHORT_ROWS), round_up(long_rows, PORTION_LONG_ROWS),
+                 1 << (long_requests - 1).bit_length() if long_requests else 0)
+        if sum(len(e.want) for e in entries) > shape[0] + shape[2]:
+            return None   # more wanted places than the shape has logit rows (a trace that wants every place): run as it is
         graph = self._portion_graphs.get(shape)
         if graph is not None:
             self._portion_graphs.move_to_end(shape)
@@ -423,7 +433,7 @@ class ModelRunner:
             evicted, _ = self._portion_graphs.popitem(last=False)
             self._shapes_seen[evicted] = 0
             self.portion_graphs_dropped += 1
-        graph = self._portion_graphs[shape] = _PortionGraph(self)
+        graph = self._portion_graphs[shape] = _PortionGraph(self, shape)
         self.portion_graphs_made += 1
         return graph
 

@@ -343,7 +343,8 @@ def test_graph_replays_match_eager_steps(model_dirs, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
-    # steps with portions of prompts whose shape of batch keeps coming (so many tokens, requests and wanted places) are
+    # steps with portions of prompts whose padded shape of batch keeps coming (the rows of short portions in steps of 16, of
+    # long portions in steps of 64, long requests in powers of two) are
     # captured (here at the second time, by option) and replayed from then on: here the same shapes come with other requests, at other
     # depths of the cache and with other places wanted, with decode replays, eager steps of other shapes and
     # synchronisations between them; every step is checked against the plain implementation, with and without graphs
@@ -405,9 +406,9 @@ def test_captured_portion_steps_match_eager_steps(model_dirs, dtype):
             handles[name] = engine.try_take_cache()
             fed[name] = 0
         run([("b", 131, [130]), ("c", 1, [0]), ("a", 2, [0])])    # Z again: captured here, the long portion from an empty cache
-        run([("a", 43, [42]), ("c", 5, [])])                      # depths 45 (a), 11 (c)
+        run([("a", 43, [42]), ("c", 5, [])])                      # depths 45 (a), 11 (c); 43 + 5 tokens fall in X's padded shape: replayed
         run([("a", 131, [7]), ("b", 1, [0]), ("c", 2, [1])])      # Z replayed: the long portion starts at 45, inside a page and a tile
-        assert engine.runner.portion_graph_steps == (9 if use_graphs else 0)
+        assert engine.runner.portion_graph_steps == (10 if use_graphs else 0)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -401,6 +401,52 @@ def test_paged_attention(K, path, dtype, n_heads, n_kv_heads, head_size, page_si
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_heads,head_size,page_size", [(3, 64, 64), (5, 48, 16), (2, 128, 32)])
+def test_prompt_attention_passes_padding_requests_by(K, dtype, n_heads, head_size, page_size):
+    # A batch laid out in a padded shape has requests that are nobody: a stored length of -1, a block table of -1, and
+    # (one of them) rows that no request owns. The kernels that go request by request pass them by.
+    rng = np.random.default_rng(head_size)
+    rnd = lambda *s: bf16_round(rng.standard_normal(s)) if dtype == torch.bfloat16 else rng.standard_normal(s).astype(np.float32).astype(np.float64)
+    shapes = [(40, 70), None, (0, 33), None]          # (stored, new) of the real requests; None: padding
+    padding_rows = 6                                   # rows that the first padding request spans
+    num_pages = 16
+    kp = torch.full((num_pages, n_heads, page_size, head_size), float("nan"), device=DEV).to(dtype)
+    vp = torch.full_like(kp, float("nan"))
+    max_blocks = 8
+    tables = np.full((len(shapes), max_blocks), -1, dtype=np.int32)
+    order = rng.permutation(num_pages).tolist()
+    q_rows, refs, starts, contexts, real_rows, at = [], [], [0], [], [], 0
+    for r, shape in enumerate(shapes):
+        if shape is None:
+            rows = padding_rows if r == 1 else 0
+            q_rows.append(np.zeros((rows, n_heads * head_size)))
+            contexts.append(-1)
+        else:
+            ctx, new = shape
+            total = ctx + new
+            k_all, v_all, q = rnd(total, n_heads * head_size), rnd(total, n_heads * head_size), rnd(new, n_heads * head_size)
+            pages = [order.pop() for _ in range((total + page_size - 1) // page_size)]
+            tables[r, : len(pages)] = pages
+            slots = np.array([pages[p // page_size] * page_size + p % page_size for p in range(total)], dtype=np.int32)
+            K.cache_write(dev(k_all, dtype), dev(v_all, dtype), kp, vp, dev(slots, torch.int32), n_heads, head_size)
+            q_rows.append(q)
+            refs.append(plain_paged_attention(q, k_all, v_all, n_heads, n_heads, None))
+            contexts.append(ctx)
+            rows = new
+            real_rows += list(range(at, at + rows))
+        at += rows
+        starts.append(at)
+    treq = np.concatenate([np.full(len(q), r if shapes[r] is not None else -1) for r, q in enumerate(q_rows)])
+    tpos = np.concatenate([np.arange(len(q)) + max(contexts[r], 0) for r, q in enumerate(q_rows)])
+    out = K.paged_attention(
+        dev(np.concatenate(q_rows), dtype), kp, vp, dev(treq, torch.int32), dev(tpos, torch.int32), dev(tables, torch.int32),
+        n_heads, n_heads, head_size, 1.0 / math.sqrt(head_size), max_q_len=70, max_len=128,
+        q_starts=dev(starts, torch.int32), context_lens=dev(contexts, torch.int32))
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(host(out)[real_rows], np.concatenate(refs), rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize(
     "n_heads,n_kv_heads,head_size,page_size,window,lengths,min_part",
     [(12, 12, 64, 64, 0, (1500,), None),                 # one token, 1,500 keys: two runs by the kernel's own rule
