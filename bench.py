@@ -430,7 +430,7 @@ def measure_serving(dtype: str, temperature: float, step_ahead: bool = True):
         torch.cuda.synchronize()
         return time.perf_counter() - begin
 
-    for _ in range(3):   # warm-up: the decode steps are captured in the first run, the padded shapes of the mixed steps at their third coming
+    for _ in range(4):   # warm-up: the decode steps are captured in the first run, the padded shapes of the mixed steps at their fourth coming
         run_once()
     for i in range(len(counts)):
         counts[i] = 0

@@ -34,11 +34,13 @@ GRAPH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 # 7.5k generated tokens a second against 28.6k without), so a batch is laid out in a padded shape (build_step_batch's
 # ``pad``): the short portions' rows in steps of 16, the long portions' rows in steps of 64 and their requests in powers
 # of two. A serving run then sees a dozen shapes, not hundreds. A capture costs about 45 ms (most of it making the graph
-# ready to launch), so a shape is captured at its PORTION_GRAPH_AFTER-th coming. Larger steps are bound by the GPU and would
-# only hold their activations' memory; so many shapes are kept, the least recently used one going first.
-PORTION_GRAPH_AFTER = 3
+# ready to launch) and a replay saves a millisecond, so a capture pays after some fifty replays: a shape is captured at its
+# PORTION_GRAPH_AFTER-th coming (a shape that has come so often will come again), and enough shapes are kept that a steady
+# load does not push its own shapes out (the least recently used one goes first, and counts anew). Larger steps are bound
+# by the GPU and would only hold their activations' memory.
+PORTION_GRAPH_AFTER = 4
 PORTION_GRAPH_MAX_TOKENS = 8192
-PORTION_GRAPHS_KEPT = 16
+PORTION_GRAPHS_KEPT = 32
 PORTION_SHAPES_COUNTED = 4096
 PORTION_SHORT_ROWS, PORTION_LONG_ROWS = 16, 64   # the rows of short and of long portions are padded to multiples of these
 
