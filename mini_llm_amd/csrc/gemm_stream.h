@@ -264,7 +264,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * WAVES_K) void gemm_stream_
         };
         // The loads of tile u + STAGES go into the stage of tile u, between the barrier in tile u (which every wave passes
         // with its reads of tile u done) and the barrier in tile u + 1: KS steps, each with its share.
-        auto share = [](int e) { return (e * LPW + KS - 1) / KS; };  // loads share(e) .. share(e + 1) go with step e after the barrier
+        // loads share(e) .. share(e + 1) go with step e after the barrier; with two stages all of them at once, behind the
+        // barrier that frees their stage: they have one tile's time to land, and none of it to spare
+        auto share = [](int e) { return STAGES == 2 ? (e >= 1 ? LPW : 0) : (e * LPW + KS - 1) / KS; };
         auto stage_of = [](int tile) { return (tile % STAGES) * STAGE_BYTES; };
 
         // before the loop: what the turns before the first would have asked for
@@ -504,6 +506,22 @@ void dispatch(const bf16_t* a, const bf16_t* w, const float* bias, const float* 
         const long blocks = (long)ceil_div(M, choices[c].bm) * ceil_div(N, choices[c].bn) * k_blocks;
         const float cost = (float)((blocks + 255) / 256) * choices[c].tile_us;
         if (c == 0 || cost < best_cost) best = c, best_cost = cost;  // (equal costs: the wider tile, which reads less)
+    }
+    // 256 x 256 (four waves of 128 x 128; the LDS holds two stages of it) brings a compute unit 40k outputs a microsecond
+    // and tile of K where the others bring 30k, but only in full rounds of at least 150 blocks: from 2,048 x 6,400 on.
+    // Measured against the choice among the others (whose costs above are those of smaller products: at these sizes
+    // they take 1.45 times as long), on one machine in one run: 2,048 x 6,400 x 1,600 52 against 59 us (as a layer's up
+    // product with its GELU 52.5 against 56.2), 8,192 x 4,096 x 1,024 74 against 85, 8,192 x 6,400 x 1,600 186 against 194;
+    // but 2,048 x 4,096 x 1,024 (128 blocks) 30.7 against 23.2. (Machines of this kind differ by a tenth between them:
+    // another one took 45.2 and 52.4 us for the first of these.)
+    // (Only with bfloat16 out, which is what the products of that size write: with 32-bit out and a residual asked for
+    // before the loop, a lane's 256 sums and 256 residual values do not fit its registers.)
+    if constexpr (sizeof(OutT) == 2) {
+        const long large = (long)ceil_div(M, 256) * ceil_div(N, 256), rounds = (large + 255) / 256;
+        if (k_blocks == 1 && large >= 150 && large * 10 >= rounds * 256 * 7 && (float)rounds * 1.6f < best_cost * 1.45f) {
+            MLLM_STREAM(256, 256, 2, 2, 1, 2);
+            return;
+        }
     }
     if (best == 0) MLLM_STREAM(128, 192, 2, 2, 1, 3);
     else if (best == 1) MLLM_STREAM(256, 128, 4, 2, 1, 3);

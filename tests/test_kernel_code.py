@@ -24,7 +24,7 @@ def test_no_scalar_load_inside_the_loop_of_the_streaming_product(tmp_path):
                    check=True, capture_output=True, timeout=600)
     text = listing.read_text()
     kernels = re.split(r"\n(?=_ZN6stream18gemm_stream_kernel[^\n]*:\s)", text)[1:]
-    assert len(kernels) >= 10  # five tiles, two output types
+    assert len(kernels) >= 11  # five tiles, two output types, and the 256 x 256 tile with bfloat16 out
     for kernel in kernels:
         name = kernel.split(":", 1)[0]
         body = kernel.split(".Lfunc_end", 1)[0].split("\n")
@@ -40,4 +40,12 @@ def test_no_scalar_load_inside_the_loop_of_the_streaming_product(tmp_path):
         for loop in loops:
             scalar_loads = [instruction.strip() for instruction in loop if re.search(r"\ts_(buffer_)?load", instruction)]
             assert not scalar_loads, (name, scalar_loads)
-        assert re.search(r"; ScratchSize: 0\b", kernel), name  # and no register of the loop lives in memory
+            # and no register of the loop lives in memory
+            assert not [instruction for instruction in loop if re.search(r"\tscratch_(load|store)", instruction)], name
+        if "Li256ELi256E" in name:
+            # the largest tile: 256 sums a lane fill the accumulation registers, and a few values of the prologue (the
+            # bias asked for early) wait in memory until the epilogue, outside the loop
+            scratch = int(re.search(r"; ScratchSize: (\d+)", kernel).group(1))
+            assert scratch <= 64, (name, scratch)
+        else:
+            assert re.search(r"; ScratchSize: 0\b", kernel), name

@@ -188,9 +188,10 @@ GEMM_SHAPES = [(1, 64, 64), (3, 100, 96), (17, 288, 320), (33, 1000, 96), (64, 1
                (2100, 2010, 104), (4100, 2010, 40),  # many rows and columns: the large tile (256 x 128; in 32-bit from 256 tiles on), ragged edges
                # K in whole tiles of 64, columns in whole pieces, 65 rows or more: in bfloat16 with a packed matrix the kernel that
                # streams its operands into LDS: tiles of 128 x 64 (with two waves sharing each 64 x 64 along K from a K of 1,536 on:
-               # here with an odd count of tiles), 128 x 192, 128 x 128 and 256 x 128, chosen by the rounds of blocks they need
+               # here with an odd count of tiles), 128 x 192, 128 x 128, 256 x 128 and 256 x 256 (the last shape: 200 tiles in one
+               # round of blocks, ragged on both sides), chosen by the rounds of blocks they need
                (300, 136, 192), (193, 2008, 128), (2100, 264, 64), (700, 776, 320), (300, 72, 1600), (2100, 2008, 128), (192, 8, 64),
-               (1000, 2312, 128), (2040, 4088, 64), (70, 136, 128), (130, 264, 64)]
+               (1000, 2312, 128), (2040, 4088, 64), (70, 136, 128), (130, 264, 64), (2000, 6392, 192)]
 
 
 @pytest.mark.parametrize("packed", [False, True])
