@@ -776,12 +776,12 @@ def test_the_callers_longest_sequence_narrows_the_models_own(model_dirs):
     engine.close()
 
 
-@pytest.mark.parametrize("seed", [0, 1])
+@pytest.mark.parametrize("seed", [0, 1, 2])
 def test_random_workloads_through_the_scheduler_match_plain_greedy(model_dirs, engines, seed):
     # random prompt lengths and lengths to generate, portions under a small budget, a pool that holds
     # a few requests (so some wait and some are preempted and recomputed): whatever the scheduler
     # does, every request gets the plain implementation's greedy tokens
-    name = "AB"[seed]
+    name = "ABC"[seed]   # (C: heads of 48, whose short portions go through the kernel that walks request by request)
     _, config, weights = model_dirs[name]
     rng = np.random.default_rng(50 + seed)
     limit = config["n_positions"]
@@ -790,7 +790,7 @@ def test_random_workloads_through_the_scheduler_match_plain_greedy(model_dirs, e
         n = int(rng.integers(1, limit // 2))
         prompts.append(random_tokens(700 + 20 * seed + i, n, config["vocab_size"]))
         new.append(int(rng.integers(1, min(24, limit - n) + 1)))
-    engine = engines(name, "float32", max_sessions=5, max_tokens=2 * limit, page_size=16, max_tokens_per_step=int(rng.integers(8, 40)))
+    engine = engines(name, "float32", max_sessions=5, max_tokens=(2 if seed < 2 else 1) * limit, page_size=16, max_tokens_per_step=int(rng.integers(8, 40)))
     before = engine.stats()["preemptions"]
     outputs = [engine.generate([prompt], max_new_tokens=n)[0] for prompt, n in zip(prompts[:2], new[:2])]   # alone
     from mini_llm_amd.engine.scheduler import Request
@@ -801,7 +801,8 @@ def test_random_workloads_through_the_scheduler_match_plain_greedy(model_dirs, e
                               max_new_tokens=n))
     engine.scheduler.run_until_idle()
     assert not errors
-    assert engine.stats()["preemptions"] > before   # the pool is that small
+    if seed < 2:
+        assert engine.stats()["preemptions"] > before   # the pool is that small (the third model's requests grow too little for it)
     for i, (prompt, n) in enumerate(zip(prompts, new)):
         assert together[i] == plain_gpt2.greedy(config, weights, prompt, n), f"request {i} ({len(prompt)} prompt tokens, {n} new)"
     assert outputs == together[:2]
